@@ -1,0 +1,448 @@
+"""Pins the CPU oracle before anything is compared with it.
+
+Each oracle function is checked against (a) the literal cases the reference's own tests
+hold (tests/golden/reference_literals.json), (b) library routines it must reduce to in
+special cases (numpy / torch sort, topk, bincount, dtype casts), (c) brute force written
+from the definition with plain Python loops on tiny inputs, and (d) structural invariants
+the reference's tests assert.  A dropped term, a wrong sign, a transposed index or a wrong
+tie-break fails at least one of them.
+"""
+from __future__ import annotations
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import arrival_plane, equal_quota_routing
+from oracle import terrace_oracle as orc
+
+
+# ----------------------------------------------------------------------------- formats
+
+def test_bf16_matches_torch_cast_bitwise():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(4096, generator=g) * 10.0 ** torch.randint(-20, 20, (4096,), generator=g)
+    x = torch.cat([x, torch.tensor([0.0, -0.0, 1.0, 65504.0, 3.3895e38, float("inf"), -float("inf")])])
+    want = x.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = orc.f32_to_bf16(x.numpy())
+    assert np.array_equal(want, got)
+    back = torch.from_numpy(got.view(np.int16)).view(torch.bfloat16).float().numpy()
+    assert np.array_equal(back, orc.bf16_to_f32(got))
+
+
+def test_bf16_ties_round_to_even():
+    # 1 + 2^-8 sits exactly between two bf16 values: goes to the even one (1.0);
+    # 1 + 3*2^-8 goes up to 1 + 2^-6.
+    x = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8], dtype=np.float32)
+    assert orc.bf16_to_f32(orc.f32_to_bf16(x)).tolist() == [1.0, 1.0 + 2.0 ** -6]
+
+
+def test_e4m3_table_matches_torch_all_codes():
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    want = codes.view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.isnan(want), np.isnan(orc.E4M3))
+    ok = ~np.isnan(want)
+    assert np.array_equal(want[ok], orc.E4M3[ok])
+
+
+def test_e4m3_encode_matches_torch_cast():
+    g = torch.Generator().manual_seed(1)
+    x = torch.cat([torch.randn(20000, generator=g) * 100, torch.randn(20000, generator=g) * 0.01,
+                   torch.tensor([0.0, 448.0, -448.0, 0.0009765625, 0.0029296875, 17.0, 18.0, 19.0])])
+    x = x.clamp(-448, 448)
+    want = x.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = orc.f32_to_e4m3(x.numpy())
+    same = (want == got) | ((x.numpy() == 0) & ((want & 0x7F) == 0) & ((got & 0x7F) == 0))
+    assert same.all()
+
+
+def test_fp8_rows_roundtrip_and_layout():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((5, 256)).astype(np.float32)
+    x[3, :128] = 0.0
+    rows = orc.fp8_quantise_rows(x)
+    assert rows.shape == (5, 256 + 8) and rows.dtype == np.uint8
+    scales = rows[:, 256:].copy().view(np.float32)
+    assert scales[3, 0] == 1.0
+    assert np.allclose(scales[0, 0], np.abs(x[0, :128]).max() / 448.0)
+    deq = orc.fp8_dequantise_rows(rows, 256)
+    assert np.abs(deq - x).max() <= np.abs(x).max() * 2.0 ** -4      # 3 mantissa bits
+    assert orc.fp8_row_bytes(7168) == 7392                            # 7168 + 56*4
+
+
+# ----------------------------------------------------------------------------- routing
+
+def _route_brute(aff, bias, E, Ng, k, M):
+    """Definition, token by token, with Python sorting on (-value, index)."""
+    g, q = E // Ng, k // M
+    idx_out, grp_out, gate_out = [], [], []
+    for t in range(aff.shape[0]):
+        s = [np.float32(aff[t, e]) + np.float32(bias[e]) for e in range(E)]
+        score = []
+        for G in range(Ng):
+            vals = sorted(s[G * g:(G + 1) * g], reverse=True)
+            score.append(np.float32(np.float32(vals[0] + vals[1]) / np.float32(2)) if g > 1 else vals[0])
+        groups = sorted(range(Ng), key=lambda G: (-score[G], G))[:M]
+        row = []
+        for G in groups:
+            best = sorted(range(G * g, (G + 1) * g), key=lambda e: (-s[e], e))[:q]
+            row += best
+        den = np.float32(0)
+        for e in row:
+            den = np.float32(den + np.float32(aff[t, e]))
+        idx_out.append(row)
+        grp_out.append(groups)
+        gate_out.append([np.float32(np.float32(aff[t, e]) / den) for e in row])
+    return np.array(idx_out), np.array(gate_out, dtype=np.float32), np.array(grp_out)
+
+
+@pytest.mark.parametrize("E,Ng,k,M", [(16, 4, 4, 2), (64, 8, 8, 4), (24, 3, 6, 3), (8, 8, 2, 2), (32, 1, 4, 1)])
+def test_route_full_equals_brute_force(E, Ng, k, M):
+    rng = np.random.default_rng(E * 100 + k)
+    aff = rng.random((23, E)).astype(np.float32)
+    bias = (rng.standard_normal(E) * 0.3).astype(np.float32)
+    e, gts, grp = orc.t_route(aff, bias, E, Ng, k, M)
+    be, bg, bgrp = _route_brute(aff, bias, E, Ng, k, M)
+    assert np.array_equal(e, be) and np.array_equal(grp, bgrp)
+    assert np.array_equal(gts, bg)
+    assert e.dtype == np.int64 and grp.dtype == np.int64 and gts.dtype == np.float32
+
+
+def test_route_group_score_is_mean_of_top_two_not_max():
+    # group 0 holds the single largest value, group 1 two good ones: mean-of-top-2 picks 1.
+    aff = np.array([[0.9, 0.1, 0.0, 0.0, 0.8, 0.8, 0.0, 0.0]], dtype=np.float32)
+    _, _, grp = orc.t_route(aff, np.zeros(8, np.float32), 8, 2, 1, 1)
+    assert grp.tolist() == [[1]]
+    _, _, grp1 = orc.t_route(aff, np.zeros(8, np.float32), 8, 2, 1, 1, pool=1)
+    assert grp1.tolist() == [[0]]
+
+
+def test_route_ties_take_lowest_index_and_order_is_descending():
+    aff = np.array([[0.5, 0.5, 0.5, 0.5, 0.5, 0.5, 0.5, 0.5]], dtype=np.float32)
+    e, _, grp = orc.t_route(aff, np.zeros(8, np.float32), 8, 4, 4, 2)
+    assert grp.tolist() == [[0, 1]] and e.tolist() == [[0, 1, 2, 3]]
+    aff = np.array([[0.1, 0.9, 0.2, 0.3, 0.8, 0.7, 0.0, 0.0]], dtype=np.float32)
+    e, _, grp = orc.t_route(aff, np.zeros(8, np.float32), 8, 4, 4, 2)
+    assert grp.tolist() == [[2, 0]]                  # scores .75, .25, .5(=(.9+.1)/2 -> .5)...
+    assert e.tolist() == [[4, 5, 1, 0]]
+
+
+def test_route_selection_uses_bias_but_gates_do_not():
+    aff = np.array([[0.2, 0.1, 0.6, 0.5]], dtype=np.float32)
+    bias = np.array([1.0, 1.0, 0.0, 0.0], dtype=np.float32)
+    e, g, _ = orc.t_route(aff, bias, 4, 2, 2, 1)
+    assert e.tolist() == [[0, 1]]
+    assert np.array_equal(g, np.array([[np.float32(0.2) / (np.float32(0.2) + np.float32(0.1)),
+                                        np.float32(0.1) / (np.float32(0.2) + np.float32(0.1))]], np.float32))
+    e2, g2, _ = orc.t_route(aff, bias, 4, 2, 2, 1, gate_affinity=np.array([[3.0, 1.0, 9.0, 9.0]], np.float32))
+    assert e2.tolist() == [[0, 1]] and g2.tolist() == [[0.75, 0.25]]
+
+
+def test_route_reduces_to_library_topk_in_special_cases():
+    g = torch.Generator().manual_seed(3)
+    aff = torch.rand(257, 32, generator=g)
+    zero = np.zeros(32, np.float32)
+    # every expert its own group: the M chosen groups are the plain top-M experts
+    e, _, grp = orc.t_route(aff.numpy(), zero, 32, 32, 4, 4)
+    want = aff.topk(4, dim=-1).indices.numpy()
+    assert np.array_equal(e, want) and np.array_equal(grp, want)
+    # one group: top-k inside it is the plain top-k
+    e, _, _ = orc.t_route(aff.numpy(), zero, 32, 1, 6, 1)
+    assert np.array_equal(e, aff.topk(6, dim=-1).indices.numpy())
+    # global_topk mode is the plain top-k by definition (terrace/routing.py:72-74)
+    e, _, grp = orc.t_route(aff.numpy(), zero, 32, 4, 4, 2, mode="global_topk")
+    assert np.array_equal(e, want) and np.array_equal(grp, want // 8)
+
+
+def test_route_structural_guarantees_reference_config(literals):
+    cfg = literals["routing_structural"]["cfg"]
+    E, Ng, k, M = cfg["n_experts"], cfg["n_groups"], cfg["top_k"], cfg["top_groups"]
+    g = torch.Generator().manual_seed(0)
+    aff = torch.sigmoid(torch.randn(512, E, generator=g)).numpy()
+    e, gates, grp = orc.t_route(aff, np.zeros(E, np.float32), E, Ng, k, M)
+    gs = E // Ng
+    for t in range(512):
+        assert len(set(e[t])) == k
+        assert set(e[t] // gs) == set(grp[t]) and len(set(grp[t])) == M
+        assert (np.bincount(e[t] // gs, minlength=Ng)[grp[t]] == k // M).all()
+    assert np.allclose(gates.sum(-1), 1.0, atol=1e-5) and (gates > 0).all()
+
+
+def test_route_adversarial_affinity_concentrates_load(literals):
+    a = literals["routing_structural"]["adversarial"]
+    E, Ng = a["n_experts"], a["n_groups"]
+    g = E // Ng
+    rng = np.random.default_rng(4)
+    aff = (rng.random((a["n_tok"], E)) * 0.01).astype(np.float32)
+    aff[:, :a["favoured_groups"] * g] += 1.0
+    e, _, grp = orc.t_route(aff, np.zeros(E, np.float32), E, Ng, a["top_k"], a["top_groups"])
+    load = np.bincount((e // g).reshape(-1), minlength=Ng)
+    assert (load[a["favoured_groups"]:] == a["unfavoured_load"]).all() and (load[:a["favoured_groups"]] > 0).all()
+    assert grp.shape[1] == a["top_groups"]
+
+
+def test_route_other_modes_and_errors():
+    rng = np.random.default_rng(5)
+    aff = rng.random((64, 32)).astype(np.float32)
+    zero = np.zeros(32, np.float32)
+    e, _, grp = orc.t_route(aff, zero, 32, 4, 8, 4, mode="quota_only")
+    assert np.array_equal(grp, np.tile(np.arange(4), (64, 1)))
+    assert (np.sort(e // 8, axis=1) == np.repeat(np.arange(4), 2)[None]).all()
+    e, _, grp = orc.t_route(aff, zero, 32, 4, 4, 2, mode="group_limited")
+    for t in range(64):
+        assert set(e[t] // 8) <= set(grp[t]) and len(set(e[t])) == 4
+        cand = np.concatenate([np.arange(G * 8, G * 8 + 8) for G in grp[t]])
+        assert set(e[t]) == set(cand[np.argsort(-aff[t, cand], kind="stable")[:4]])
+    with pytest.raises(ValueError, match="unknown routing mode"):
+        orc.t_route(aff, zero, 32, 4, 4, 2, mode="Full")
+    for bad in [(30, 4, 4, 2), (32, 4, 6, 4), (32, 16, 8, 2)]:
+        with pytest.raises(ValueError):
+            orc.check_route_config(*bad)
+
+
+def test_expert_load_and_bias_update():
+    e = np.array([[0, 3], [3, 1]])
+    load = orc.expert_load(e, 5)
+    assert load.dtype == np.float32 and load.tolist() == [1, 1, 0, 2, 0]
+    b = orc.update_bias(np.zeros(5, np.float32), load, 0.5)
+    assert b.tolist() == [-0.5, -0.5, 0.5, -0.5, 0.5]                   # mean load 0.8
+
+
+# ----------------------------------------------------------------------------- plan
+
+def test_plan_literal_guard_cases(literals):
+    lit = literals["plan_quota_guard"]
+    geo = lit["geometry"]
+    for case in lit["cases"]:
+        idx = np.array([case["expert_idx_row"]] * case["repeat"], dtype=np.int64)
+        if case["raises"]:
+            with pytest.raises(ValueError, match=case["raises"]):
+                orc.plan_ta2a(idx, geo["world"], geo["n_experts"], geo["rpn"], case["groups_m"])
+        else:
+            u_src, u_node, counts, inv = orc.plan_ta2a(idx, geo["world"], geo["n_experts"], geo["rpn"],
+                                                       case["groups_m"])
+            assert u_src.size == case["n_rows"] and int(counts.sum()) == case["counts_sum"]
+
+
+def _plan_brute(e, slots, n_nodes):
+    T, k = e.shape
+    pairs = sorted({(int(e[t, j]) // slots, t) for t in range(T) for j in range(k)})
+    row = {p: i for i, p in enumerate(pairs)}
+    inv = [row[(int(e[t, j]) // slots, t)] for t in range(T) for j in range(k)]
+    counts = [sum(1 for n, _ in pairs if n == b) for b in range(n_nodes)]
+    return ([t for _, t in pairs], [n for n, _ in pairs], counts, inv)
+
+
+def test_plan_equals_sorted_pair_list(literals):
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        n_nodes, slots = world // rpn, (E // world) * rpn
+        for seed in range(2):
+            e = equal_quota_routing(T, k, E, n_nodes, M, 500 + seed)
+            for gm in (M, None):
+                got = orc.plan_ta2a(e, world, E, rpn, gm)
+                want = _plan_brute(e, slots, n_nodes)
+                for a, b in zip(got, want):
+                    assert a.dtype == np.int64 and a.tolist() == b
+            u_src, u_node, counts, inv = got
+            assert (u_src[inv].reshape(T, k) == np.arange(T)[:, None]).all()
+            assert (u_node[inv].reshape(T, k) == e // slots).all()
+            assert orc.send_offsets(counts).tolist() == [int(sum(counts[:i])) for i in range(n_nodes)]
+
+
+def test_plan_general_fanout_without_groups_m():
+    e = np.array([[0, 1, 2, 3], [0, 4, 5, 6], [7, 6, 5, 4]], dtype=np.int64)   # fan-outs 1, 2, 1
+    u_src, u_node, counts, inv = orc.plan_ta2a(e, 4, 8, 2, None)
+    assert u_src.tolist() == [0, 1, 1, 2] and u_node.tolist() == [0, 0, 1, 1]
+    assert counts.tolist() == [2, 2] and inv.tolist() == [0, 0, 0, 0, 1, 2, 2, 2, 3, 3, 3, 3]
+    assert orc.dispatch_stats(e, 4, 8, 2)["rows_ta2a"] == 4
+
+
+def test_plan_key_range_guard():
+    with pytest.raises(ValueError, match="2\\^24"):
+        orc.plan_ta2a(np.zeros((1 << 21, 1), np.int64), 64, 64, 8, None)
+
+
+# ----------------------------------------------------------------------------- pack
+
+def _check_pack_by_definition(e, gates, hidden, out, slots, q):
+    payload, mask, gate_rows, u_src, counts = out
+    T, k = e.shape
+    r = 0
+    for n in range(len(counts)):
+        for t in range(T):
+            mine = sorted(int(x) for x in e[t] if x // slots == n)
+            if not mine:
+                continue
+            assert u_src[r] == t and np.array_equal(payload[r], hidden[t])
+            assert mask[r].tolist() == [x % slots for x in mine]
+            assert gate_rows[r].tolist() == [gates[t, list(e[t]).index(x)] for x in mine]
+            r += 1
+        assert counts[n] == r - int(sum(counts[:n]))
+    assert r == payload.shape[0]
+
+
+@pytest.mark.parametrize("sort_rows", [True, False])
+def test_k2_pack_by_definition_on_reference_geometries(literals, sort_rows):
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        n_nodes, slots = world // rpn, (E // world) * rpn
+        for fmt in ("f32", "u16"):
+            rng = np.random.default_rng(T * 7 + k)
+            e = equal_quota_routing(T, k, E, n_nodes, M, 500, sort_rows)
+            if fmt == "f32":
+                hidden = rng.standard_normal((T, 16)).astype(np.float32)
+                gates = rng.random((T, k)).astype(np.float32)
+            else:
+                hidden = rng.integers(0, 65536, (T, 16)).astype(np.uint16)
+                gates = rng.integers(0, 65536, (T, k)).astype(np.uint16)
+            out = orc.k2_pack(hidden, e, gates, world, E, rpn, M)
+            _check_pack_by_definition(e, gates, hidden, out, slots, k // M)
+            assert out[0].shape == (T * M, 16) and out[1].shape == (T * M, k // M)
+            assert out[1].dtype == np.int64 and out[2].dtype == gates.dtype
+            assert np.array_equal(out[1], np.sort(out[1], axis=1))
+            assert int(out[4].sum()) == T * M
+
+
+def test_k2_pack_errors():
+    h = np.zeros((4, 8), np.float32)
+    e = np.array([[0, 2, 4, 6]] * 4, dtype=np.int64)
+    g = np.zeros((4, 4), np.float32)
+    with pytest.raises(ValueError):
+        orc.k2_pack(h, e, g, 4, 8, 3, 2)                      # world % rpn
+    with pytest.raises(ValueError, match="slots"):
+        orc.k2_pack(h, e, g, 8, 512, 8, 2)                    # 64 slots per node
+    with pytest.raises(ValueError, match="out of range"):
+        orc.k2_pack(h, e + 8, g, 4, 8, 2, 2)
+    with pytest.raises(ValueError):
+        orc.k2_pack(h, e, g[:, :3], 4, 8, 2, 2)
+
+
+# ----------------------------------------------------------------------------- arrival
+
+def test_k1_equals_library_stable_sort(literals):
+    for R, q, epr, rpn, H in literals["k1_geometries"]["rows"]:
+        for seed in range(2):
+            rslot = arrival_plane(R, q, epr, rpn, 100 + seed)
+            rng = np.random.default_rng(seed)
+            rx = rng.standard_normal((R, H)).astype(np.float32)
+            rgate = rng.random((R, q)).astype(np.float32)
+            send, gp, r_idx, s_idx, i_send = orc.k1_arrival(rx, rslot, rgate, q, epr, rpn)
+            owner = torch.from_numpy(rslot.reshape(-1) // epr)
+            ordo = torch.sort(owner, stable=True).indices.numpy()
+            assert np.array_equal(r_idx, ordo // q) and np.array_equal(s_idx, rslot.reshape(-1)[ordo])
+            assert np.array_equal(send, rx[ordo // q]) and np.array_equal(gp, rgate.reshape(-1)[ordo])
+            assert np.array_equal(i_send, np.bincount(owner.numpy(), minlength=rpn))
+            assert i_send.shape == (rpn,) and i_send.dtype == np.int64 and r_idx.dtype == np.int64
+            # counting-sort view: owners non-decreasing, flat pair ids increasing inside an owner
+            o = s_idx // epr
+            assert (np.diff(o) >= 0).all()
+            assert all((np.diff(ordo[o == b]) > 0).all() for b in range(rpn))
+            pos = orc.arrival_positions(rslot, epr, rpn)
+            assert np.array_equal(pos[ordo], np.arange(R * q))
+
+
+def test_k1_degenerate_and_empty(literals):
+    d = literals["k1_degenerate"]["all_zero_slot_rows"]
+    rslot = arrival_plane(d["R"], d["quota"], d["epr"], d["rpn"], 5, degenerate=True)
+    rx = np.arange(d["R"] * d["H"], dtype=np.float32).reshape(d["R"], d["H"])
+    rg = np.arange(d["R"] * d["quota"], dtype=np.float32).reshape(d["R"], d["quota"])
+    send, gp, r_idx, s_idx, i_send = orc.k1_arrival(rx, rslot, rg, d["quota"], d["epr"], d["rpn"])
+    assert r_idx.tolist() == [p // d["quota"] for p in range(d["R"] * d["quota"])]
+    assert i_send.tolist() == [d["R"] * d["quota"]] + [0] * (d["rpn"] - 1)
+    assert np.array_equal(gp, rg.reshape(-1)) and (s_idx == 0).all()
+    z = literals["k1_degenerate"]["empty_arrival"]
+    out = orc.k1_arrival(np.zeros((0, z["H"]), np.float32), np.zeros((0, z["quota"]), np.int64),
+                         np.zeros((0, z["quota"]), np.float32), z["quota"], z["epr"], z["rpn"])
+    assert out[0].shape == (0, z["H"]) and out[4].shape == (z["rpn"],) and int(out[4].sum()) == z["i_send_sum"]
+
+
+def test_hist_and_argsort_reduce_to_library():
+    rng = np.random.default_rng(6)
+    for n in (0, 1, 100, 24576):
+        key = rng.integers(0, 8, n)
+        assert np.array_equal(orc.fixed_hist(key, 8), np.bincount(key, minlength=8))
+        assert np.array_equal(orc.stable_argsort_small(key, 8),
+                              torch.sort(torch.from_numpy(key), stable=True).indices.numpy())
+    with pytest.raises(IndexError):
+        orc.fixed_hist(np.array([0, 8]), 8)
+
+
+def test_regroup_dropless_and_capacity():
+    my_slot = np.array([5, 4, 5, 5, 4, 7, 5], dtype=np.int64)         # card 1 of epr 4: experts 4..7
+    rows = np.arange(7 * 3, dtype=np.float32).reshape(7, 3)
+    permuted, order, tpe = orc.regroup(rows, my_slot, epr=4, my_local=1)
+    assert order.tolist() == [1, 4, 0, 2, 3, 6, 5] and tpe.tolist() == [2, 4, 0, 1]
+    assert np.array_equal(permuted, rows[order])
+    padded, dest, kept, tpe2, kpe = orc.regroup(rows, my_slot, epr=4, my_local=1, capacity=3)
+    assert tpe2.tolist() == [2, 4, 0, 1] and kpe.tolist() == [2, 3, 0, 1]
+    assert dest.tolist() == [3, 0, 4, 5, 1, 9, -1] and kept.tolist() == [1, 1, 1, 1, 1, 1, 0]
+    assert padded.shape == (12, 3)
+    assert np.array_equal(padded[[0, 1, 3, 4, 5, 9]], rows[[1, 4, 0, 2, 3, 5]])
+    assert (padded[[2, 6, 7, 8, 10, 11]] == 0).all()
+    # a capacity nobody reaches is the drop-less layout with gaps
+    padded, dest, kept, _, _ = orc.regroup(rows, my_slot, epr=4, my_local=1, capacity=7)
+    assert kept.all()
+    assert np.array_equal(np.concatenate([padded[x * 7:x * 7 + c] for x, c in enumerate(tpe)]), permuted)
+
+
+# ----------------------------------------------------------------------------- combine
+
+def test_gather_reduce_small_literal_and_drop():
+    src = np.array([[1.0, 2.0], [10.0, 20.0], [100.0, 200.0]], dtype=np.float32)
+    idx = np.array([[0, 2], [1, -1]])
+    w = np.array([[0.5, 0.25], [2.0, 9.0]], dtype=np.float32)
+    assert orc.gather_reduce(src, idx, w).tolist() == [[25.5, 51.0], [20.0, 40.0]]
+    assert orc.gather_reduce(src, idx, None).tolist() == [[101.0, 202.0], [10.0, 20.0]]
+
+
+def test_combine_order_is_fp32_left_to_right():
+    # (1 + 2^-24) + 2^-24 : left to right stays 1.0 twice; right to left would reach 1+2^-23
+    src = np.array([[1.0], [2.0 ** -24], [2.0 ** -24]], dtype=np.float32)
+    assert orc.gather_reduce(src, np.array([[0, 1, 2]]), None)[0, 0] == np.float32(1.0)
+    assert orc.gather_reduce(src, np.array([[1, 2, 0]]), None)[0, 0] == np.float32(1.0 + 2.0 ** -23)
+
+
+def test_one_level_table_reproduces_reference_two_level_sum(literals):
+    """The fused combine adds a token's k rows in ascending expert id; that is the same
+    fp32 sum the two reference ``index_add`` levels perform (slot ascending inside a send
+    row, node ascending across a token's rows) whenever each level starts from zero --
+    except that two-level adds level-1 partial sums, so the comparison is to tolerance,
+    while for M == 1 or quota == 1 it is exact."""
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        n_nodes, slots, q = world // rpn, (E // world) * rpn, k // M
+        epr = E // world
+        rng = np.random.default_rng(k * 13 + T)
+        e = equal_quota_routing(T, k, E, n_nodes, M, 700)
+        gates = rng.random((T, k)).astype(np.float32)
+        x = rng.standard_normal((T, 8)).astype(np.float32)
+        payload, mask, gate_rows, u_src, _ = orc.k2_pack(x, e, gates, world, E, rpn, M)
+        send, gp, r_idx, s_idx, _ = orc.k1_arrival(payload, mask, gate_rows, q, epr, rpn)
+        ye = (send * ((s_idx[:, None] + 1) / np.float32(slots))).astype(np.float32)   # "expert" output
+        two = orc.combine_reference_order(ye, gp, r_idx, u_src, T * M, T)
+        _, _, _, inverse = orc.plan_ta2a(e, world, E, rpn, M)
+        pair_tab, order = orc.token_pair_table(e, inverse, q)
+        pos = orc.arrival_positions(mask, epr, rpn)
+        one = orc.gather_reduce(ye, pos[pair_tab], np.take_along_axis(gates, order, 1))
+        if M == 1 or q == 1:
+            assert np.array_equal(one, two)
+        assert np.allclose(one, two, rtol=1e-5, atol=1e-6)
+        # and both are the plain definition y[t] = sum_j gate * x[t] * (slot+1)/slots
+        want = (x.astype(np.float64) * (gates.astype(np.float64) * ((e % slots + 1) / slots)).sum(1)[:, None])
+        assert np.allclose(one, want, rtol=1e-5, atol=1e-6)
+
+
+def test_combine_formats():
+    rng = np.random.default_rng(8)
+    src = rng.standard_normal((6, 256)).astype(np.float32)
+    idx = np.array([[0, 1, 2], [3, 4, 5]])
+    w = rng.random((2, 3)).astype(np.float32)
+    ref = orc.gather_reduce(src, idx, w)
+    bf = orc.f32_to_bf16(src)
+    got = orc.combine(bf, idx, w, "bf16", "bf16")
+    assert got.dtype == np.uint16
+    assert np.allclose(orc.bf16_to_f32(got), ref, rtol=2e-2, atol=2e-2)
+    rows8 = orc.fp8_quantise_rows(src)
+    got8 = orc.combine(rows8, idx, w, "fp8", "f32", hidden=256)
+    assert np.allclose(got8, ref, rtol=0.15, atol=0.15)
+    assert np.array_equal(orc.combine(src, idx, w), ref)
