@@ -1,0 +1,197 @@
+/*
+ * terrace_hip.h -- C ABI of libterrace_hip.so: one rank's TerraceMoE dispatch/combine data
+ * path as hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * Every entry point
+ *   - takes plain device pointers and sizes (no torch types), a caller-provided workspace
+ *     where one is needed, and the HIP stream to launch on (a hipStream_t passed as void*);
+ *   - only enqueues work: it never allocates, frees, synchronises or keeps a pointer, and
+ *     keeps no mutable global state, so it may be called from any host thread on any stream;
+ *   - returns TERRACE_OK or a negative terrace_status and never throws.
+ * Outputs are allocated by the caller (the Python binding uses torch's caching allocator,
+ * as the reference binding uses at::empty: terrace/ops/csrc/terrace_ops.cpp:147-160).
+ *
+ * Index planes are int64 and gate planes travel in the payload's storage type, exactly as
+ * the reference operators return them.  Payload rows are moved as opaque bytes: `row_bytes`
+ * is hidden*itemsize (or the fp8-with-scales row width); any value is accepted, rows whose
+ * width and base pointers are multiples of 16 bytes take the 16-byte-per-lane path.
+ *
+ * `status` arguments point to TERRACE_STATUS_WORDS int32 in device memory that the call
+ * overwrites: word 0 is a bit set of terrace_fault values (0 = inputs were well formed).
+ * Kernels cannot raise, so malformed input is contained (ids clamped, results unspecified
+ * but in range) and reported there; the caller decides when to pay the read-back, as the
+ * reference's plan does on its first and every 256th call (terrace/ta2a.py:161-204).
+ */
+#ifndef TERRACE_HIP_H
+#define TERRACE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *terrace_stream_t; /* hipStream_t */
+
+#if defined(__GNUC__)
+#define TERRACE_API __attribute__((visibility("default")))
+#else
+#define TERRACE_API
+#endif
+
+enum terrace_status {
+    TERRACE_OK = 0,
+    TERRACE_EINVAL = -22,  /* bad geometry / null pointer / unsupported size */
+    TERRACE_ENOSPC = -28,  /* workspace smaller than the matching *_workspace() answer */
+    TERRACE_ELAUNCH = -5   /* the HIP runtime refused a launch (hipGetLastError != 0) */
+};
+
+enum terrace_dtype {
+    TERRACE_F32 = 0,
+    TERRACE_BF16 = 1,
+    TERRACE_F16 = 2,
+    TERRACE_FP8_E4M3_B128 = 3 /* row = hidden e4m3 codes, then hidden/128 fp32 block scales */
+};
+
+enum terrace_route_mode { /* terrace/routing.py:66 _MODES, same order */
+    TERRACE_ROUTE_FULL = 0,
+    TERRACE_ROUTE_GROUP_LIMITED = 1,
+    TERRACE_ROUTE_QUOTA_ONLY = 2,
+    TERRACE_ROUTE_GLOBAL_TOPK = 3,
+    /* or-ed into `mode`: use the LDS-staged kernel even where the register-resident one
+     * applies (both give identical results; this exists so tests can compare them) */
+    TERRACE_ROUTE_FORCE_GENERIC = 0x100
+};
+
+enum terrace_fault {
+    TERRACE_FAULT_ID_RANGE = 1, /* an expert / slot id outside its range was clamped */
+    TERRACE_FAULT_QUOTA = 2,    /* a token's run on a node does not hold exactly k/M experts */
+    TERRACE_FAULT_FANOUT = 4    /* a token does not touch exactly M distinct nodes */
+};
+
+#define TERRACE_STATUS_WORDS 4
+
+TERRACE_API const char *terrace_version(void);
+TERRACE_API const char *terrace_strerror(int status);
+
+/* Identity copy of nbytes; the streaming-copy roofline probe.
+ * Replaces terrace::passthrough (terrace/ops/csrc/terrace_ops.cpp:230, kernel
+ * terrace/ops/ascendc/op_kernel/terrace_passthrough.cpp:119). */
+TERRACE_API int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t stream);
+
+/* T-Route (terrace/routing.py:45-96).  affinity [T,E] f32, bias [E] f32, gate_affinity
+ * [T,E] f32 or NULL (= affinity).  Writes expert_idx [T,k] i64, gates [T,k] f32,
+ * group_idx [T,G] i64 with G = top_groups (full, group_limited), n_groups (quota_only) or
+ * top_k (global_topk).  Ties go to the lowest index; gates are raw/sum(raw) with the sum
+ * taken left to right in fp32.  pool = TRouteConfig.group_score_pool (1 or 2). */
+TERRACE_API int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T,
+                    int n_experts, int n_groups, int top_k, int top_groups, int pool, int mode,
+                    int64_t *expert_idx, float *gates, int64_t *group_idx, terrace_stream_t stream);
+
+/* expert_load (terrace/routing.py:112-113) and fixed_hist (terrace/ta2a_fwd.py:299-321):
+ * out[b] = #{i : idx[i] == b}; out is int64 [n_buckets] or, with as_float != 0, float32. */
+TERRACE_API size_t terrace_hist_workspace(int64_t n, int n_buckets);
+TERRACE_API int terrace_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status,
+                 void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+
+/* _stable_argsort_small (terrace/ta2a_fwd.py:324-345): order [n] i64 = stable ascending
+ * argsort of key (values in [0, n_buckets)); hist [n_buckets] i64 may be NULL. */
+TERRACE_API size_t terrace_argsort_small_workspace(int64_t n, int n_buckets);
+TERRACE_API int terrace_argsort_small(const int64_t *key, int64_t n, int n_buckets, int64_t *order, int64_t *hist,
+                          int32_t *status, void *workspace, size_t workspace_bytes,
+                          terrace_stream_t stream);
+
+/* Send side: dispatch index build + Hop-A deduplicated pack under equal quota.
+ * Replaces terrace::k2_pack (terrace/ops/csrc/terrace_k2_pack.cpp:209-211; spec
+ * terrace/ops/k2_ref.py:70-134) = plan_ta2a(groups_m=M) (terrace/ta2a.py:70-275)
+ * + hidden[u_src] (terrace/ta2a_fwd.py:473) + _pack_quota_wire (terrace/ta2a_fwd.py:177-249).
+ *   hidden [T,row_bytes] (NULL: index build only, payload ignored), expert_idx [T,k] i64,
+ *   gates [T,k] elements of gate_bytes (2 or 4) bytes (NULL: gate_rows ignored).
+ * Writes payload [T*M,row_bytes], mask [T*M,q] i64 ascending node-local slot ids, gate_rows
+ * [T*M,q], u_src [T*M] i64, node_counts [n_nodes] i64; each of the optional planes may be
+ * NULL: u_node [T*M] i64, inverse [T*k] i64 (row carrying slot (t,j)), node_offsets
+ * [n_nodes] i64 (exclusive prefix of node_counts), pair_table [T,k] i64 (flat Hop-A pair id
+ * row*q+i of the token's s-th smallest expert), sort_order [T,k] i64 (its column j),
+ * token_rows [T,M] i64 (the token's send rows, node ascending) and gate_sorted [T,k] (the
+ * token's gates in ascending expert order, gate_bytes-wide elements).
+ * Rows come out in (node ascending, token ascending) order.
+ * status word 1 = number of occupied (token, node) pairs, word 2 = how many of them hold other
+ * than k/M experts (the two quantities the guard of terrace/ta2a.py:170-204 tests). */
+TERRACE_API size_t terrace_k2_pack_workspace(int64_t T, int k, int n_nodes, int groups_m);
+TERRACE_API int terrace_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T,
+                    int64_t row_bytes, int gate_bytes, int k, int world, int n_experts, int rpn,
+                    int groups_m, void *payload, int64_t *mask, void *gate_rows, int64_t *u_src,
+                    int64_t *node_counts, int64_t *u_node, int64_t *inverse, int64_t *node_offsets,
+                    int64_t *pair_table, int64_t *sort_order, int64_t *token_rows, void *gate_sorted,
+                    int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+
+/* _pack_quota_wire (terrace/ta2a_fwd.py:177-249) for a caller that already holds `inverse`:
+ * for the token's s-th smallest expert (column j), run m = s/q, i = s%q:
+ *   slot_tab[inverse[t,j0(m)]][i] = expert % slots, gate_tab[same] = gates[t,j]
+ * where j0(m) is the column of the run's first expert.  slot_tab [n_rows,q] i64 and gate_tab
+ * [n_rows,q] must be zero-filled by the caller (rows never named keep slot 0 / gate 0);
+ * rows outside [0, n_rows) are skipped and reported as TERRACE_FAULT_ID_RANGE. */
+TERRACE_API int terrace_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse,
+                                        int64_t T, int k, int gate_bytes, int64_t n_rows, int slots, int quota,
+                                        int64_t *slot_tab, void *gate_tab, int32_t *status,
+                                        terrace_stream_t stream);
+
+/* Hop-B arrival chain.  Replaces terrace::k1_arrival (terrace/ops/csrc/terrace_ops.cpp:231-232;
+ * spec terrace/ops/__init__.py:255-300; kernel terrace/ops/ascendc/op_kernel/terrace_k1_arrival.cpp).
+ *   rx [R,row_bytes] (NULL: index planes only), rslot [R,quota] i64, rgate [R,quota] of
+ *   gate_bytes-wide elements (NULL: gate_pairs ignored).
+ * Pairs p = r*quota+i are placed in stable ascending order of rslot[p]/epr.  Writes send_buf
+ * [P,row_bytes], gate_pairs [P], r_idx [P] i64, slot_idx [P] i64, i_send [rpn] i64 and, when
+ * not NULL, pair_pos [P] i64 (the place pair p landed at: the inverse permutation). */
+TERRACE_API size_t terrace_k1_arrival_workspace(int64_t R, int quota, int rpn);
+TERRACE_API int terrace_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
+                       int64_t row_bytes, int gate_bytes, int quota, int epr, int rpn, int my_local,
+                       void *send_buf, void *gate_pairs, int64_t *r_idx, int64_t *slot_idx,
+                       int64_t *i_send, int64_t *pair_pos, int32_t *status, void *workspace,
+                       size_t workspace_bytes, terrace_stream_t stream);
+
+/* Expert-order regroup on the expert card (terrace/ta2a_fwd.py:641-646), optionally with a
+ * per-expert capacity (no counterpart in the reference, which is drop-less:
+ * terrace/ta2a_dispatch.py:248-250).  exp_j = my_slot - my_local*epr in [0, epr).
+ *   capacity < 0: permuted [P,row_bytes] = node_rx[order], order [P] i64 stable by exp_j.
+ *   capacity >= 0: permuted [epr*capacity,row_bytes], expert x keeps its first `capacity`
+ *     rows in stable order at x*capacity+rank, unused rows are zero; dest [P] i64 is that
+ *     place or -1 for a dropped row; kept [P] u8.
+ * tokens_per_expert [epr] i64 counts before the cut; kept_per_expert [epr] i64 (may be NULL).
+ * node_rx NULL: index planes only.  gate planes ride along when my_gate != NULL:
+ * permuted_gate has one gate_bytes-wide element per permuted row. */
+TERRACE_API size_t terrace_regroup_workspace(int64_t P, int epr, int64_t capacity);
+TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P,
+                    int64_t row_bytes, int gate_bytes, int epr, int my_local, int64_t capacity,
+                    void *permuted, void *permuted_gate, int64_t *order, int64_t *dest, uint8_t *kept,
+                    int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status,
+                    void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+
+/* out[i] = src[idx[i]] for i < n_out (row gather; idx < 0 writes a zero row). */
+TERRACE_API int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes,
+                        void *out, terrace_stream_t stream);
+
+/* out[i] = table[idx[i]] over int64 planes; idx < 0 or table value < 0 gives -1. */
+TERRACE_API int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out,
+                        terrace_stream_t stream);
+
+/* Gate-weighted combine (terrace/ta2a_fwd.py:658-670; one level: terrace/ep_dist.py:121-122):
+ *   out[i,:] = sum_{j<fan} w[i,j] * decode(src[idx[i,j],:])      (idx < 0 contributes nothing)
+ * accumulated in fp32 as acc = fl(acc + fl(w*x)) for j = 0..fan-1, rounded once to out_dtype.
+ * src rows are src_dtype (F32, BF16, F16 or FP8_E4M3_B128 with `hidden` elements per row),
+ * weights [n_out,fan] are w_dtype (F32, BF16, F16) or NULL (all ones), idx is [n_out,fan] i64,
+ * out is [n_out,hidden] of out_dtype (F32, BF16 or F16). */
+TERRACE_API int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const void *weights,
+                    int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
+                    terrace_stream_t stream);
+
+/* Hop-A counts exchange buffer (terrace/ta2a_dispatch.py:197-211): send [world] i64 is zero
+ * except send[n*rpn + my_local] = node_counts[n]. */
+TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local,
+                             int64_t *send, terrace_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TERRACE_HIP_H */

@@ -1,0 +1,161 @@
+// extern "C" surface of libterrace_hip.so: argument checks and dispatch to the launchers.
+#include "common.hpp"
+
+namespace terrace {
+int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
+int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
+                   int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
+int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
+int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s);
+template <typename I>
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
+int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
+                int k, int M, int pool, int mode, int64_t *expert_idx, float *gates, int64_t *group_idx,
+                int force_generic, hipStream_t s);
+size_t hist_workspace(int64_t n, int n_buckets);
+int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status, void *ws,
+             size_t ws_bytes, hipStream_t s);
+int run_argsort_small(const int64_t *key, int64_t n, int n_buckets, int64_t *order, int64_t *hist, int32_t *status,
+                      void *ws, size_t ws_bytes, hipStream_t s);
+size_t k1_workspace(int64_t R, int quota, int rpn);
+int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                   int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
+                   int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
+                   size_t ws_bytes, hipStream_t s);
+size_t regroup_workspace(int64_t P, int epr, int64_t capacity);
+int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
+                int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
+                int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
+                int32_t *status, void *ws, size_t ws_bytes, hipStream_t s);
+size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m);
+int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
+                int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
+                void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node, int64_t *inverse,
+                int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order, int64_t *token_rows,
+                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, hipStream_t s);
+int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
+                        int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
+                        int32_t *status, hipStream_t s);
+}  // namespace terrace
+
+using namespace terrace;
+
+static bool float_dtype(int d) { return d == TERRACE_F32 || d == TERRACE_BF16 || d == TERRACE_F16; }
+
+extern "C" {
+
+const char *terrace_version(void) { return "terrace-hip 0.1 (gfx950)"; }
+
+const char *terrace_strerror(int status) {
+    switch (status) {
+        case TERRACE_OK: return "ok";
+        case TERRACE_EINVAL: return "invalid argument (geometry, null pointer or unsupported size)";
+        case TERRACE_ENOSPC: return "workspace too small";
+        case TERRACE_ELAUNCH: return "HIP kernel launch failed";
+        default: return "unknown status";
+    }
+}
+
+int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t stream) {
+    if (nbytes && (!x || !y)) return TERRACE_EINVAL;
+    return launch_copy(x, y, nbytes, (hipStream_t)stream);
+}
+
+int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int n_experts,
+                    int n_groups, int top_k, int top_groups, int pool, int mode, int64_t *expert_idx, float *gates,
+                    int64_t *group_idx, terrace_stream_t stream) {
+    const int force = (mode & TERRACE_ROUTE_FORCE_GENERIC) ? 1 : 0;
+    return run_t_route(affinity, bias, gate_affinity, T, n_experts, n_groups, top_k, top_groups, pool,
+                       mode & ~TERRACE_ROUTE_FORCE_GENERIC, expert_idx, gates, group_idx, force, (hipStream_t)stream);
+}
+
+size_t terrace_hist_workspace(int64_t n, int n_buckets) { return hist_workspace(n, n_buckets); }
+
+int terrace_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status,
+                 void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_hist(idx, n, n_buckets, out, as_float, status, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+size_t terrace_argsort_small_workspace(int64_t n, int n_buckets) { return hist_workspace(n, n_buckets); }
+
+int terrace_argsort_small(const int64_t *key, int64_t n, int n_buckets, int64_t *order, int64_t *hist,
+                          int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_argsort_small(key, n, n_buckets, order, hist, status, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+size_t terrace_k2_pack_workspace(int64_t T, int k, int n_nodes, int groups_m) {
+    return k2_workspace(T, k, n_nodes, groups_m);
+}
+
+int terrace_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
+                    int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload,
+                    int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
+                    int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
+                    int64_t *token_rows, void *gate_sorted, int32_t *status, void *workspace,
+                    size_t workspace_bytes, terrace_stream_t stream) {
+    return run_k2_pack(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, world, n_experts, rpn, groups_m,
+                       payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets, pair_table,
+                       sort_order, token_rows, gate_sorted, status, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
+                            int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
+                            int32_t *status, terrace_stream_t stream) {
+    return run_pack_quota_wire(expert_idx, gates, inverse, T, k, gate_bytes, n_rows, slots, quota, slot_tab,
+                               gate_tab, status, (hipStream_t)stream);
+}
+
+size_t terrace_k1_arrival_workspace(int64_t R, int quota, int rpn) { return k1_workspace(R, quota, rpn); }
+
+int terrace_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                       int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
+                       int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status,
+                       void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_k1_arrival(rx, rslot, rgate, R, row_bytes, gate_bytes, quota, epr, rpn, my_local, send_buf,
+                          gate_pairs, r_idx, slot_idx, i_send, pair_pos, status, workspace, workspace_bytes,
+                          (hipStream_t)stream);
+}
+
+size_t terrace_regroup_workspace(int64_t P, int epr, int64_t capacity) { return regroup_workspace(P, epr, capacity); }
+
+int terrace_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
+                    int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
+                    int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert,
+                    int64_t *kept_per_expert, int32_t *status, void *workspace, size_t workspace_bytes,
+                    terrace_stream_t stream) {
+    return run_regroup(node_rx, my_slot, my_gate, P, row_bytes, gate_bytes, epr, my_local, capacity, permuted,
+                       permuted_gate, order, dest, kept, tokens_per_expert, kept_per_expert, status, workspace,
+                       workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes, void *out,
+                        terrace_stream_t stream) {
+    if (n_out < 0 || row_bytes < 0) return TERRACE_EINVAL;
+    if (n_out && row_bytes && (!src || !idx || !out)) return TERRACE_EINVAL;
+    return launch_gather_rows<int64_t>(src, out, idx, n_out, row_bytes, (hipStream_t)stream);
+}
+
+int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream) {
+    if (n < 0 || (n && (!table || !idx || !out))) return TERRACE_EINVAL;
+    return launch_index_chain(table, idx, n, out, (hipStream_t)stream);
+}
+
+int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const void *weights, int w_dtype,
+                    int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, terrace_stream_t stream) {
+    if (n_out < 0 || fan <= 0 || hidden < 0) return TERRACE_EINVAL;
+    if (src_dtype < TERRACE_F32 || src_dtype > TERRACE_FP8_E4M3_B128 || !float_dtype(out_dtype)) return TERRACE_EINVAL;
+    if (weights && !float_dtype(w_dtype)) return TERRACE_EINVAL;
+    if (src_dtype == TERRACE_FP8_E4M3_B128 && hidden % 128) return TERRACE_EINVAL;
+    if (n_out && hidden && (!src || !idx || !out)) return TERRACE_EINVAL;
+    return launch_combine(src, src_dtype, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
+                          (hipStream_t)stream);
+}
+
+int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send,
+                             terrace_stream_t stream) {
+    if (world <= 0 || rpn <= 0 || world % rpn || my_local < 0 || my_local >= rpn || !node_counts || !send)
+        return TERRACE_EINVAL;
+    return launch_send_splits(node_counts, world, rpn, my_local, send, (hipStream_t)stream);
+}
+
+}  // extern "C"

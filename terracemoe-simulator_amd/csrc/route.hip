@@ -1,0 +1,397 @@
+// T-Route: group-limited top-k with equal per-group quota, one wavefront per token.
+//
+// Selection order everywhere is the strict total order (value descending, index ascending):
+// "the next pick" is the largest candidate strictly after the previous pick in that order, so
+// no taken-flags are needed and ties always go to the lowest index.
+//
+//   route_wave_kernel     mode "full" when the E (padded) scores map onto the wave as VPL
+//                         consecutive values per lane and every group covers a power-of-two
+//                         number of whole lanes.  Scores never leave registers: group top-2 by a
+//                         DPP butterfly inside the group's lanes, top-M groups by a butterfly
+//                         across groups, then all M selected groups pick their q experts at once.
+//   route_generic_kernel  every mode and every geometry; scores staged in wave-private LDS.
+//
+// Both write expert_idx / group_idx as int64 and gates = raw / (raw_0 + raw_1 + ... ) with the
+// sum taken left to right in fp32 (terrace/routing.py:94-95).
+#include "common.hpp"
+
+#include <math.h>
+
+namespace terrace {
+
+constexpr float kNegInf = -INFINITY;
+constexpr float kPosInf = INFINITY;
+
+// (v, i) strictly after (pv, pi) in (value desc, index asc) order
+__device__ __forceinline__ bool after(float v, int i, float pv, int pi) { return v < pv || (v == pv && i > pi); }
+// (v, i) ahead of (bv, bi)
+__device__ __forceinline__ bool ahead(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+// One butterfly step of a symmetric wave reduction at distance D.  Distances 4 and 8 use the
+// DPP half-row / row mirrors, which pair a lane with one whose lower bits differ as well; that
+// is the same reduction because every caller reduces at distances D/2, D/4, ... first (or the
+// lanes below D already agree), so all lanes of the mirrored sub-row hold one value.
+template <int D>
+__device__ __forceinline__ int bfly_i(int v) {
+    if constexpr (D == 1) return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false);
+    else if constexpr (D == 2) return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false);
+    else if constexpr (D == 4) return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false);
+    else if constexpr (D == 8) return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false);
+    else if constexpr (D == 16) return __builtin_amdgcn_ds_swizzle(v, 0x401F);
+    else return __shfl_xor(v, 32, kWave);
+}
+template <int D>
+__device__ __forceinline__ float bfly_f(float v) { return __int_as_float(bfly_i<D>(__float_as_int(v))); }
+
+template <int D>
+__device__ __forceinline__ void top2_step(float &a1, float &a2) {
+    const float b1 = bfly_f<D>(a1), b2 = bfly_f<D>(a2);
+    const float hi = fmaxf(a1, b1), lo = fminf(a1, b1);
+    a2 = fmaxf(lo, fmaxf(a2, b2));
+    a1 = hi;
+}
+
+template <int D>
+__device__ __forceinline__ void best_step(float &v, int &i) {
+    const float ov = bfly_f<D>(v);
+    const int oi = bfly_i<D>(i);
+    if (ahead(ov, oi, v, i)) {
+        v = ov;
+        i = oi;
+    }
+}
+
+// Reduce over lane distances [from, to): from and to are powers of two (uniform).
+__device__ __forceinline__ void top2_range(float &a1, float &a2, int from, int to) {
+    if (from <= 1 && to > 1) top2_step<1>(a1, a2);
+    if (from <= 2 && to > 2) top2_step<2>(a1, a2);
+    if (from <= 4 && to > 4) top2_step<4>(a1, a2);
+    if (from <= 8 && to > 8) top2_step<8>(a1, a2);
+    if (from <= 16 && to > 16) top2_step<16>(a1, a2);
+    if (from <= 32 && to > 32) top2_step<32>(a1, a2);
+}
+__device__ __forceinline__ void best_range(float &v, int &i, int from, int to) {
+    if (from <= 1 && to > 1) best_step<1>(v, i);
+    if (from <= 2 && to > 2) best_step<2>(v, i);
+    if (from <= 4 && to > 4) best_step<4>(v, i);
+    if (from <= 8 && to > 8) best_step<8>(v, i);
+    if (from <= 16 && to > 16) best_step<16>(v, i);
+    if (from <= 32 && to > 32) best_step<32>(v, i);
+}
+
+// Shared epilogue: sel[0..k) holds the chosen expert ids (wave-private LDS).
+// An id outside [0, E) can only come from NaN scores (never ranked); it is clamped to 0.
+__device__ __forceinline__ void write_token(int *sel, float *raw, const float *gate_row, int k, int E, int64_t t,
+                                            int64_t *expert_idx, float *gates) {
+    const int lane = lane_id();
+    for (int j = lane; j < k; j += kWave) {
+        if ((unsigned)sel[j] >= (unsigned)E) sel[j] = 0;
+        raw[j] = gate_row[sel[j]];
+    }
+    __builtin_amdgcn_wave_barrier();
+    float den = 0.0f;
+    for (int j = 0; j < k; ++j) den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
+    for (int j = lane; j < k; j += kWave) {
+        expert_idx[t * k + j] = sel[j];
+        gates[t * k + j] = __fdiv_rn(((volatile float *)raw)[j], den);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// register-resident kernel, mode "full"
+// ---------------------------------------------------------------------------------------------
+template <int VPL>
+__global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restrict__ affinity,
+                                                            const float *__restrict__ bias,
+                                                            const float *__restrict__ gate_affinity, int64_t T, int E,
+                                                            int g, int k, int M, int pool, int lpg,
+                                                            int64_t *__restrict__ expert_idx,
+                                                            float *__restrict__ gates,
+                                                            int64_t *__restrict__ group_idx) {
+    extern __shared__ int32_t lds[];
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    int *sel = lds + w * 2 * k;
+    float *raw = (float *)(sel + k);
+    const int q = k / M;
+    const int my_group = lane / lpg;
+    const bool group_head = (lane & (lpg - 1)) == 0;
+    float b[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+        const int e = lane * VPL + i;
+        b[i] = e < E ? bias[e] : 0.0f;
+    }
+    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += (int64_t)gridDim.x * kWavesPerBlock) {
+        const float *row = affinity + t * E;
+        float s[VPL];
+        if (E == kWave * VPL) {
+            typedef float fvec __attribute__((ext_vector_type(VPL)));
+            if constexpr (VPL == 1) {
+                s[0] = row[lane];
+            } else if constexpr (VPL <= 4) {
+                const fvec v = *(const fvec *)(row + lane * VPL);
+#pragma unroll
+                for (int i = 0; i < VPL; ++i) s[i] = v[i];
+            } else {
+                typedef float f4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+                for (int c = 0; c < VPL / 4; ++c) {
+                    const f4 v = *(const f4 *)(row + lane * VPL + 4 * c);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[4 * c + i] = v[i];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) s[i] = __fadd_rn(s[i], b[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int e = lane * VPL + i;
+                s[i] = e < E ? __fadd_rn(row[e], b[i]) : kNegInf;
+            }
+        }
+        // group score: mean of the top two (or the top one) of the group's g values
+        float a1 = kNegInf, a2 = kNegInf;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const float v = s[i];
+            a2 = fmaxf(fminf(a1, v), a2);
+            a1 = fmaxf(a1, v);
+        }
+        top2_range(a1, a2, 1, lpg);
+        const bool real_group = my_group * g < E;
+        float score = (pool >= 2 && g >= 2) ? __fmul_rn(__fadd_rn(a1, a2), 0.5f) : a1;
+        if (!real_group) score = kNegInf;
+        const int gid = real_group ? my_group : 0x7FFFFFFF;
+        // top-M groups
+        int my_rank = -1;
+        float pv = kPosInf;
+        int pi = -1;
+        for (int m = 0; m < M; ++m) {
+            float cv = kNegInf;
+            int ci = 0x7FFFFFFF;
+            if (real_group && after(score, gid, pv, pi)) {
+                cv = score;
+                ci = gid;
+            }
+            best_range(cv, ci, lpg, kWave);
+            if (real_group && ci == gid) my_rank = m;
+            pv = cv;
+            pi = ci;
+            if (lane == 0) group_idx[t * M + m] = ci;
+        }
+        // every selected group picks its q experts, all groups at once
+        float ev = kPosInf;
+        int ei = -1;
+        for (int i = 0; i < q; ++i) {
+            float cv = kNegInf;
+            int ci = 0x7FFFFFFF;
+#pragma unroll
+            for (int x = 0; x < VPL; ++x) {
+                const int e = lane * VPL + x;
+                if (e < E && after(s[x], e, ev, ei) && ahead(s[x], e, cv, ci)) {
+                    cv = s[x];
+                    ci = e;
+                }
+            }
+            best_range(cv, ci, 1, lpg);
+            ev = cv;
+            ei = ci;
+            if (group_head && my_rank >= 0) sel[my_rank * q + i] = ci;
+        }
+        __builtin_amdgcn_wave_barrier();
+        write_token(sel, raw, (gate_affinity ? gate_affinity : affinity) + t * E, k, E, t, expert_idx, gates);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// generic kernel: all modes, scores in wave-private LDS
+// ---------------------------------------------------------------------------------------------
+// Wave-wide best of per-lane candidates.
+__device__ __forceinline__ void wave_best(float &v, int &i) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const float ov = __shfl_xor(v, d, kWave);
+        const int oi = __shfl_xor(i, d, kWave);
+        if (ahead(ov, oi, v, i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__restrict__ affinity,
+                                                               const float *__restrict__ bias,
+                                                               const float *__restrict__ gate_affinity, int64_t T,
+                                                               int E, int n_groups, int k, int M, int pool, int mode,
+                                                               int n_group_out, int64_t *__restrict__ expert_idx,
+                                                               float *__restrict__ gates,
+                                                               int64_t *__restrict__ group_idx) {
+    extern __shared__ int32_t lds[];
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    const int g = E / n_groups;
+    const int per_wave = E + n_groups + 2 * k + n_groups;
+    volatile float *s = (volatile float *)(lds + w * per_wave);
+    volatile float *gsc = s + E;
+    int *sel = (int *)(gsc + n_groups);
+    float *raw = (float *)(sel + k);
+    volatile int *selg = (volatile int *)(raw + k);
+    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += (int64_t)gridDim.x * kWavesPerBlock) {
+        const float *row = affinity + t * E;
+        for (int e = lane; e < E; e += kWave) s[e] = __fadd_rn(row[e], bias[e]);
+        __builtin_amdgcn_wave_barrier();
+        int n_sel_groups = 0, per_group = 0;
+        if (mode == TERRACE_ROUTE_FULL || mode == TERRACE_ROUTE_GROUP_LIMITED) {
+            for (int G = lane; G < n_groups; G += kWave) {
+                float a1 = kNegInf, a2 = kNegInf;
+                for (int x = 0; x < g; ++x) {
+                    const float v = s[G * g + x];
+                    a2 = fmaxf(fminf(a1, v), a2);
+                    a1 = fmaxf(a1, v);
+                }
+                gsc[G] = (pool >= 2 && g >= 2) ? __fmul_rn(__fadd_rn(a1, a2), 0.5f) : a1;
+            }
+            __builtin_amdgcn_wave_barrier();
+            float pv = kPosInf;
+            int pi = -1;
+            for (int m = 0; m < M; ++m) {
+                float cv = kNegInf;
+                int ci = 0x7FFFFFFF;
+                for (int G = lane; G < n_groups; G += kWave) {
+                    const float v = gsc[G];
+                    if (after(v, G, pv, pi) && ahead(v, G, cv, ci)) {
+                        cv = v;
+                        ci = G;
+                    }
+                }
+                wave_best(cv, ci);
+                pv = cv;
+                pi = ci;
+                if (lane == 0) selg[m] = ci;
+            }
+            n_sel_groups = M;
+            per_group = k / M;
+        } else if (mode == TERRACE_ROUTE_QUOTA_ONLY) {
+            for (int G = lane; G < n_groups; G += kWave) selg[G] = G;
+            n_sel_groups = n_groups;
+            per_group = k / n_groups;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (mode == TERRACE_ROUTE_FULL || mode == TERRACE_ROUTE_QUOTA_ONLY) {
+            for (int m = 0; m < n_sel_groups; ++m) {
+                const int G = selg[m];
+                float pv = kPosInf;
+                int pi = -1;
+                for (int i = 0; i < per_group; ++i) {
+                    float cv = kNegInf;
+                    int ci = 0x7FFFFFFF;
+                    for (int x = lane; x < g; x += kWave) {
+                        const float v = s[G * g + x];
+                        if (after(v, x, pv, pi) && ahead(v, x, cv, ci)) {
+                            cv = v;
+                            ci = x;
+                        }
+                    }
+                    wave_best(cv, ci);
+                    pv = cv;
+                    pi = ci;
+                    if (lane == 0) sel[m * per_group + i] = G * g + ci;
+                }
+            }
+            for (int m = lane; m < n_sel_groups; m += kWave) group_idx[t * n_group_out + m] = selg[m];
+        } else if (mode == TERRACE_ROUTE_GROUP_LIMITED) {
+            // free top-k over the M*g candidates; ties by candidate position (group rank first)
+            float pv = kPosInf;
+            int pi = -1;
+            for (int j = 0; j < k; ++j) {
+                float cv = kNegInf;
+                int ci = 0x7FFFFFFF;
+                for (int c = lane; c < M * g; c += kWave) {
+                    const float v = s[selg[c / g] * g + c % g];
+                    if (after(v, c, pv, pi) && ahead(v, c, cv, ci)) {
+                        cv = v;
+                        ci = c;
+                    }
+                }
+                wave_best(cv, ci);
+                pv = cv;
+                pi = ci;
+                if (lane == 0) sel[j] = selg[ci / g] * g + ci % g;
+            }
+            for (int m = lane; m < M; m += kWave) group_idx[t * n_group_out + m] = selg[m];
+        } else {
+            float pv = kPosInf;
+            int pi = -1;
+            for (int j = 0; j < k; ++j) {
+                float cv = kNegInf;
+                int ci = 0x7FFFFFFF;
+                for (int e = lane; e < E; e += kWave) {
+                    const float v = s[e];
+                    if (after(v, e, pv, pi) && ahead(v, e, cv, ci)) {
+                        cv = v;
+                        ci = e;
+                    }
+                }
+                wave_best(cv, ci);
+                pv = cv;
+                pi = ci;
+                if (lane == 0) {
+                    sel[j] = ci;
+                    group_idx[t * n_group_out + j] = ci / g;
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        write_token(sel, raw, (gate_affinity ? gate_affinity : affinity) + t * E, k, E, t, expert_idx, gates);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
+                int k, int M, int pool, int mode, int64_t *expert_idx, float *gates, int64_t *group_idx,
+                int force_generic, hipStream_t s) {
+    if (T < 0 || E <= 0 || n_groups <= 0 || k <= 0 || M <= 0 || pool < 1 || pool > 2 || mode < 0 || mode > 3)
+        return TERRACE_EINVAL;
+    if (E % n_groups || k % M || k > E || E > 2048 || M > n_groups) return TERRACE_EINVAL;
+    const int g = E / n_groups;
+    if ((mode == TERRACE_ROUTE_FULL && k / M > g) || (mode == TERRACE_ROUTE_GROUP_LIMITED && k > M * g) ||
+        (mode == TERRACE_ROUTE_QUOTA_ONLY && (k % n_groups || k / n_groups > g)))
+        return TERRACE_EINVAL;
+    if (T == 0) return TERRACE_OK;
+    if (!affinity || !bias || !expert_idx || !gates || !group_idx) return TERRACE_EINVAL;
+    int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 256 * 8) blocks = 256 * 8;
+    int vpl = 1;
+    while (vpl * kWave < E) vpl *= 2;
+    const bool aligned = (((uintptr_t)affinity) & 15) == 0;
+    if (!force_generic && mode == TERRACE_ROUTE_FULL && vpl <= 16 && g % vpl == 0 && is_pow2(g / vpl) &&
+        g / vpl <= kWave && (E != kWave * vpl || aligned)) {
+        const int lpg = g / vpl;
+        const size_t lds = (size_t)kWavesPerBlock * 2 * k * sizeof(int32_t);
+#define TERRACE_ROUTE(V)                                                                                      \
+    route_wave_kernel<V><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, g, k, M, pool, \
+                                                          lpg, expert_idx, gates, group_idx)
+        switch (vpl) {
+            case 1: TERRACE_ROUTE(1); break;
+            case 2: TERRACE_ROUTE(2); break;
+            case 4: TERRACE_ROUTE(4); break;
+            case 8: TERRACE_ROUTE(8); break;
+            default: TERRACE_ROUTE(16); break;
+        }
+#undef TERRACE_ROUTE
+        return check_launch();
+    }
+    const int n_group_out = mode == TERRACE_ROUTE_QUOTA_ONLY ? n_groups : (mode == TERRACE_ROUTE_GLOBAL_TOPK ? k : M);
+    const size_t lds = (size_t)kWavesPerBlock * (E + 2 * n_groups + 2 * k) * sizeof(int32_t);
+    route_generic_kernel<<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, n_groups, k, M, pool,
+                                                          mode, n_group_out, expert_idx, gates, group_idx);
+    return check_launch();
+}
+
+}  // namespace terrace

@@ -1,0 +1,488 @@
+// Row movers: the HBM-bound kernels of the dispatch/combine path.
+//
+//   copy_kernel          y = x                              (streaming-copy roofline probe)
+//   scatter_rows_kernel  dst[pos[r*fan+f]] = src[r]         (Hop-A pack, Hop-B arrival: a source
+//                                                            row is read once and written fan times)
+//   gather_rows_kernel   out[i] = src[idx[i]] or zeros      (expert-order regroup, capacity padding)
+//   combine_kernel       out[i] = sum_j w[i,j]*src[idx[i,j]] in fp32, one rounding at the end
+//
+// A workgroup is 256 threads split into sub-groups of 64/128/256 lanes; a sub-group owns one
+// row at a time, so every index it needs is wave-uniform and each lane keeps several
+// independent 16-byte loads in flight.  Nothing here is a contraction: no MFMA, no LDS.
+#include "common.hpp"
+
+namespace terrace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename V>
+__device__ __forceinline__ V ld_stream(const V *p) { return __builtin_nontemporal_load(p); }
+template <typename V>
+__device__ __forceinline__ void st_stream(V *p, V v) { __builtin_nontemporal_store(v, p); }
+
+template <typename V>
+__device__ __forceinline__ V zero_of() { return V(0); }
+template <>
+__device__ __forceinline__ u32x4 zero_of<u32x4>() { return u32x4{0u, 0u, 0u, 0u}; }
+
+// ---------------------------------------------------------------------------------------------
+// streaming copy
+// ---------------------------------------------------------------------------------------------
+template <typename V, int UNROLL>
+__global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V *__restrict__ y, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock * UNROLL;
+    for (int64_t base = (int64_t)blockIdx.x * kBlock * UNROLL + threadIdx.x; base < n; base += stride) {
+        V v[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t i = base + (int64_t)u * kBlock;
+            if (i < n) v[u] = ld_stream(x + i);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t i = base + (int64_t)u * kBlock;
+            if (i < n) st_stream(y + i, v[u]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// scatter: one read, fan writes
+// ---------------------------------------------------------------------------------------------
+template <typename V, int VPT>
+__global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restrict__ src, V *__restrict__ dst,
+                                                              const int32_t *__restrict__ pos, int64_t n_src,
+                                                              int fan, int64_t row_vecs, int tpr_log2) {
+    const int tpr = 1 << tpr_log2;
+    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
+    const int lane = threadIdx.x & (tpr - 1);
+    const int rows_per_iter = kBlock >> tpr_log2;
+    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_src;
+         row += (int64_t)gridDim.x * rows_per_iter) {
+        const V *s = src + row * row_vecs;
+        const int32_t *p = pos + row * fan;
+        for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
+            V v[VPT];
+#pragma unroll
+            for (int u = 0; u < VPT; ++u) {
+                const int64_t i = base + (int64_t)u * tpr;
+                if (i < row_vecs) v[u] = ld_stream(s + i);
+            }
+            for (int f = 0; f < fan; ++f) {
+                const int64_t d = p[f];
+                if (d < 0) continue;
+                V *o = dst + d * row_vecs;
+#pragma unroll
+                for (int u = 0; u < VPT; ++u) {
+                    const int64_t i = base + (int64_t)u * tpr;
+                    if (i < row_vecs) st_stream(o + i, v[u]);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// gather: out[i] = src[idx[i]], zero row when idx[i] < 0
+// ---------------------------------------------------------------------------------------------
+template <typename V, int VPT, typename I>
+__global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict__ src, V *__restrict__ out,
+                                                             const I *__restrict__ idx, int64_t n_out,
+                                                             int64_t row_vecs, int tpr_log2) {
+    const int tpr = 1 << tpr_log2;
+    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
+    const int lane = threadIdx.x & (tpr - 1);
+    const int rows_per_iter = kBlock >> tpr_log2;
+    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_out;
+         row += (int64_t)gridDim.x * rows_per_iter) {
+        const int64_t from = (int64_t)idx[row];
+        V *o = out + row * row_vecs;
+        if (from < 0) {
+            for (int64_t i = lane; i < row_vecs; i += tpr) st_stream(o + i, zero_of<V>());
+            continue;
+        }
+        const V *s = src + from * row_vecs;
+        for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
+            V v[VPT];
+#pragma unroll
+            for (int u = 0; u < VPT; ++u) {
+                const int64_t i = base + (int64_t)u * tpr;
+                if (i < row_vecs) v[u] = ld_stream(s + i);
+            }
+#pragma unroll
+            for (int u = 0; u < VPT; ++u) {
+                const int64_t i = base + (int64_t)u * tpr;
+                if (i < row_vecs) st_stream(o + i, v[u]);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// combine
+// ---------------------------------------------------------------------------------------------
+// One chunk = 16 bytes of a source row: 4 fp32, 8 bf16/f16 or 16 e4m3 values.
+template <int SRC>
+struct Chunk;
+template <>
+struct Chunk<TERRACE_F32> { static constexpr int N = 4; };
+template <>
+struct Chunk<TERRACE_BF16> { static constexpr int N = 8; };
+template <>
+struct Chunk<TERRACE_F16> { static constexpr int N = 8; };
+template <>
+struct Chunk<TERRACE_FP8_E4M3_B128> { static constexpr int N = 16; };
+
+template <int SRC>
+__device__ __forceinline__ void decode_chunk(u32x4 raw, float *f) {
+    if constexpr (SRC == TERRACE_F32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(raw[i]);
+    } else if constexpr (SRC == TERRACE_BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(raw[i] << 16);
+            f[2 * i + 1] = __uint_as_float(raw[i] & 0xFFFF0000u);
+        }
+    } else if constexpr (SRC == TERRACE_F16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __half2float(__ushort_as_half((unsigned short)(raw[i] & 0xFFFFu)));
+            f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(raw[i] >> 16)));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) f[4 * i + b] = e4m3_to_f32((raw[i] >> (8 * b)) & 0xFFu);
+        }
+    }
+}
+
+__device__ __forceinline__ float load_weight(const void *w, int w_dtype, int64_t i) {
+    if (w_dtype == TERRACE_F32) return ((const float *)w)[i];
+    const uint32_t b = ((const uint16_t *)w)[i];
+    if (w_dtype == TERRACE_BF16) return bf16_bits_to_f32(b);
+    return __half2float(__ushort_as_half((unsigned short)b));
+}
+
+template <int OUT, int N>
+__device__ __forceinline__ void store_chunk(void *out_row, int64_t first_elem, const float *acc) {
+    if constexpr (OUT == TERRACE_F32) {
+        u32x4 *o = (u32x4 *)((float *)out_row + first_elem);
+#pragma unroll
+        for (int v = 0; v < N / 4; ++v) {
+            u32x4 t;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[i] = __float_as_uint(acc[4 * v + i]);
+            st_stream(o + v, t);
+        }
+    } else {
+        uint32_t packed[N / 2];
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            uint32_t lo, hi;
+            if constexpr (OUT == TERRACE_BF16) {
+                lo = f32_to_bf16_bits(acc[2 * i]);
+                hi = f32_to_bf16_bits(acc[2 * i + 1]);
+            } else {
+                lo = __half_as_ushort(__float2half_rn(acc[2 * i]));
+                hi = __half_as_ushort(__float2half_rn(acc[2 * i + 1]));
+            }
+            packed[i] = (lo & 0xFFFFu) | (hi << 16);
+        }
+        uint16_t *o16 = (uint16_t *)out_row + first_elem;
+        if constexpr (N == 4) {
+            st_stream((u32x2 *)o16, u32x2{packed[0], packed[1]});
+        } else {
+#pragma unroll
+            for (int v = 0; v < N / 8; ++v)
+                st_stream((u32x4 *)o16 + v, u32x4{packed[4 * v], packed[4 * v + 1], packed[4 * v + 2], packed[4 * v + 3]});
+        }
+    }
+}
+
+// Vector path: rows are 16-byte aligned multiples of 16 bytes.
+template <int SRC, int OUT, int FANC>
+__global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restrict__ src, int64_t src_row_bytes,
+                                                         const int64_t *__restrict__ idx, const void *__restrict__ w,
+                                                         int w_dtype, int64_t n_out, int fan, int64_t hidden,
+                                                         uint8_t *__restrict__ out, int64_t out_row_bytes,
+                                                         int tpr_log2) {
+    constexpr int N = Chunk<SRC>::N;
+    const int tpr = 1 << tpr_log2;
+    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
+    const int lane = threadIdx.x & (tpr - 1);
+    const int rows_per_iter = kBlock >> tpr_log2;
+    const int64_t chunks = hidden / N;
+    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_out;
+         row += (int64_t)gridDim.x * rows_per_iter) {
+        uint8_t *out_row = out + row * out_row_bytes;
+        for (int64_t c = lane; c < chunks; c += tpr) {
+            float acc[N];
+#pragma unroll
+            for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+            for (int j0 = 0; j0 < fan; j0 += FANC) {
+                u32x4 raw[FANC];
+                float wj[FANC], sc[FANC];
+                bool live[FANC];
+#pragma unroll
+                for (int jj = 0; jj < FANC; ++jj) {
+                    const int j = j0 + jj;
+                    live[jj] = false;
+                    wj[jj] = 1.0f;
+                    sc[jj] = 1.0f;
+                    if (j < fan) {
+                        const int64_t from = idx[row * fan + j];
+                        if (from >= 0) {
+                            live[jj] = true;
+                            const uint8_t *s = src + from * src_row_bytes;
+                            raw[jj] = ld_stream((const u32x4 *)s + c);
+                            if constexpr (SRC == TERRACE_FP8_E4M3_B128)
+                                sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
+                            if (w) wj[jj] = load_weight(w, w_dtype, row * fan + j);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int jj = 0; jj < FANC; ++jj) {
+                    if (!live[jj]) continue;
+                    float f[N];
+                    decode_chunk<SRC>(raw[jj], f);
+#pragma unroll
+                    for (int i = 0; i < N; ++i) {
+                        float x = f[i];
+                        if constexpr (SRC == TERRACE_FP8_E4M3_B128) x = __fmul_rn(x, sc[jj]);
+                        if (w) x = __fmul_rn(x, wj[jj]);
+                        acc[i] = __fadd_rn(acc[i], x);
+                    }
+                }
+            }
+            store_chunk<OUT, N>(out_row, c * N, acc);
+        }
+    }
+}
+
+// Element path: any hidden, any alignment.
+__device__ __forceinline__ float load_elem(const uint8_t *row, int src_dtype, int64_t e, int64_t hidden) {
+    switch (src_dtype) {
+        case TERRACE_F32: return ((const float *)row)[e];
+        case TERRACE_BF16: return bf16_bits_to_f32(((const uint16_t *)row)[e]);
+        case TERRACE_F16: return __half2float(__ushort_as_half(((const uint16_t *)row)[e]));
+        default: {
+            float sc;
+            const uint8_t *sp = row + hidden + 4 * (e / 128);
+            uint32_t bits = sp[0] | (sp[1] << 8) | (sp[2] << 16) | ((uint32_t)sp[3] << 24);
+            sc = __uint_as_float(bits);
+            return __fmul_rn(e4m3_to_f32(row[e]), sc);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void combine_elem_kernel(const uint8_t *__restrict__ src, int src_dtype,
+                                                              int64_t src_row_bytes, const int64_t *__restrict__ idx,
+                                                              const void *__restrict__ w, int w_dtype, int64_t n_out,
+                                                              int fan, int64_t hidden, uint8_t *__restrict__ out,
+                                                              int out_dtype) {
+    for (int64_t row = blockIdx.x; row < n_out; row += gridDim.x) {
+        for (int64_t e = threadIdx.x; e < hidden; e += kBlock) {
+            float acc = 0.0f;
+            for (int j = 0; j < fan; ++j) {
+                const int64_t from = idx[row * fan + j];
+                if (from < 0) continue;
+                float x = load_elem(src + from * src_row_bytes, src_dtype, e, hidden);
+                if (w) x = __fmul_rn(x, load_weight(w, w_dtype, row * fan + j));
+                acc = __fadd_rn(acc, x);
+            }
+            if (out_dtype == TERRACE_F32) ((float *)out)[row * hidden + e] = acc;
+            else if (out_dtype == TERRACE_BF16) ((uint16_t *)out)[row * hidden + e] = (uint16_t)f32_to_bf16_bits(acc);
+            else ((uint16_t *)out)[row * hidden + e] = __half_as_ushort(__float2half_rn(acc));
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void index_chain_kernel(const int64_t *__restrict__ table,
+                                                             const int64_t *__restrict__ idx, int64_t n,
+                                                             int64_t *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t a = idx[i];
+    out[i] = a < 0 ? -1 : table[a];
+}
+
+__global__ void send_splits_kernel(const int64_t *__restrict__ node_counts, int world, int rpn, int my_local,
+                                   int64_t *__restrict__ send) {
+    for (int i = threadIdx.x; i < world; i += blockDim.x)
+        send[i] = (i % rpn == my_local) ? node_counts[i / rpn] : 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// host-side launch helpers
+// ---------------------------------------------------------------------------------------------
+static int grid_for(int64_t n_rows, int rows_per_iter) {
+    const int64_t need = (n_rows + rows_per_iter - 1) / rows_per_iter;
+    const int64_t cap = 256 * 16;               // 256 CUs, up to 16 resident workgroups' worth of rows each
+    return (int)(need < 1 ? 1 : (need > cap ? cap : need));
+}
+
+// Lanes per row: enough that a lane holds about 4 vectors, at least one wave, at most the block.
+static int tpr_log2_for(int64_t row_vecs) {
+    int l = 6;
+    while (l < 8 && ((int64_t)4 << l) < row_vecs) ++l;
+    return l;
+}
+
+static int vec_bytes_for(int64_t row_bytes, const void *a, const void *b) {
+    const uintptr_t bits = (uintptr_t)row_bytes | (uintptr_t)a | (uintptr_t)b;
+    if ((bits & 15) == 0) return 16;
+    if ((bits & 7) == 0) return 8;
+    if ((bits & 3) == 0) return 4;
+    if ((bits & 1) == 0) return 2;
+    return 1;
+}
+
+template <typename V>
+static void launch_scatter_t(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan,
+                             int64_t row_vecs, hipStream_t s) {
+    const int l = tpr_log2_for(row_vecs);
+    const int rpi = kBlock >> l;
+    const int grid = grid_for(n_src, rpi);
+    if (row_vecs > ((int64_t)2 << l))
+        scatter_rows_kernel<V, 4><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+    else if (row_vecs > ((int64_t)1 << l))
+        scatter_rows_kernel<V, 2><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+    else
+        scatter_rows_kernel<V, 1><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+}
+
+int launch_scatter_rows(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan, int64_t row_bytes,
+                        hipStream_t s) {
+    if (n_src <= 0 || row_bytes <= 0 || fan <= 0) return TERRACE_OK;
+    switch (vec_bytes_for(row_bytes, src, dst)) {
+        case 16: launch_scatter_t<u32x4>(src, dst, pos, n_src, fan, row_bytes / 16, s); break;
+        case 8: launch_scatter_t<u32x2>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
+        case 4: launch_scatter_t<uint32_t>(src, dst, pos, n_src, fan, row_bytes / 4, s); break;
+        case 2: launch_scatter_t<uint16_t>(src, dst, pos, n_src, fan, row_bytes / 2, s); break;
+        default: launch_scatter_t<uint8_t>(src, dst, pos, n_src, fan, row_bytes, s); break;
+    }
+    return check_launch();
+}
+
+template <typename V, typename I>
+static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_vecs,
+                            hipStream_t s) {
+    const int l = tpr_log2_for(row_vecs);
+    const int rpi = kBlock >> l;
+    const int grid = grid_for(n_out, rpi);
+    if (row_vecs > ((int64_t)2 << l))
+        gather_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+    else if (row_vecs > ((int64_t)1 << l))
+        gather_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+    else
+        gather_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+}
+
+template <typename I>
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s) {
+    if (n_out <= 0 || row_bytes <= 0) return TERRACE_OK;
+    switch (vec_bytes_for(row_bytes, src, out)) {
+        case 16: launch_gather_t<u32x4, I>(src, out, idx, n_out, row_bytes / 16, s); break;
+        case 8: launch_gather_t<u32x2, I>(src, out, idx, n_out, row_bytes / 8, s); break;
+        case 4: launch_gather_t<uint32_t, I>(src, out, idx, n_out, row_bytes / 4, s); break;
+        case 2: launch_gather_t<uint16_t, I>(src, out, idx, n_out, row_bytes / 2, s); break;
+        default: launch_gather_t<uint8_t, I>(src, out, idx, n_out, row_bytes, s); break;
+    }
+    return check_launch();
+}
+template int launch_gather_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int64_t, hipStream_t);
+template int launch_gather_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int64_t, hipStream_t);
+
+static int64_t dtype_row_bytes(int dtype, int64_t hidden) {
+    switch (dtype) {
+        case TERRACE_F32: return hidden * 4;
+        case TERRACE_BF16:
+        case TERRACE_F16: return hidden * 2;
+        case TERRACE_FP8_E4M3_B128: return hidden + 4 * (hidden / 128);
+        default: return -1;
+    }
+}
+
+template <int SRC, int OUT>
+static void launch_combine_so(const void *src, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
+                              int fan, int64_t hidden, void *out, hipStream_t s) {
+    const int64_t chunks = hidden / Chunk<SRC>::N;
+    int l = 6;
+    while (l < 8 && ((int64_t)2 << l) < chunks) ++l;
+    const int rpi = kBlock >> l;
+    const int grid = grid_for(n_out, rpi);
+    const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
+#define TERRACE_COMBINE_LAUNCH(F)                                                                          \
+    combine_kernel<SRC, OUT, F><<<grid, kBlock, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, \
+                                                        fan, hidden, (uint8_t *)out, orb, l)
+    if (fan >= 8) TERRACE_COMBINE_LAUNCH(8);
+    else if (fan >= 4) TERRACE_COMBINE_LAUNCH(4);
+    else if (fan >= 2) TERRACE_COMBINE_LAUNCH(2);
+    else TERRACE_COMBINE_LAUNCH(1);
+#undef TERRACE_COMBINE_LAUNCH
+}
+
+template <int SRC>
+static void launch_combine_s(const void *src, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
+                             int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
+    if (out_dtype == TERRACE_F32) launch_combine_so<SRC, TERRACE_F32>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+    else if (out_dtype == TERRACE_BF16) launch_combine_so<SRC, TERRACE_BF16>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+    else launch_combine_so<SRC, TERRACE_F16>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+}
+
+int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
+                   int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
+    if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
+    const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
+    const int n = src_dtype == TERRACE_F32 ? 4 : (src_dtype == TERRACE_FP8_E4M3_B128 ? 16 : 8);
+    const bool vec = hidden % n == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
+                     srb % 16 == 0 && orb % 16 == 0;
+    if (!vec) {
+        const int grid = (int)(n_out > 4096 ? 4096 : n_out);
+        combine_elem_kernel<<<grid, kBlock, 0, s>>>((const uint8_t *)src, src_dtype, srb, idx, w, w_dtype, n_out, fan,
+                                                    hidden, (uint8_t *)out, out_dtype);
+        return check_launch();
+    }
+    switch (src_dtype) {
+        case TERRACE_F32: launch_combine_s<TERRACE_F32>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_BF16: launch_combine_s<TERRACE_BF16>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_F16: launch_combine_s<TERRACE_F16>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+    }
+    return check_launch();
+}
+
+int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s) {
+    if (nbytes == 0) return TERRACE_OK;
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)y | (uintptr_t)nbytes;
+    if ((bits & 15) == 0) {
+        const int64_t n = (int64_t)(nbytes / 16);
+        int64_t blocks = (n + kBlock * 4 - 1) / (kBlock * 4);
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        copy_kernel<u32x4, 4><<<(int)blocks, kBlock, 0, s>>>((const u32x4 *)x, (u32x4 *)y, n);
+    } else {
+        const int64_t n = (int64_t)nbytes;
+        int64_t blocks = (n + kBlock * 4 - 1) / (kBlock * 4);
+        if (blocks > 256 * 16) blocks = 256 * 16;
+        copy_kernel<uint8_t, 4><<<(int)blocks, kBlock, 0, s>>>((const uint8_t *)x, (uint8_t *)y, n);
+    }
+    return check_launch();
+}
+
+int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s) {
+    if (n <= 0) return TERRACE_OK;
+    index_chain_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(table, idx, n, out);
+    return check_launch();
+}
+
+int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s) {
+    send_splits_kernel<<<1, 256, 0, s>>>(node_counts, world, rpn, my_local, send);
+    return check_launch();
+}
+
+}  // namespace terrace

@@ -1,0 +1,727 @@
+// Index build: stable counting sorts over small key ranges, without atomics.
+//
+// All three index stages of the path are the same object -- "put items in stable ascending
+// order of a key with few distinct values":
+//   send side   item = (token, run)   key = destination node      (plan + Hop-A wire planes)
+//   arrival     item = (row, slot i)  key = owner card            (Hop-B arrival chain)
+//   expert card item = received row   key = local expert          (expert-order regroup)
+// Unordered atomic cursors cannot give a stable order, so placement is
+//   dest = start[key] + (items with that key in earlier units) + (rank inside the unit),
+// built in three launches:
+//   count  each wave owns a contiguous "unit" of items and histograms it in wave-private LDS;
+//   scan   one workgroup turns the [unit][bucket] counts into exclusive cursors (bucket-major);
+//   rank   each wave replays its unit, ranks items with wave ballots, and emits the outputs.
+// The row payload itself is moved afterwards by the scatter/gather kernels of rows.hip.
+#include "common.hpp"
+
+namespace terrace {
+
+constexpr int kMaxBuckets = 2048;
+constexpr int kScanThreads = 1024;
+
+struct Units {
+    int64_t n_items;
+    int chunks;       // 64-item chunks per unit
+    int n_units;
+    int n_buckets;
+};
+
+Units make_units(int64_t n_items, int n_buckets) {
+    Units u;
+    u.n_items = n_items;
+    u.n_buckets = n_buckets;
+    int64_t ch = 4;
+    while ((n_items + 64 * ch - 1) / (64 * ch) > 4096) ch *= 2;
+    u.chunks = (int)ch;
+    u.n_units = (int)((n_items + 64 * ch - 1) / (64 * ch));
+    if (u.n_units < 1) u.n_units = 1;
+    return u;
+}
+
+size_t units_table_bytes(const Units &u) {
+    return align_up(((size_t)u.n_units * u.n_buckets + u.n_buckets + 1) * sizeof(int32_t), 256);
+}
+
+// ---------------------------------------------------------------------------------------------
+// key functors: return the bucket of an item, clamped into range; *bad is set for ids outside it
+// ---------------------------------------------------------------------------------------------
+struct KeyAffine {           // bucket = (plane[item] - sub) / div
+    const int64_t *plane;
+    int64_t sub;
+    int div;
+    int n_buckets;
+    __device__ __forceinline__ int operator()(int64_t item, bool *bad) const {
+        const int64_t v = plane[item] - sub;
+        if (v < 0 || v >= (int64_t)n_buckets * div) {
+            *bad = true;
+            return 0;
+        }
+        return (int)((uint32_t)v / (uint32_t)div);
+    }
+};
+
+// A token's k expert ids, in registers when k <= KMAX (KMAX > 0), else re-read through L1.
+template <int KMAX>
+struct RowIds {
+    int v[KMAX > 0 ? KMAX : 1];
+    const int64_t *row;
+    int k;
+    __device__ __forceinline__ void load(const int64_t *r, int k_) {
+        row = r;
+        k = k_;
+        if constexpr (KMAX > 0) {
+#pragma unroll
+            for (int j = 0; j < KMAX; ++j) v[j] = j < k ? (int)r[j] : 0x7FFFFFFF;
+        }
+    }
+    __device__ __forceinline__ int at(int j) const {
+        if constexpr (KMAX > 0) return v[j];
+        else return (int)row[j];
+    }
+    __device__ __forceinline__ int bound() const { return KMAX > 0 ? KMAX : k; }
+};
+
+template <int KMAX>
+__device__ __forceinline__ int rank_in_row(const RowIds<KMAX> &ids, int j) {
+    const int e = ids.at(j);
+    int r = 0;
+    if constexpr (KMAX > 0) {
+#pragma unroll
+        for (int i = 0; i < KMAX; ++i) r += (ids.v[i] < e) ? 1 : 0;
+    } else {
+        for (int i = 0; i < ids.k; ++i) r += (ids.at(i) < e) ? 1 : 0;
+    }
+    return r;
+}
+
+// Expert id of the element whose ascending rank inside the row is `want` (-1 if none: duplicates).
+template <int KMAX>
+__device__ __forceinline__ int id_with_rank(const RowIds<KMAX> &ids, int want) {
+    int found = -1;
+    if constexpr (KMAX > 0) {
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j)
+            if (j < ids.k && rank_in_row(ids, j) == want) found = ids.v[j];
+    } else {
+        for (int j = 0; j < ids.k; ++j)
+            if (rank_in_row(ids, j) == want) found = ids.at(j);
+    }
+    return found;
+}
+
+template <int KMAX>
+struct KeyRun {              // item = t*M + m  ->  node of the m-th run of token t's ascending row
+    const int64_t *expert_idx;
+    int k, groups_m, quota, slots, n_nodes;
+    __device__ __forceinline__ int operator()(int64_t item, bool *bad) const {
+        const int64_t t = item / groups_m;
+        const int m = (int)(item - t * groups_m);
+        RowIds<KMAX> ids;
+        ids.load(expert_idx + t * k, k);
+        const int e = id_with_rank(ids, m * quota);
+        if (e < 0 || e / slots >= n_nodes) {
+            *bad = true;
+            return 0;
+        }
+        return e / slots;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// count
+// ---------------------------------------------------------------------------------------------
+template <typename KeyFn>
+__global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, int32_t *__restrict__ table) {
+    extern __shared__ int32_t lds[];
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    volatile int32_t *hist = lds + w * u.n_buckets;
+    const int unit = blockIdx.x * kWavesPerBlock + w;
+    if (unit >= u.n_units) return;
+    for (int b = lane; b < u.n_buckets; b += kWave) hist[b] = 0;
+    __builtin_amdgcn_wave_barrier();
+    const int64_t first = (int64_t)unit * u.chunks * kWave;
+    for (int c = 0; c < u.chunks; ++c) {
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        const bool valid = item < u.n_items;
+        bool bad = false;
+        const int key = valid ? key_of(item, &bad) : 0;
+        uint64_t todo = __ballot(valid);
+        while (todo) {
+            const int leader = __builtin_ctzll(todo);
+            const int kk = read_lane(key, leader);
+            const uint64_t peers = __ballot(valid && key == kk);
+            if (lane == leader) hist[kk] = hist[kk] + __popcll(peers);
+            todo &= ~peers;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)unit * u.n_buckets + b] = hist[b];
+}
+
+// ---------------------------------------------------------------------------------------------
+// scan: table[unit][bucket] counts -> exclusive cursors in (bucket, unit) order, in place.
+// Also start[b] (int32, n_buckets+1 entries after the table), the caller's histogram and
+// offsets planes, and a zeroed status block.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table,
+                                                            int64_t *__restrict__ hist_i64,
+                                                            float *__restrict__ hist_f32,
+                                                            int64_t *__restrict__ offsets_i64,
+                                                            int32_t *__restrict__ status, int divide_by) {
+    __shared__ int32_t wave_tot[kScanThreads / kWave];
+    __shared__ int32_t grand_total;
+    int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
+    const int tid = threadIdx.x;
+    const int64_t n = (int64_t)u.n_units * u.n_buckets;
+    const int64_t per = (n + kScanThreads - 1) / kScanThreads;
+    const int64_t lo = tid * per, hi = lo + per < n ? lo + per : n;
+    if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
+    int32_t sum = 0;
+    for (int64_t i = lo; i < hi; ++i) {
+        const int64_t b = i / u.n_units, un = i - b * u.n_units;
+        sum += table[un * u.n_buckets + b];
+    }
+    int32_t incl = wave_inclusive_scan(sum);
+    if (lane_id() == kWave - 1) wave_tot[tid >> 6] = incl;
+    __syncthreads();
+    if (tid < kWave) {
+        int32_t t = tid < kScanThreads / kWave ? wave_tot[tid] : 0;
+        int32_t ti = wave_inclusive_scan(t);
+        if (tid < kScanThreads / kWave) wave_tot[tid] = ti - t;
+        if (tid == kScanThreads / kWave - 1) grand_total = ti;
+    }
+    __syncthreads();
+    int32_t run = wave_tot[tid >> 6] + incl - sum;
+    for (int64_t i = lo; i < hi; ++i) {
+        const int64_t b = i / u.n_units, un = i - b * u.n_units;
+        const int32_t c = table[un * u.n_buckets + b];
+        table[un * u.n_buckets + b] = run;
+        if (un == 0) start[b] = run;
+        run += c;
+    }
+    if (tid == 0) start[u.n_buckets] = grand_total;
+    __syncthreads();
+    for (int b = tid; b < u.n_buckets; b += kScanThreads) {
+        const int32_t s0 = start[b], s1 = start[b + 1];
+        const int32_t cnt = (s1 - s0) / divide_by;
+        if (hist_i64) hist_i64[b] = cnt;
+        if (hist_f32) hist_f32[b] = (float)cnt;
+        if (offsets_i64) offsets_i64[b] = s0 / divide_by;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// rank
+// ---------------------------------------------------------------------------------------------
+template <typename KeyFn, typename EmitFn>
+__global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit, Units u,
+                                                      const int32_t *__restrict__ table,
+                                                      int32_t *__restrict__ status) {
+    extern __shared__ int32_t lds[];
+    const int lane = lane_id();
+    const int w = wave_in_block();
+    volatile int32_t *cursor = lds + w * u.n_buckets;
+    const int unit = blockIdx.x * kWavesPerBlock + w;
+    if (unit >= u.n_units) return;
+    for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)unit * u.n_buckets + b];
+    __builtin_amdgcn_wave_barrier();
+    const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
+    const int64_t first = (int64_t)unit * u.chunks * kWave;
+    int fault = 0;
+    int tally[2] = {0, 0};
+    for (int c = 0; c < u.chunks; ++c) {
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        const bool valid = item < u.n_items;
+        bool bad = false;
+        const int key = valid ? key_of(item, &bad) : 0;
+        if (bad) fault |= TERRACE_FAULT_ID_RANGE;
+        int32_t dest = 0;
+        uint64_t todo = __ballot(valid);
+        while (todo) {
+            const int leader = __builtin_ctzll(todo);
+            const int kk = read_lane(key, leader);
+            const uint64_t peers = __ballot(valid && key == kk);
+            const int32_t base = cursor[kk];
+            if (valid && key == kk) dest = base + __popcll(peers & lanes_below(lane));
+            __builtin_amdgcn_wave_barrier();
+            if (lane == leader) cursor[kk] = base + __popcll(peers);
+            todo &= ~peers;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (valid) fault |= emit(item, key, dest, start, tally);
+    }
+    if (!status) return;
+    if (fault) atomicOr(&status[0], fault);
+    if (EmitFn::kTallies) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            int v = tally[i];
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) v += __shfl_xor(v, d, kWave);
+            if (lane == 0 && v) atomicAdd(&status[1 + i], v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// emit functors
+// ---------------------------------------------------------------------------------------------
+struct EmitOrder {           // plain stable argsort: order[dest] = item
+    int64_t *order;
+    static constexpr bool kTallies = false;
+    __device__ __forceinline__ int operator()(int64_t item, int, int32_t dest, const int32_t *, int *) const {
+        order[dest] = item;
+        return 0;
+    }
+};
+
+struct EmitNothing {
+    static constexpr bool kTallies = false;
+    __device__ __forceinline__ int operator()(int64_t, int, int32_t, const int32_t *, int *) const { return 0; }
+};
+
+struct EmitArrival {         // terrace/ops/__init__.py:287-299
+    const int64_t *rslot;
+    const void *rgate;
+    int gate_bytes, quota;
+    void *gate_pairs;
+    int64_t *r_idx, *slot_idx, *pair_pos;
+    int32_t *pos32;
+    static constexpr bool kTallies = false;
+    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, const int32_t *, int *) const {
+        r_idx[dest] = p / quota;
+        slot_idx[dest] = rslot[p];
+        if (rgate) {
+            if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = ((const uint32_t *)rgate)[p];
+            else ((uint16_t *)gate_pairs)[dest] = ((const uint16_t *)rgate)[p];
+        }
+        pos32[p] = dest;
+        if (pair_pos) pair_pos[p] = dest;
+        return 0;
+    }
+};
+
+struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
+    int64_t capacity;        // < 0: drop-less
+    int64_t *order, *dest_out;
+    uint8_t *kept;
+    int32_t *order32;
+    static constexpr bool kTallies = false;
+    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, const int32_t *start, int *) const {
+        order32[dest] = (int32_t)p;
+        if (order) order[dest] = p;
+        if (capacity >= 0) {
+            const int64_t rank = dest - start[key];
+            const bool keep = rank < capacity;
+            if (dest_out) dest_out[p] = keep ? key * capacity + rank : -1;
+            if (kept) kept[p] = keep ? 1 : 0;
+        } else {
+            if (dest_out) dest_out[p] = dest;
+            if (kept) kept[p] = 1;
+        }
+        return 0;
+    }
+};
+
+template <int KMAX>
+struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:236-248
+    const int64_t *expert_idx;
+    const void *gates;
+    int gate_bytes, k, groups_m, quota, slots, n_experts;
+    int64_t *mask, *u_src, *u_node, *inverse, *pair_table, *sort_order, *token_rows;
+    void *gate_rows, *gate_sorted;
+    int32_t *pos32;
+    // status word 1 receives the number of occupied (token, node) pairs, word 2 the number of
+    // those holding other than k/M experts: the two quantities terrace/ta2a.py:170-204 checks.
+    static constexpr bool kTallies = true;
+    __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, const int32_t *,
+                                              int *tally) const {
+        const int64_t t = item / groups_m;
+        const int m = (int)(item - t * groups_m);
+        RowIds<KMAX> ids;
+        ids.load(expert_idx + t * k, k);
+        int fault = 0;
+        if (m == 0) {
+            int occupied = 0, off_quota = 0;
+            auto census = [&](int j) {
+                const int nj = ids.at(j) / slots;
+                int same = 0, earlier = 0;
+                auto cmp = [&](int i) {
+                    const bool hit = (ids.at(i) / slots) == nj;
+                    same += hit ? 1 : 0;
+                    earlier += (hit && i < j) ? 1 : 0;
+                };
+                if constexpr (KMAX > 0) {
+#pragma unroll
+                    for (int i = 0; i < KMAX; ++i)
+                        if (i < k) cmp(i);
+                } else {
+                    for (int i = 0; i < k; ++i) cmp(i);
+                }
+                if (earlier == 0) {
+                    occupied += 1;
+                    off_quota += same != quota ? 1 : 0;
+                }
+            };
+            if constexpr (KMAX > 0) {
+#pragma unroll
+                for (int j = 0; j < KMAX; ++j)
+                    if (j < k) census(j);
+            } else {
+                for (int j = 0; j < k; ++j) census(j);
+            }
+            tally[0] += occupied;
+            tally[1] += off_quota;
+            if (occupied != groups_m) fault |= TERRACE_FAULT_FANOUT;
+            if (off_quota) fault |= TERRACE_FAULT_QUOTA;
+        }
+        u_src[row] = t;
+        if (u_node) u_node[row] = node;
+        if (token_rows) token_rows[item] = row;
+        pos32[item] = row;
+        auto body = [&](int j) {
+            const int e = ids.at(j);
+            if (e < 0 || e >= n_experts) fault |= TERRACE_FAULT_ID_RANGE;
+            const int r = rank_in_row(ids, j);
+            if (r / quota != m) return;
+            const int i = r - m * quota;
+            const int64_t cell = (int64_t)row * quota + i;
+            mask[cell] = e >= 0 ? e % slots : 0;
+            if (gates) {
+                if (gate_bytes == 4) {
+                    const uint32_t gv = ((const uint32_t *)gates)[t * k + j];
+                    ((uint32_t *)gate_rows)[cell] = gv;
+                    if (gate_sorted) ((uint32_t *)gate_sorted)[t * k + r] = gv;
+                } else {
+                    const uint16_t gv = ((const uint16_t *)gates)[t * k + j];
+                    ((uint16_t *)gate_rows)[cell] = gv;
+                    if (gate_sorted) ((uint16_t *)gate_sorted)[t * k + r] = gv;
+                }
+            }
+            if (inverse) inverse[t * k + j] = row;
+            if (pair_table) pair_table[t * k + r] = cell;
+            if (sort_order) sort_order[t * k + r] = j;
+        };
+        if constexpr (KMAX > 0) {
+#pragma unroll
+            for (int j = 0; j < KMAX; ++j)
+                if (j < k) body(j);
+        } else {
+            for (int j = 0; j < k; ++j) body(j);
+        }
+        return fault;
+    }
+};
+
+// Per-place source row for the capacity layout: gidx[x*C + r] = order[start[x] + r] or -1
+// (places = epr*C; with places = 0 only kept_per_expert = min(count, capacity) is written).
+__global__ __launch_bounds__(kBlock) void capacity_index_kernel(const int32_t *__restrict__ order32,
+                                                                const int32_t *__restrict__ start, int epr,
+                                                                int64_t capacity, int64_t places,
+                                                                int32_t *__restrict__ gidx,
+                                                                int64_t *__restrict__ kept_per_expert) {
+    const int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (d < epr && kept_per_expert) {
+        const int64_t c = start[d + 1] - start[d];
+        kept_per_expert[d] = c < capacity ? c : capacity;
+    }
+    if (d >= places) return;
+    const int x = (int)(d / capacity);
+    const int64_t r = d - x * capacity;
+    const int64_t c = start[x + 1] - start[x];
+    gidx[d] = r < c ? order32[start[x] + r] : -1;
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(uint8_t *__restrict__ p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gather_elems_kernel(const T *__restrict__ src,
+                                                              const int32_t *__restrict__ idx, int64_t n,
+                                                              T *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int32_t a = idx[i];
+    out[i] = a < 0 ? T(0) : src[a];
+}
+
+__global__ void empty_outputs_kernel(int64_t *hist, float *hist_f, int64_t *offsets, int n, int32_t *status) {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        if (hist) hist[i] = 0;
+        if (hist_f) hist_f[i] = 0.0f;
+        if (offsets) offsets[i] = 0;
+    }
+    if (status && threadIdx.x < TERRACE_STATUS_WORDS) status[threadIdx.x] = 0;
+}
+
+// _pack_quota_wire for a caller-provided inverse: one lane per token.
+template <int KMAX>
+__global__ __launch_bounds__(kBlock) void pack_quota_wire_kernel(const int64_t *__restrict__ expert_idx,
+                                                                 const void *__restrict__ gates,
+                                                                 const int64_t *__restrict__ inverse, int64_t T, int k,
+                                                                 int gate_bytes, int64_t n_rows, int slots, int quota,
+                                                                 int64_t *__restrict__ slot_tab,
+                                                                 void *__restrict__ gate_tab,
+                                                                 int32_t *__restrict__ status) {
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= T) return;
+    RowIds<KMAX> ids;
+    ids.load(expert_idx + t * k, k);
+    bool bad = false;
+    auto body = [&](int j) {
+        const int e = ids.at(j);
+        const int r = rank_in_row(ids, j);
+        const int m = r / quota, i = r - m * quota;
+        // the run's row is the one `inverse` names for its first (smallest) expert
+        int64_t row = -1;
+        auto find = [&](int jj) {
+            if (rank_in_row(ids, jj) == m * quota) row = inverse[t * k + jj];
+        };
+        if constexpr (KMAX > 0) {
+#pragma unroll
+            for (int jj = 0; jj < KMAX; ++jj)
+                if (jj < k) find(jj);
+        } else {
+            for (int jj = 0; jj < k; ++jj) find(jj);
+        }
+        if (row < 0 || row >= n_rows) {
+            bad = true;
+            return;
+        }
+        const int64_t cell = row * quota + i;
+        slot_tab[cell] = ((e % slots) + slots) % slots;
+        if (gates) {
+            if (gate_bytes == 4) ((uint32_t *)gate_tab)[cell] = ((const uint32_t *)gates)[t * k + j];
+            else ((uint16_t *)gate_tab)[cell] = ((const uint16_t *)gates)[t * k + j];
+        }
+    };
+    if constexpr (KMAX > 0) {
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j)
+            if (j < k) body(j);
+    } else {
+        for (int j = 0; j < k; ++j) body(j);
+    }
+    if (bad && status) atomicOr(&status[0], TERRACE_FAULT_ID_RANGE);
+}
+
+// ---------------------------------------------------------------------------------------------
+// host drivers
+// ---------------------------------------------------------------------------------------------
+int launch_scatter_rows(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan, int64_t row_bytes,
+                        hipStream_t s);
+template <typename I>
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
+
+static int blocks_for_units(const Units &u) { return (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock; }
+static size_t lds_for(const Units &u) { return (size_t)kWavesPerBlock * u.n_buckets * sizeof(int32_t); }
+
+template <typename KeyFn, typename EmitFn>
+static int run_sort(const KeyFn &key, const EmitFn &emit, const Units &u, int32_t *table, int64_t *hist,
+                    float *hist_f, int64_t *offsets, int32_t *status, int divide_by, bool do_rank, hipStream_t s) {
+    count_kernel<KeyFn><<<blocks_for_units(u), kBlock, lds_for(u), s>>>(key, u, table);
+    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist, hist_f, offsets, status, divide_by);
+    if (do_rank) rank_kernel<KeyFn, EmitFn><<<blocks_for_units(u), kBlock, lds_for(u), s>>>(key, emit, u, table, status);
+    return check_launch();
+}
+
+static int empty_outputs(int64_t *hist, float *hist_f, int64_t *offsets, int n, int32_t *status, hipStream_t s) {
+    empty_outputs_kernel<<<1, 256, 0, s>>>(hist, hist_f, offsets, n, status);
+    return check_launch();
+}
+
+// ---- histogram / argsort --------------------------------------------------------------------
+size_t hist_workspace(int64_t n, int n_buckets) {
+    if (n <= 0 || n_buckets <= 0 || n_buckets > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(n, n_buckets));
+}
+
+int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status, void *ws,
+             size_t ws_bytes, hipStream_t s) {
+    if (n_buckets <= 0 || n_buckets > kMaxBuckets || n < 0 || !out) return TERRACE_EINVAL;
+    int64_t *h = as_float ? nullptr : (int64_t *)out;
+    float *hf = as_float ? (float *)out : nullptr;
+    if (n == 0) return empty_outputs(h, hf, nullptr, n_buckets, status, s);
+    if (!idx || !ws) return TERRACE_EINVAL;
+    const Units u = make_units(n, n_buckets);
+    if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
+    KeyAffine key{idx, 0, 1, n_buckets};
+    // the rank pass runs only to report out-of-range ids
+    return run_sort(key, EmitNothing{}, u, (int32_t *)ws, h, hf, nullptr, status, 1, status != nullptr, s);
+}
+
+int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *order, int64_t *hist, int32_t *status,
+                      void *ws, size_t ws_bytes, hipStream_t s) {
+    if (n_buckets <= 0 || n_buckets > kMaxBuckets || n < 0) return TERRACE_EINVAL;
+    if (n == 0) return empty_outputs(hist, nullptr, nullptr, hist ? n_buckets : 0, status, s);
+    if (!keyp || !order || !ws) return TERRACE_EINVAL;
+    const Units u = make_units(n, n_buckets);
+    if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
+    KeyAffine key{keyp, 0, 1, n_buckets};
+    return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, hist, nullptr, nullptr, status, 1, true, s);
+}
+
+// ---- Hop-B arrival ----------------------------------------------------------------------------
+size_t k1_workspace(int64_t R, int quota, int rpn) {
+    const int64_t P = R * quota;
+    if (P <= 0 || rpn <= 0 || rpn > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(P, rpn)) + align_up((size_t)P * sizeof(int32_t), 256);
+}
+
+int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                   int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
+                   int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
+                   size_t ws_bytes, hipStream_t s) {
+    if (R < 0 || quota <= 0 || epr <= 0 || rpn <= 0 || rpn > kMaxBuckets || my_local < 0 || my_local >= rpn ||
+        !i_send || (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0)
+        return TERRACE_EINVAL;
+    const int64_t P = R * quota;
+    if (P >= (int64_t)1 << 31) return TERRACE_EINVAL;
+    if (P == 0) return empty_outputs(i_send, nullptr, nullptr, rpn, status, s);
+    if (!rslot || !r_idx || !slot_idx || !ws || (rx && !send_buf) || (rgate && !gate_pairs)) return TERRACE_EINVAL;
+    const Units u = make_units(P, rpn);
+    const size_t table_bytes = units_table_bytes(u);
+    if (ws_bytes < table_bytes + align_up((size_t)P * sizeof(int32_t), 256)) return TERRACE_ENOSPC;
+    int32_t *table = (int32_t *)ws;
+    int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
+    KeyAffine key{rslot, 0, epr, rpn};
+    EmitArrival emit{rslot, rgate, gate_bytes, quota, gate_pairs, r_idx, slot_idx, pair_pos, pos32};
+    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, 1, true, s);
+    if (rc != TERRACE_OK || !rx) return rc;
+    return launch_scatter_rows(rx, send_buf, pos32, R, quota, row_bytes, s);
+}
+
+// ---- expert-order regroup ---------------------------------------------------------------------
+size_t regroup_workspace(int64_t P, int epr, int64_t capacity) {
+    if (P <= 0 || epr <= 0 || epr > kMaxBuckets) return 256;
+    size_t b = units_table_bytes(make_units(P, epr)) + align_up((size_t)P * sizeof(int32_t), 256);
+    if (capacity >= 0) b += align_up((size_t)epr * (size_t)capacity * sizeof(int32_t), 256);
+    return b;
+}
+
+int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
+                int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
+                int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
+                int32_t *status, void *ws, size_t ws_bytes, hipStream_t s) {
+    if (P < 0 || epr <= 0 || epr > kMaxBuckets || my_local < 0 || !tokens_per_expert || row_bytes < 0 ||
+        (gate_bytes != 2 && gate_bytes != 4) || P >= (int64_t)1 << 31 ||
+        (capacity >= 0 && (int64_t)epr * capacity >= (int64_t)1 << 31))
+        return TERRACE_EINVAL;
+    if ((node_rx && !permuted) || (my_gate && !permuted_gate)) return TERRACE_EINVAL;
+    const int64_t places = capacity >= 0 ? (int64_t)epr * capacity : P;
+    if (P == 0) {
+        int rc = empty_outputs(tokens_per_expert, nullptr, kept_per_expert, epr, status, s);
+        if (rc != TERRACE_OK || places == 0) return rc;
+        if (node_rx && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        if (my_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
+        return check_launch();
+    }
+    if (!my_slot || !ws) return TERRACE_EINVAL;
+    const Units u = make_units(P, epr);
+    const size_t table_bytes = units_table_bytes(u);
+    if (ws_bytes < regroup_workspace(P, epr, capacity)) return TERRACE_ENOSPC;
+    int32_t *table = (int32_t *)ws;
+    int32_t *order32 = (int32_t *)((char *)ws + table_bytes);
+    int32_t *gidx = (int32_t *)((char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
+    KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr};
+    EmitRegroup emit{capacity, order, dest, kept, order32};
+    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, 1, true, s);
+    if (rc != TERRACE_OK) return rc;
+    const int32_t *src_of_place = order32;
+    const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
+    if (capacity >= 0) {
+        const int64_t n = places > epr ? places : epr;
+        capacity_index_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(order32, start, epr, capacity,
+                                                                                 places, gidx, kept_per_expert);
+        src_of_place = gidx;
+    } else if (kept_per_expert) {
+        capacity_index_kernel<<<(epr + kBlock - 1) / kBlock, kBlock, 0, s>>>(order32, start, epr, INT64_MAX, 0,
+                                                                            nullptr, kept_per_expert);
+    }
+    if (my_gate && places > 0) {
+        const int grid = (int)((places + kBlock - 1) / kBlock);
+        if (gate_bytes == 4)
+            gather_elems_kernel<uint32_t><<<grid, kBlock, 0, s>>>((const uint32_t *)my_gate, src_of_place, places, (uint32_t *)permuted_gate);
+        else
+            gather_elems_kernel<uint16_t><<<grid, kBlock, 0, s>>>((const uint16_t *)my_gate, src_of_place, places, (uint16_t *)permuted_gate);
+    }
+    rc = check_launch();
+    if (rc != TERRACE_OK || !node_rx) return rc;
+    return launch_gather_rows<int32_t>(node_rx, permuted, src_of_place, places, row_bytes, s);
+}
+
+int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
+                        int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
+                        int32_t *status, hipStream_t s) {
+    if (T < 0 || k <= 0 || quota <= 0 || k % quota || slots <= 0 || n_rows < 0 ||
+        (gate_bytes != 2 && gate_bytes != 4))
+        return TERRACE_EINVAL;
+    empty_outputs_kernel<<<1, 64, 0, s>>>(nullptr, nullptr, nullptr, 0, status);
+    if (T == 0) return check_launch();
+    if (!expert_idx || !inverse || !slot_tab || (gates && !gate_tab)) return TERRACE_EINVAL;
+    const int grid = (int)((T + kBlock - 1) / kBlock);
+    if (k <= 8)
+        pack_quota_wire_kernel<8><<<grid, kBlock, 0, s>>>(expert_idx, gates, inverse, T, k, gate_bytes, n_rows, slots, quota, slot_tab, gate_tab, status);
+    else if (k <= 16)
+        pack_quota_wire_kernel<16><<<grid, kBlock, 0, s>>>(expert_idx, gates, inverse, T, k, gate_bytes, n_rows, slots, quota, slot_tab, gate_tab, status);
+    else
+        pack_quota_wire_kernel<0><<<grid, kBlock, 0, s>>>(expert_idx, gates, inverse, T, k, gate_bytes, n_rows, slots, quota, slot_tab, gate_tab, status);
+    return check_launch();
+}
+
+// ---- send side: plan + Hop-A pack ---------------------------------------------------------------
+size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m) {
+    const int64_t S = T * groups_m;
+    if (S <= 0 || n_nodes <= 0 || n_nodes > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(S, n_nodes)) + align_up((size_t)S * sizeof(int32_t), 256);
+}
+
+template <int KMAX>
+static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
+                    int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
+                    int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
+                    int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
+                    int64_t *token_rows, void *gate_sorted, int32_t *status, const Units &u, int32_t *table,
+                    int32_t *pos32, hipStream_t s) {
+    const int quota = k / groups_m;
+    KeyRun<KMAX> key{expert_idx, k, groups_m, quota, slots, n_nodes};
+    EmitPack<KMAX> emit{expert_idx, gates, gate_bytes, k, groups_m, quota, slots, n_experts,
+                        mask, u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_rows, gate_sorted,
+                        pos32};
+    int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, 1, true, s);
+    if (rc != TERRACE_OK || !hidden) return rc;
+    return launch_scatter_rows(hidden, payload, pos32, T, groups_m, row_bytes, s);
+}
+
+int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
+                int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
+                void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node, int64_t *inverse,
+                int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order, int64_t *token_rows,
+                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, hipStream_t s) {
+    if (T < 0 || k <= 0 || world <= 0 || rpn <= 0 || n_experts <= 0 || groups_m <= 0 || world % rpn ||
+        n_experts % world || k % groups_m || row_bytes < 0 || (gate_bytes != 2 && gate_bytes != 4) || !node_counts)
+        return TERRACE_EINVAL;
+    const int n_nodes = world / rpn;
+    const int slots = (n_experts / world) * rpn;
+    const int64_t S = T * groups_m;
+    if (n_nodes > kMaxBuckets || T * k >= (int64_t)1 << 31 || S >= (int64_t)1 << 31) return TERRACE_EINVAL;
+    if (S == 0) return empty_outputs(node_counts, nullptr, node_offsets, n_nodes, status, s);
+    if (!expert_idx || !mask || !u_src || !ws || (hidden && !payload) || (gates && !gate_rows)) return TERRACE_EINVAL;
+    const Units u = make_units(S, n_nodes);
+    const size_t table_bytes = units_table_bytes(u);
+    if (ws_bytes < table_bytes + align_up((size_t)S * sizeof(int32_t), 256)) return TERRACE_ENOSPC;
+    int32_t *table = (int32_t *)ws;
+    int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
+#define TERRACE_K2(KM)                                                                                        \
+    run_k2_t<KM>(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts, groups_m, \
+                 payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets, pair_table,     \
+                 sort_order, token_rows, gate_sorted, status, u, table, pos32, s)
+    if (k <= 8) return TERRACE_K2(8);
+    if (k <= 16) return TERRACE_K2(16);
+    return TERRACE_K2(0);
+#undef TERRACE_K2
+}
+
+}  // namespace terrace

@@ -1,0 +1,144 @@
+"""ctypes binding of libterrace_hip.so (the C ABI declared in include/terrace_hip.h).
+
+torch is used for device memory and for the current HIP stream only; every computation on
+the path is a kernel of the library.  There is no CPU or composed-torch fallback: a missing
+library, or a tensor that is not on a ROCm device, raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import glob
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+ENV_LIB = "TERRACE_OPS_LIB"
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(os.path.dirname(PKG_DIR), "lib")
+
+OK = 0
+F32, BF16, F16, FP8_B128 = 0, 1, 2, 3
+MODE_CODES = {"full": 0, "group_limited": 1, "quota_only": 2, "global_topk": 3}
+FORCE_GENERIC = 0x100
+FAULT_ID_RANGE, FAULT_QUOTA, FAULT_FANOUT = 1, 2, 4
+STATUS_WORDS = 4
+
+_P, _I, _L, _Z = c_void_p, c_int, c_int64, c_size_t
+
+# name -> (restype, argtypes); must list every function include/terrace_hip.h declares
+SIGNATURES = {
+    "terrace_version": (c_char_p, []),
+    "terrace_strerror": (c_char_p, [_I]),
+    "terrace_passthrough": (_I, [_P, _P, _Z, _P]),
+    "terrace_t_route": (_I, [_P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P]),
+    "terrace_hist_workspace": (_Z, [_L, _I]),
+    "terrace_hist": (_I, [_P, _L, _I, _P, _I, _P, _P, _Z, _P]),
+    "terrace_argsort_small_workspace": (_Z, [_L, _I]),
+    "terrace_argsort_small": (_I, [_P, _L, _I, _P, _P, _P, _P, _Z, _P]),
+    "terrace_k2_pack_workspace": (_Z, [_L, _I, _I, _I]),
+    "terrace_k2_pack": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I,
+                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_pack_quota_wire": (_I, [_P, _P, _P, _L, _I, _I, _L, _I, _I, _P, _P, _P, _P]),
+    "terrace_k1_arrival_workspace": (_Z, [_L, _I, _I]),
+    "terrace_k1_arrival": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I,
+                                _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_regroup_workspace": (_Z, [_L, _I, _L]),
+    "terrace_regroup": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _L,
+                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_gather_rows": (_I, [_P, _P, _L, _L, _P, _P]),
+    "terrace_index_chain": (_I, [_P, _P, _L, _P, _P]),
+    "terrace_combine": (_I, [_P, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
+    "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
+}
+
+
+class LibraryError(RuntimeError):
+    """libterrace_hip.so could not be found or loaded, or lacks a declared symbol."""
+
+
+_LIB = None
+_LIB_PATH = None
+
+
+def find_library() -> str:
+    explicit = os.environ.get(ENV_LIB)
+    if explicit:
+        if not os.path.isfile(explicit):
+            raise LibraryError(f"{ENV_LIB}={explicit} does not exist")
+        return explicit
+    hits = sorted(glob.glob(os.path.join(LIB_DIR, "libterrace_hip*.so")))
+    if not hits:
+        raise LibraryError(f"no libterrace_hip.so under {LIB_DIR}; build it with "
+                           f"`python terracemoe-simulator_amd/csrc/build.py`")
+    return hits[0]
+
+
+def load(path: str | None = None):
+    """Load (once) and type every entry point.  Raises LibraryError on any problem."""
+    global _LIB, _LIB_PATH
+    if _LIB is not None and (path is None or path == _LIB_PATH):
+        return _LIB
+    path = path or find_library()
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise LibraryError(f"dlopen({path}) failed: {e}") from e
+    missing = [n for n in SIGNATURES if not hasattr(lib, n)]
+    if missing:
+        raise LibraryError(f"{path} lacks {missing}")
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    _LIB, _LIB_PATH = lib, path
+    return lib
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def unload_for_tests():
+    global _LIB, _LIB_PATH
+    _LIB = _LIB_PATH = None
+
+
+def call(name: str, *args):
+    rc = getattr(load(), name)(*args)
+    if rc != OK:
+        msg = load().terrace_strerror(rc).decode()
+        raise RuntimeError(f"{name} failed: {msg} (status {rc})")
+
+
+def query(name: str, *args) -> int:
+    return int(getattr(load(), name)(*args))
+
+
+def need_device(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("terrace (MI355X build): tensors must live on a ROCm device; this build has no "
+                               "CPU path")
+
+
+def ptr(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def stream(device) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def float_code(dtype) -> int:
+    try:
+        return {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}[dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported floating dtype {dtype}") from None
+
+
+def workspace(nbytes: int, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def new_status(device):
+    return torch.empty(STATUS_WORDS, dtype=torch.int32, device=device)

@@ -1,0 +1,549 @@
+"""terrace.ops: loader switch and operator entry points of the MI355X kernel library.
+
+Mirrors the reference plugin boundary (terrace/ops/__init__.py:53-179 there): the same
+``TERRACE_CUSTOM_OPS`` / ``TERRACE_OPS_LIB`` environment switch read once and cached,
+``status() / custom_ops_enabled() / reset()``, ``OpsState``, ``OpsLoadError``, and the
+operators ``passthrough``, ``k1_arrival``, ``k1_arrival_segment`` plus ``k2_pack`` -- also
+registered as ``torch.ops.terrace.{passthrough,k1_arrival,k2_pack}`` with the reference
+schemas (terrace/ops/csrc/terrace_ops.cpp:230-232, terrace/ops/csrc/terrace_k2_pack.cpp:209-211).
+
+One deliberate difference: this build contains no composed torch chain to fall back to, so
+the library is the only implementation.  Switch values:
+
+    unset, "1"       load the library; a failure is logged once as a WARNING and every
+                     operator then raises OpsLoadError when called (never a silent fallback)
+    "require" / "2"  a load failure raises RuntimeError from status()
+    "0"              explicitly off: no load attempt, operators raise OpsLoadError
+"""
+from __future__ import annotations
+
+import logging
+import os
+from dataclasses import dataclass
+
+import torch
+
+from .. import _hip
+
+_LOG = logging.getLogger("terrace.ops")
+
+_ENV_SWITCH = "TERRACE_CUSTOM_OPS"
+_ENV_LIB = _hip.ENV_LIB
+_REQUIRED_OPS = ("passthrough", "k1_arrival")
+
+
+class OpsLoadError(RuntimeError):
+    """The kernel library failed to load (.so not found / dlopen failed / symbol missing)."""
+
+
+@dataclass(frozen=True)
+class OpsState:
+    requested: str        # "0" | "1" | "require" (normalised)
+    loaded: bool
+    lib: str | None
+    reason: str           # "ok" when loaded
+
+
+_STATE: OpsState | None = None
+
+
+def _normalized_switch() -> str:
+    raw = os.environ.get(_ENV_SWITCH, "1").strip()
+    if raw in ("2", "require"):
+        return "require"
+    if raw == "0":
+        return "0"
+    return "1"
+
+
+def _initialize() -> OpsState:
+    switch = _normalized_switch()
+    if switch == "0":
+        return OpsState("0", False, None, f"{_ENV_SWITCH}=0 (explicitly off; no load attempted)")
+    try:
+        _hip.load()
+        _register_torch_ops()
+        _LOG.info("terrace kernel library loaded: %s", _hip.library_path())
+        return OpsState(switch, True, _hip.library_path(), "ok")
+    except _hip.LibraryError as e:
+        if switch == "require":
+            raise RuntimeError(f"{_ENV_SWITCH}={os.environ.get(_ENV_SWITCH)} requires the kernel library, "
+                               f"but loading failed: {e}") from e
+        _LOG.warning("terrace kernel library unavailable (%s) -- operators will raise when called", e)
+        return OpsState(switch, False, None, str(e))
+
+
+def status() -> OpsState:
+    global _STATE
+    if _STATE is None:
+        _STATE = _initialize()
+    return _STATE
+
+
+def custom_ops_enabled() -> bool:
+    return status().loaded
+
+
+def reset() -> None:
+    """Forget the cached verdict (test hook); the next status() re-reads the environment."""
+    global _STATE
+    _STATE = None
+    _hip.unload_for_tests()
+
+
+def _require():
+    st = status()
+    if not st.loaded:
+        raise OpsLoadError(f"terrace kernel library not loaded: {st.reason}")
+
+
+# --------------------------------------------------------------------------------------
+# raw operators (forward only, no autograd)
+# --------------------------------------------------------------------------------------
+
+def _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local):
+    """Same refusals as the reference binding (terrace/ops/csrc/terrace_ops.cpp:123-144),
+    minus its NPU-only limits (63 slots, 32-byte rows)."""
+    if rx.dim() != 2 or rslot.dim() != 2 or rgate.dim() != 2:
+        raise RuntimeError("terrace::k1_arrival: rx/rslot/rgate must be 2-D")
+    if rslot.dtype != torch.int64:
+        raise RuntimeError("terrace::k1_arrival: rslot must be int64 (quota wire format)")
+    if rgate.dtype != rx.dtype and rx.dtype != torch.uint8:
+        raise RuntimeError("terrace::k1_arrival: rgate dtype must equal rx dtype (the gate plane is "
+                           "allocated from the payload)")
+    if not (rslot.shape[1] == quota and rgate.shape[1] == quota and rslot.shape[0] == rx.shape[0]
+            and rgate.shape[0] == rx.shape[0]):
+        raise RuntimeError(f"terrace::k1_arrival: geometry mismatch (rx {tuple(rx.shape)}, rslot "
+                           f"{tuple(rslot.shape)}, rgate {tuple(rgate.shape)}, quota {quota})")
+    if not (quota > 0 and epr > 0 and rpn > 0 and 0 <= my_local < rpn):
+        raise RuntimeError("terrace::k1_arrival: bad geometry scalars")
+    if rgate.element_size() not in (2, 4):
+        raise RuntimeError(f"terrace::k1_arrival: unsupported gate dtype {rgate.dtype}")
+
+
+def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=False, status_out=None):
+    """(send_buf, gate_pairs, r_idx, slot_idx, i_send[, pair_pos]) -- one library call."""
+    _require()
+    _hip.need_device(rx, rslot, rgate)
+    _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local)
+    rx, rslot, rgate = rx.contiguous(), rslot.contiguous(), rgate.contiguous()
+    dev = rx.device
+    R, H = rx.shape
+    P = R * quota
+    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev)
+    gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
+    r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
+    pair_pos = torch.empty((P,), dtype=torch.int64, device=dev) if want_pair_pos else None
+    st = status_out if status_out is not None else _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
+    _hip.call("terrace_k1_arrival", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, H * rx.element_size(),
+              rgate.element_size(), quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(gate_pairs),
+              _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    out = (send_buf, gate_pairs, r_idx, slot_idx, i_send)
+    return out + (pair_pos,) if want_pair_pos else out
+
+
+def _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+    """Refusals of terrace/ops/k2_ref.py:87-108 (same exception classes), minus the id-range
+    read-back (reported through the status words instead) and the 63-slot mask bound."""
+    if expert_idx.dim() != 2 or hidden.dim() != 2 or gates.dim() != 2:
+        raise ValueError("k2_pack: hidden/expert_idx/gates must be 2-D")
+    T, k = expert_idx.shape
+    if hidden.shape[0] != T or gates.shape != expert_idx.shape:
+        raise ValueError(f"k2_pack: geometry mismatch (hidden {tuple(hidden.shape)}, expert_idx "
+                         f"{tuple(expert_idx.shape)}, gates {tuple(gates.shape)})")
+    if gates.dtype != hidden.dtype and hidden.dtype != torch.uint8:
+        raise RuntimeError(f"k2_pack: gates dtype {gates.dtype} != hidden dtype {hidden.dtype} -- the gate "
+                           f"plane derives from the payload; cast at the caller")
+    if gates.element_size() not in (2, 4):
+        raise RuntimeError(f"k2_pack: unsupported gate dtype {gates.dtype}")
+    if expert_idx.dtype != torch.int64:
+        raise RuntimeError("k2_pack: expert_idx must be int64")
+    if world <= 0 or rpn <= 0 or groups_m <= 0 or n_experts <= 0:
+        raise ValueError("k2_pack: bad geometry scalars")
+    if world % rpn or n_experts % world or k % groups_m:
+        raise ValueError(f"k2_pack: world={world} rpn={rpn} n_experts={n_experts} k={k} "
+                         f"groups_m={groups_m} not divisible")
+
+
+def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=False, status_out=None):
+    """(payload, mask, gate_rows, u_src, node_counts) and, with ``extras``, a dict holding
+    u_node, inverse, node_offsets, pair_table, sort_order, token_rows, gate_sorted and the
+    status words."""
+    _require()
+    _hip.need_device(hidden, expert_idx, gates)
+    _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+    hidden, expert_idx, gates = hidden.contiguous(), expert_idx.contiguous(), gates.contiguous()
+    dev = expert_idx.device
+    T, k = expert_idx.shape
+    H = hidden.shape[1]
+    S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
+    payload = torch.empty((S, H), dtype=hidden.dtype, device=dev)
+    mask = torch.empty((S, q), dtype=torch.int64, device=dev)
+    gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
+    u_src = torch.empty((S,), dtype=torch.int64, device=dev)
+    node_counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
+    ex = {}
+    if extras:
+        ex = {"u_node": torch.empty((S,), dtype=torch.int64, device=dev),
+              "inverse": torch.empty((T * k,), dtype=torch.int64, device=dev),
+              "node_offsets": torch.empty((n_nodes,), dtype=torch.int64, device=dev),
+              "pair_table": torch.empty((T, k), dtype=torch.int64, device=dev),
+              "sort_order": torch.empty((T, k), dtype=torch.int64, device=dev),
+              "token_rows": torch.empty((T, groups_m), dtype=torch.int64, device=dev),
+              "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
+    st = status_out if status_out is not None else _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
+    _hip.call("terrace_k2_pack", _hip.ptr(hidden), _hip.ptr(expert_idx), _hip.ptr(gates), T,
+              H * hidden.element_size(), gates.element_size(), k, world, n_experts, rpn, groups_m,
+              _hip.ptr(payload), _hip.ptr(mask), _hip.ptr(gate_rows), _hip.ptr(u_src), _hip.ptr(node_counts),
+              _hip.ptr(ex.get("u_node")), _hip.ptr(ex.get("inverse")), _hip.ptr(ex.get("node_offsets")),
+              _hip.ptr(ex.get("pair_table")), _hip.ptr(ex.get("sort_order")), _hip.ptr(ex.get("token_rows")),
+              _hip.ptr(ex.get("gate_sorted")), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    out = (payload, mask, gate_rows, u_src, node_counts)
+    if extras:
+        ex["status"] = st
+        return out, ex
+    return out
+
+
+def plan_raw(expert_idx, world, n_experts, rpn, groups_m):
+    """Index build only: (u_src, u_node, node_counts, inverse, extras incl. mask planes, status)."""
+    _require()
+    _hip.need_device(expert_idx)
+    expert_idx = expert_idx.contiguous()
+    dev = expert_idx.device
+    T, k = expert_idx.shape
+    S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
+    mask = torch.empty((S, q), dtype=torch.int64, device=dev)
+    u_src = torch.empty((S,), dtype=torch.int64, device=dev)
+    u_node = torch.empty((S,), dtype=torch.int64, device=dev)
+    inverse = torch.empty((T * k,), dtype=torch.int64, device=dev)
+    counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
+    _hip.call("terrace_k2_pack", None, _hip.ptr(expert_idx), None, T, 0, 4, k, world, n_experts, rpn, groups_m,
+              None, _hip.ptr(mask), None, _hip.ptr(u_src), _hip.ptr(counts), _hip.ptr(u_node),
+              _hip.ptr(inverse), None, None, None, None, None, _hip.ptr(st), _hip.ptr(ws), ws.numel(),
+              _hip.stream(dev))
+    return u_src, u_node, counts, inverse, mask, st
+
+
+def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
+    """Expert-order regroup of the rows an expert card received.
+
+    Drop-less (``capacity=None``; terrace/ta2a_fwd.py:641-646 of the reference):
+    returns ``(permuted, order, tokens_per_expert)`` (+ ``permuted_gate`` when ``my_gate``).
+    With ``capacity`` (this build's own definition): expert x keeps its first ``capacity``
+    rows in stable order; returns ``(padded [epr*capacity, H], dest [P], kept [P] bool,
+    tokens_per_expert, kept_per_expert)`` (+ ``padded_gate``).
+    """
+    _require()
+    _hip.need_device(node_rx, my_slot, my_gate)
+    if my_slot.dtype != torch.int64:
+        raise RuntimeError("regroup: my_slot must be int64")
+    node_rx, my_slot = node_rx.contiguous(), my_slot.contiguous().reshape(-1)
+    dev = my_slot.device
+    P = my_slot.numel()
+    if node_rx.dim() != 2 or node_rx.shape[0] != P:
+        raise RuntimeError(f"regroup: node_rx {tuple(node_rx.shape)} does not have one row per slot id ({P})")
+    H = node_rx.shape[1]
+    cap = -1 if capacity is None else int(capacity)
+    places = P if capacity is None else epr * cap
+    permuted = torch.empty((places, H), dtype=node_rx.dtype, device=dev)
+    tpe = torch.empty((epr,), dtype=torch.int64, device=dev)
+    kpe = torch.empty((epr,), dtype=torch.int64, device=dev)
+    order = torch.empty((P,), dtype=torch.int64, device=dev) if capacity is None else None
+    dest = torch.empty((P,), dtype=torch.int64, device=dev) if capacity is not None else None
+    kept = torch.empty((P,), dtype=torch.uint8, device=dev) if capacity is not None else None
+    pgate = None
+    gate_bytes = 4
+    if my_gate is not None:
+        my_gate = my_gate.contiguous().reshape(-1)
+        gate_bytes = my_gate.element_size()
+        pgate = torch.empty((places,), dtype=my_gate.dtype, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, cap), dev)
+    _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), _hip.ptr(my_gate), P,
+              H * node_rx.element_size(), gate_bytes, epr, my_local, cap, _hip.ptr(permuted), _hip.ptr(pgate),
+              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    if capacity is None:
+        out = (permuted, order, tpe)
+    else:
+        out = (permuted, dest, kept.bool(), tpe, kpe)
+    return out + (pgate,) if my_gate is not None else out
+
+
+def gather_rows(src, idx):
+    """``src[idx]`` for a 2-D ``src``; negative indices give zero rows."""
+    _require()
+    _hip.need_device(src, idx)
+    src, idx = src.contiguous(), idx.contiguous().reshape(-1)
+    if idx.dtype != torch.int64:
+        raise RuntimeError("gather_rows: idx must be int64")
+    out = torch.empty((idx.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+    row_bytes = src.element_size()
+    for d in src.shape[1:]:
+        row_bytes *= int(d)
+    _hip.call("terrace_gather_rows", _hip.ptr(src), _hip.ptr(idx), idx.numel(), row_bytes, _hip.ptr(out),
+              _hip.stream(src.device))
+    return out
+
+
+def index_chain(table, idx):
+    """``table[idx]`` over int64 planes (negative entries propagate as -1)."""
+    _require()
+    _hip.need_device(table, idx)
+    table, idx = table.contiguous(), idx.contiguous()
+    out = torch.empty_like(idx)
+    _hip.call("terrace_index_chain", _hip.ptr(table), _hip.ptr(idx), idx.numel(), _hip.ptr(out),
+              _hip.stream(idx.device))
+    return out
+
+
+def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
+    """``out[i] = sum_j weights[i,j] * src[idx[i,j]]`` accumulated in fp32 in the order ``idx``
+    lists the rows, rounded once to ``out_dtype`` (default: ``src.dtype``, or bf16 for fp8 rows).
+
+    ``src`` is [n, H] float32 / bfloat16 / float16, or with ``fp8_hidden=H`` a uint8
+    [n, H + H/32] plane of e4m3 rows followed by their per-128 fp32 scales.
+    """
+    _require()
+    _hip.need_device(src, idx, weights)
+    src, idx = src.contiguous(), idx.contiguous()
+    if idx.dim() != 2 or idx.dtype != torch.int64:
+        raise RuntimeError("combine: idx must be a 2-D int64 table")
+    n_out, fan = idx.shape
+    if fp8_hidden is not None:
+        hidden = int(fp8_hidden)
+        if src.dtype != torch.uint8 or src.shape[1] != hidden + hidden // 32 or hidden % 128:
+            raise RuntimeError("combine: fp8 rows must be uint8 [n, H + H/32] with H a multiple of 128")
+        src_code = _hip.FP8_B128
+        out_dtype = out_dtype or torch.bfloat16
+    else:
+        hidden = src.shape[1]
+        src_code = _hip.float_code(src.dtype)
+        out_dtype = out_dtype or src.dtype
+    w_code = 0
+    if weights is not None:
+        weights = weights.contiguous()
+        if tuple(weights.shape) != (n_out, fan):
+            raise RuntimeError("combine: weights must match idx")
+        w_code = _hip.float_code(weights.dtype)
+    out = torch.empty((n_out, hidden), dtype=out_dtype, device=src.device)
+    _hip.call("terrace_combine", _hip.ptr(src), src_code, _hip.ptr(idx), _hip.ptr(weights), w_code, n_out, fan,
+              hidden, _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
+    return out
+
+
+def hist(idx, n_buckets, as_float=False):
+    _require()
+    _hip.need_device(idx)
+    idx = idx.contiguous().reshape(-1)
+    if idx.dtype != torch.int64:
+        raise RuntimeError("hist: idx must be int64")
+    dev = idx.device
+    out = torch.empty((n_buckets,), dtype=torch.float32 if as_float else torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_hist_workspace", idx.numel(), n_buckets), dev)
+    _hip.call("terrace_hist", _hip.ptr(idx), idx.numel(), n_buckets, _hip.ptr(out), int(as_float), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return out, st
+
+
+def argsort_small(key, n_buckets):
+    _require()
+    _hip.need_device(key)
+    key = key.contiguous().reshape(-1)
+    if key.dtype != torch.int64:
+        raise RuntimeError("argsort_small: key must be int64")
+    dev = key.device
+    order = torch.empty_like(key)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_argsort_small_workspace", key.numel(), n_buckets), dev)
+    _hip.call("terrace_argsort_small", _hip.ptr(key), key.numel(), n_buckets, _hip.ptr(order), None, _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return order, st
+
+
+def hopa_send_splits(node_counts, world, rpn, my_local):
+    """Hop-A counts-exchange send buffer (terrace/ta2a_dispatch.py:197-211 of the reference)."""
+    _require()
+    _hip.need_device(node_counts)
+    node_counts = node_counts.contiguous()
+    send = torch.empty((world,), dtype=torch.int64, device=node_counts.device)
+    _hip.call("terrace_hopa_send_splits", _hip.ptr(node_counts), world, rpn, my_local, _hip.ptr(send),
+              _hip.stream(node_counts.device))
+    return send
+
+
+# --------------------------------------------------------------------------------------
+# torch.ops.terrace registration (reference schemas)
+# --------------------------------------------------------------------------------------
+
+_TORCH_LIB = None
+
+
+def _register_torch_ops():
+    global _TORCH_LIB
+    if _TORCH_LIB is not None:
+        return
+    lib = torch.library.Library("terrace", "DEF")
+    lib.define("passthrough(Tensor x) -> Tensor")
+    lib.define("k1_arrival(Tensor rx, Tensor rslot, Tensor rgate, int quota, int epr, int rpn, int my_local) "
+               "-> (Tensor, Tensor, Tensor, Tensor, Tensor)")
+    lib.define("k2_pack(Tensor hidden, Tensor expert_idx, Tensor gates, int world, int n_experts, int rpn, "
+               "int groups_m) -> (Tensor, Tensor, Tensor, Tensor, Tensor)")
+
+    def _pass(x):
+        _hip.need_device(x)
+        xc = x.contiguous()
+        y = torch.empty_like(xc)
+        _hip.call("terrace_passthrough", _hip.ptr(xc), _hip.ptr(y), xc.numel() * xc.element_size(),
+                  _hip.stream(x.device))
+        return y
+
+    def _k1(rx, rslot, rgate, quota, epr, rpn, my_local):
+        return k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local)
+
+    def _k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+        return k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+
+    def _k1_meta(rx, rslot, rgate, quota, epr, rpn, my_local):
+        P, H = rslot.shape[0] * quota, rx.shape[1]
+        return (rx.new_empty((P, H)), rgate.new_empty((P,)), rslot.new_empty((P,)), rslot.new_empty((P,)),
+                rslot.new_empty((rpn,)))
+
+    def _k2_meta(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+        n_rows, q = expert_idx.shape[0] * groups_m, expert_idx.shape[1] // groups_m
+        return (hidden.new_empty((n_rows, hidden.shape[1])), expert_idx.new_empty((n_rows, q)),
+                gates.new_empty((n_rows, q)), expert_idx.new_empty((n_rows,)),
+                expert_idx.new_empty((world // rpn,)))
+
+    lib.impl("passthrough", _pass, "CUDA")
+    lib.impl("k1_arrival", _k1, "CUDA")
+    lib.impl("k2_pack", _k2, "CUDA")
+    lib.impl("passthrough", lambda x: torch.empty_like(x), "Meta")
+    lib.impl("k1_arrival", _k1_meta, "Meta")
+    lib.impl("k2_pack", _k2_meta, "Meta")
+    _TORCH_LIB = lib
+
+
+# --------------------------------------------------------------------------------------
+# autograd wrappers and functional entry points (reference names)
+# --------------------------------------------------------------------------------------
+
+class TerracePassthroughFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        return torch.ops.terrace.passthrough(x)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        return grad_out
+
+
+def passthrough(x: torch.Tensor) -> torch.Tensor:
+    """Identity copy through the streaming-copy kernel: a new tensor, bit-equal to ``x``."""
+    _require()
+    return TerracePassthroughFn.apply(x)
+
+
+def _k1_grad_rx(g_send, pair_pos, rx_shape, quota):
+    """Adjoint of ``send_buf = rx[r_idx]``: row r sums its quota pairs, in pair order."""
+    return combine(g_send, pair_pos.view(rx_shape[0], quota), None, out_dtype=g_send.dtype)
+
+
+def _k1_grad_rgate(g_gate, pair_pos, rgate_shape):
+    """Adjoint of ``gate_pairs = rgate.flatten()[ordo]``: a permutation, so a plain gather."""
+    return gather_rows(g_gate.reshape(-1, 1), pair_pos).view(rgate_shape)
+
+
+class TerraceK1ArrivalFn(torch.autograd.Function):
+    """Forward = the arrival kernel; backward = the two gather adjoints
+    (terrace/ops/__init__.py:303-365 of the reference), also as kernels."""
+
+    @staticmethod
+    def forward(ctx, rx, rslot, rgate, quota, epr, rpn, my_local):
+        send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = k1_arrival_raw(
+            rx, rslot, rgate, quota, epr, rpn, my_local, want_pair_pos=True)
+        ctx.save_for_backward(pair_pos)
+        ctx.k1_geom = (quota, rx.shape, rgate.shape)
+        ctx.mark_non_differentiable(r_idx, slot_idx, i_send)
+        return send_buf, gate_pairs, r_idx, slot_idx, i_send
+
+    @staticmethod
+    def backward(ctx, g_send, g_gate, _g_r, _g_s, _g_i):
+        (pair_pos,) = ctx.saved_tensors
+        quota, rx_shape, rgate_shape = ctx.k1_geom
+        grad_rx = grad_rgate = None
+        if ctx.needs_input_grad[0] and g_send is not None:
+            grad_rx = _k1_grad_rx(g_send.contiguous(), pair_pos, rx_shape, quota)
+        if ctx.needs_input_grad[2] and g_gate is not None:
+            grad_rgate = _k1_grad_rgate(g_gate.contiguous(), pair_pos, rgate_shape)
+        return grad_rx, None, grad_rgate, None, None, None, None
+
+
+def k1_arrival(rx, rslot, rgate, quota: int, epr: int, rpn: int, my_local: int = 0):
+    """Arrival-side fused chain: (send_buf, gate_pairs, r_idx, slot_idx, i_send)."""
+    _require()
+    if rx.requires_grad or rgate.requires_grad:
+        return TerraceK1ArrivalFn.apply(rx, rslot, rgate, quota, epr, rpn, my_local)
+    return k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local)
+
+
+class _K1SendEdge(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rx, pair_pos, send_buf, quota):
+        ctx.save_for_backward(pair_pos)
+        ctx.geom = (rx.shape, quota)
+        return send_buf
+
+    @staticmethod
+    def backward(ctx, g_send):
+        (pair_pos,) = ctx.saved_tensors
+        rx_shape, quota = ctx.geom
+        g = _k1_grad_rx(g_send.contiguous(), pair_pos, rx_shape, quota) if ctx.needs_input_grad[0] else None
+        return g, None, None, None
+
+
+class _K1GateEdge(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, rgate, pair_pos, gate_pairs):
+        ctx.save_for_backward(pair_pos)
+        ctx.geom = rgate.shape
+        return gate_pairs
+
+    @staticmethod
+    def backward(ctx, g_gate):
+        (pair_pos,) = ctx.saved_tensors
+        g = _k1_grad_rgate(g_gate.contiguous(), pair_pos, ctx.geom) if ctx.needs_input_grad[0] else None
+        return g, None, None
+
+
+def k1_arrival_segment(rx, rslot, rgate, quota: int, epr: int, rpn: int, my_local: int = 0):
+    """Same values as ``k1_arrival``; the two float outputs hang on separate autograd edges
+    rooted at ``rx`` / ``rgate`` (terrace/ops/__init__.py:452-474 of the reference)."""
+    with torch.no_grad():
+        send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = k1_arrival_raw(
+            rx.detach(), rslot, rgate.detach(), quota, epr, rpn, my_local, want_pair_pos=True)
+    send_buf = _K1SendEdge.apply(rx, pair_pos, send_buf, quota)
+    gate_pairs = _K1GateEdge.apply(rgate, pair_pos, gate_pairs)
+    return send_buf, gate_pairs, r_idx, slot_idx, i_send
+
+
+def k2_pack(hidden, expert_idx, gates, world: int, n_experts: int, rpn: int, groups_m: int):
+    """Send-side fused chain: (payload, mask, gate_rows, u_src, node_counts)."""
+    _require()
+    return k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+
+
+__all__ = [
+    "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
+    "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
+    "regroup", "combine", "gather_rows", "index_chain", "hist", "argsort_small", "hopa_send_splits",
+]

@@ -1,0 +1,155 @@
+"""T-A2A forward primitives on MI355X, and the one-GPU loop-back forward.
+
+Same names as the reference module (terrace/ta2a_fwd.py there) for the primitives the
+dispatch/combine path is made of: ``fixed_hist``, ``_stable_argsort_small``,
+``_pack_quota_wire``, ``_expand_arrival_quota``.  The reference's ``ta2a_moe_forward`` strings
+them together around four all-to-all exchanges; on one GPU those exchanges cannot run, so
+``ta2a_loopback_forward`` runs the same stages with the rank's own Hop-A send buffer looped
+back as its arrival buffer (slot ids are node-local, so that is a well-formed arrival set of
+the balanced size) and every expert slot of the node treated as local.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _hip
+from . import ops as _ops
+
+
+def fixed_hist(idx: torch.Tensor, n_buckets: int) -> torch.Tensor:
+    """Fixed-length int64 histogram (``bincount(idx, minlength=n_buckets)`` without the sync)."""
+    out, _ = _ops.hist(idx, n_buckets)
+    return out
+
+
+def _stable_argsort_small(key: torch.Tensor, n_buckets: int) -> torch.Tensor:
+    """Stable ascending argsort of a small-range integer key (a counting sort)."""
+    order, _ = _ops.argsort_small(key, n_buckets)
+    return order
+
+
+def _pack_quota_wire(expert_idx, gates, inverse, payload, n_rows: int, slots: int, quota: int,
+                     n_experts: int, *, sorted_rows: bool = False):
+    """Quota Hop-A id/gate planes: ``[n_rows, quota]`` ascending node-local slot ids (int64)
+    and the co-indexed gates in the payload's dtype.  ``sorted_rows`` is accepted for
+    signature compatibility; the kernel ranks each row itself, which is the identity on an
+    ascending row."""
+    _ops._require()
+    _hip.need_device(expert_idx, gates, inverse, payload)
+    if gates.dtype != payload.dtype and payload.dtype != torch.uint8:
+        raise RuntimeError(f"Index put requires the source and destination dtypes match, got {payload.dtype} "
+                           f"for the destination and {gates.dtype} for the source.")
+    expert_idx, gates, inverse = expert_idx.contiguous(), gates.contiguous(), inverse.contiguous()
+    T, k = expert_idx.shape
+    dev = expert_idx.device
+    slot_tab = torch.zeros((n_rows, quota), dtype=torch.int64, device=dev)
+    gate_tab = torch.zeros((n_rows, quota), dtype=gates.dtype, device=dev)
+    st = _hip.new_status(dev)
+    _hip.call("terrace_pack_quota_wire", _hip.ptr(expert_idx), _hip.ptr(gates), _hip.ptr(inverse), T, k,
+              gates.element_size(), n_rows, slots, quota, _hip.ptr(slot_tab), _hip.ptr(gate_tab), _hip.ptr(st),
+              _hip.stream(dev))
+    return slot_tab, gate_tab
+
+
+def _expand_arrival_quota(rslot: torch.Tensor):
+    """(r_idx, slot_idx) pairs straight off the quota wire table, row-major."""
+    R, quota = rslot.shape
+    r_idx = torch.arange(R, device=rslot.device, dtype=torch.int64).unsqueeze(1).expand(R, quota).reshape(-1)
+    return r_idx, rslot.reshape(-1)
+
+
+@dataclass
+class LoopbackState:
+    """What the combine needs from the dispatch, and what a caller may want to inspect."""
+    payload: torch.Tensor
+    mask: torch.Tensor
+    gate_rows: torch.Tensor
+    u_src: torch.Tensor
+    node_counts: torch.Tensor
+    extras: dict
+    send_buf: torch.Tensor
+    gate_pairs: torch.Tensor
+    r_idx: torch.Tensor
+    slot_idx: torch.Tensor
+    i_send: torch.Tensor
+    pair_pos: torch.Tensor
+    permuted: torch.Tensor
+    tokens_per_expert: torch.Tensor
+    place: torch.Tensor            # [P] where each arrival row sits in the expert-order buffer, -1 = dropped
+    kept: torch.Tensor | None
+    capacity: int | None
+
+
+def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8, groups_m: int = 1,
+                      capacity: int | None = None) -> LoopbackState:
+    """Stages 2-4 on one GPU: index build + Hop-A pack, arrival chain, expert-order regroup."""
+    epr = n_experts // world
+    slots = epr * rpn
+    k = expert_idx.shape[1]
+    quota = k // groups_m
+    (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
+        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+    send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = _ops.k1_arrival_raw(
+        payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True)
+    if capacity is None:
+        permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots)
+        kept = None
+    else:
+        permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity)
+    return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
+                         slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
+
+
+def _regroup_with_place(node_rx, my_slot, epr):
+    """Drop-less regroup that also returns each input row's place (the inverse of ``order``)."""
+    _ops._require()
+    node_rx, my_slot = node_rx.contiguous(), my_slot.contiguous().reshape(-1)
+    dev = my_slot.device
+    P, H = node_rx.shape
+    permuted = torch.empty_like(node_rx)
+    order = torch.empty((P,), dtype=torch.int64, device=dev)
+    place = torch.empty((P,), dtype=torch.int64, device=dev)
+    tpe = torch.empty((epr,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, -1), dev)
+    _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), None, P, H * node_rx.element_size(), 4, epr,
+              0, -1, _hip.ptr(permuted), None, _hip.ptr(order), _hip.ptr(place), None, _hip.ptr(tpe), None,
+              _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return permuted, order, tpe, place
+
+
+def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, weights=None):
+    """Stage 5, fused: ``y[t] = sum_s gate[t,s] * ye[place of (t, s-th smallest expert)]``.
+
+    The k rows of a token are added in ascending expert id -- slot ascending inside a send row,
+    node ascending across the token's rows -- which is the order the reference's two
+    ``index_add`` levels add in (terrace/ta2a_fwd.py:661-670 there), accumulated in fp32.
+    """
+    where = _ops.index_chain(st.place, _ops.index_chain(st.pair_pos, st.extras["pair_table"]))
+    w = st.extras["gate_sorted"] if weights is None else weights
+    return _ops.combine(ye, where, w, out_dtype=out_dtype, fp8_hidden=fp8_hidden)
+
+
+def twolevel_combine(ye, st: LoopbackState, out_dtype=None):
+    """Stage 5 in the reference's two levels (what a multi-GPU run would execute either side
+    of the return exchanges): un-permute, per-row gate-weighted sum over the quota pairs, then
+    per-token sum over the M rows.  Each level rounds to the payload dtype, as the reference."""
+    R, q = st.mask.shape
+    ret_place = _ops.index_chain(st.place, st.pair_pos).view(R, q)      # ye row of pair (r, i)
+    red = _ops.combine(ye, ret_place, st.gate_rows, out_dtype=out_dtype)
+    return _ops.combine(red, st.extras["token_rows"], None, out_dtype=out_dtype)
+
+
+def ta2a_loopback_forward(x, expert_idx, gates, expert_fn, world: int, n_experts: int, rpn: int = 8,
+                          groups_m: int = 1, capacity: int | None = None):
+    """dispatch -> ``expert_fn(permuted, tokens_per_expert) -> ye`` -> combine, on one GPU."""
+    st = loopback_dispatch(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity)
+    ye = expert_fn(st.permuted, st.tokens_per_expert)
+    return loopback_combine(ye, st), st
+
+
+def ta2a_moe_forward(*_args, **_kwargs):
+    raise NotImplementedError("ta2a_moe_forward needs the all-to-all exchanges of a multi-GPU run; this "
+                              "one-GPU build provides ta2a_loopback_forward and the per-stage operators")

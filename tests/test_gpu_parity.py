@@ -1,0 +1,448 @@
+"""HIP path vs the CPU oracle on identical seeded inputs -- through the C ABI (ctypes) only.
+
+Bit-exact for every index / count / offset plane and every moved row; the combine is
+bit-exact against the oracle's fp32 left-to-right definition and within the stated
+tolerance (1e-5 fp32, 1e-2 bf16) of a float64 evaluation of the same sum.
+"""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import arrival_plane, equal_quota_routing
+from oracle import terrace_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+DT = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def to_np(t: torch.Tensor) -> np.ndarray:
+    t = t.detach().cpu()
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    if t.dtype == torch.bool:
+        return t.numpy()
+    return t.numpy()
+
+
+def rows_of(x_f32: torch.Tensor, fmt: str) -> torch.Tensor:
+    return x_f32.to(DT[fmt])
+
+
+def same(a: torch.Tensor, b: np.ndarray, what: str):
+    got = to_np(a)
+    assert got.shape == tuple(b.shape), f"{what}: shape {got.shape} != {b.shape}"
+    assert got.dtype == b.dtype, f"{what}: dtype {got.dtype} != {b.dtype}"
+    assert np.array_equal(got, b), f"{what}: values differ"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _ops_loaded():
+    import terrace.ops as tops
+    tops.reset()
+    assert tops.status().loaded, tops.status().reason
+    yield
+
+
+# ------------------------------------------------------------------------------- passthrough
+
+@pytest.mark.parametrize("shape,dtype", [((0,), torch.float32), ((1,), torch.uint8), ((17,), torch.uint8),
+                                          ((33, 7), torch.bfloat16), ((4096, 1024), torch.float32),
+                                          ((1000, 7168), torch.bfloat16)])
+def test_passthrough_is_a_bitwise_copy(shape, dtype):
+    import terrace.ops as tops
+    announce("passthrough", shape, dtype)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randint(0, 255, shape, generator=g, dtype=torch.uint8) if dtype == torch.uint8 else \
+        torch.randn(shape, generator=g).to(dtype)
+    xd = x.to(DEV)
+    y = tops.passthrough(xd)
+    assert y.data_ptr() != xd.data_ptr() or xd.numel() == 0
+    assert y.dtype == x.dtype and y.shape == x.shape and torch.equal(y.cpu(), x)
+    assert torch.equal(torch.ops.terrace.passthrough(xd).cpu(), x)
+
+
+# ------------------------------------------------------------------------------- routing
+
+ROUTE_GEOMS = [  # (T, E, N_g, k, M)
+    (512, 64, 8, 8, 4), (4096, 64, 8, 4, 2), (2048, 256, 8, 8, 4), (1024, 128, 16, 8, 2),
+    (257, 16, 4, 4, 2), (33, 24, 3, 6, 3), (64, 8, 8, 2, 2), (100, 32, 1, 4, 1), (65, 96, 4, 8, 4),
+    (31, 512, 8, 8, 4), (9, 1024, 8, 16, 4), (40, 40, 5, 4, 2),
+]
+
+
+@pytest.mark.parametrize("geom", ROUTE_GEOMS, ids=lambda g: "T%dE%dG%dk%dM%d" % g)
+@pytest.mark.parametrize("generic", [False, True])
+def test_route_full_bit_exact(geom, generic):
+    import terrace
+    T, E, Ng, k, M = geom
+    announce("route", geom, "generic" if generic else "auto")
+    g = torch.Generator().manual_seed(T + E)
+    logits = torch.randn(T, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.1
+    cfg = terrace.TRouteConfig(E, Ng, k, M)
+    e, gt, grp = terrace.t_route(logits.to(DEV), bias.to(DEV), cfg, _force_generic=generic)
+    oe, og, ogrp = orc.t_route(logits.numpy(), bias.numpy(), E, Ng, k, M)
+    same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
+    # sigmoid affinities with a separate gate table
+    aff = torch.sigmoid(logits)
+    gate_tab = torch.exp(logits - logits.max(-1, keepdim=True).values)
+    e, gt, grp = terrace.t_route(aff.to(DEV), bias.to(DEV), cfg, gate_affinity=gate_tab.to(DEV),
+                                 _force_generic=generic)
+    oe, og, ogrp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, gate_affinity=gate_tab.numpy())
+    same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
+
+
+@pytest.mark.parametrize("generic", [False, True])
+def test_route_ties_and_pool(generic):
+    import terrace
+    announce("route ties", generic)
+    aff = torch.full((5, 64), 0.5)
+    aff[1, 10] = 0.75
+    aff[2, 63] = 0.25
+    aff[3] = torch.arange(64).float().div(64).roll(7)
+    aff[4, ::2] = 0.125
+    zero = torch.zeros(64)
+    for pool in (1, 2):
+        cfg = terrace.TRouteConfig(64, 8, 8, 4, group_score_pool=pool)
+        e, gt, grp = terrace.t_route(aff.to(DEV), zero.to(DEV), cfg, _force_generic=generic)
+        oe, og, ogrp = orc.t_route(aff.numpy(), zero.numpy(), 64, 8, 8, 4, pool=pool)
+        same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
+    assert to_np(e)[0].tolist() == [0, 1, 8, 9, 16, 17, 24, 25]
+
+
+@pytest.mark.parametrize("mode", ["group_limited", "quota_only", "global_topk"])
+def test_route_other_modes(mode):
+    import terrace
+    announce("route mode", mode)
+    g = torch.Generator().manual_seed(11)
+    for (T, E, Ng, k, M) in [(300, 64, 8, 8, 4), (77, 32, 4, 8, 2), (50, 256, 8, 8, 4)]:
+        aff = torch.rand(T, E, generator=g)
+        bias = torch.randn(E, generator=g) * 0.05
+        cfg = terrace.TRouteConfig(E, Ng, k, M)
+        e, gt, grp = terrace.t_route(aff.to(DEV), bias.to(DEV), cfg, mode=mode)
+        oe, og, ogrp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, mode=mode)
+        same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
+
+
+def test_expert_load_and_hist_and_argsort():
+    import terrace
+    from terrace.ta2a_fwd import _stable_argsort_small, fixed_hist
+    announce("hist/argsort")
+    rng = np.random.default_rng(3)
+    for n, nb in [(0, 8), (1, 8), (100, 8), (24576, 8), (300000, 32), (5000, 256), (70000, 1)]:
+        key = rng.integers(0, nb, n).astype(np.int64)
+        kd = torch.from_numpy(key).to(DEV)
+        same(fixed_hist(kd, nb), orc.fixed_hist(key, nb), "fixed_hist")
+        same(_stable_argsort_small(kd, nb), orc.stable_argsort_small(key, nb), "argsort")
+    e = rng.integers(0, 64, (4096, 8)).astype(np.int64)
+    same(terrace.expert_load(torch.from_numpy(e).to(DEV), 64), orc.expert_load(e, 64), "expert_load")
+
+
+# ------------------------------------------------------------------------------- plan + pack
+
+def _k2_case(world, rpn, E, T, k, M, fmt, sort_rows, seed, H=16):
+    n_nodes = world // rpn
+    e = equal_quota_routing(T, k, E, n_nodes, M, seed, sort_rows)
+    g = torch.Generator().manual_seed(seed)
+    hidden = rows_of(torch.randn(T, H, generator=g), fmt)
+    gates = rows_of(torch.rand(T, k, generator=g), fmt)
+    return e, hidden, gates
+
+
+@pytest.mark.parametrize("fmt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("sort_rows", [True, False])
+def test_k2_pack_reference_geometries(literals, fmt, sort_rows):
+    import terrace.ops as tops
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        for seed in (500, 501):
+            announce("k2", (world, rpn, E, T, k, M), fmt, sort_rows, seed)
+            e, hidden, gates = _k2_case(world, rpn, E, T, k, M, fmt, sort_rows, seed)
+            want = orc.k2_pack(to_np(hidden), e, to_np(gates), world, E, rpn, M)
+            ed = torch.from_numpy(e).to(DEV)
+            got, ex = tops.k2_pack_raw(hidden.to(DEV), ed, gates.to(DEV), world, E, rpn, M, extras=True)
+            for name, a, b in zip(("payload", "mask", "gate_rows", "u_src", "node_counts"), got, want):
+                same(a, b, name)
+            assert got[0].dtype == hidden.dtype and got[2].dtype == gates.dtype
+            u_src, u_node, counts, inverse = orc.plan_ta2a(e, world, E, rpn, M)
+            same(ex["u_node"], u_node, "u_node"), same(ex["inverse"], inverse, "inverse")
+            same(ex["node_offsets"], orc.send_offsets(counts), "node_offsets")
+            pair_tab, order = orc.token_pair_table(e, inverse, k // M)
+            same(ex["pair_table"], pair_tab, "pair_table"), same(ex["sort_order"], order, "sort_order")
+            same(ex["token_rows"], pair_tab[:, ::k // M] // (k // M), "token_rows")
+            same(ex["gate_sorted"], np.take_along_axis(to_np(gates), order, 1), "gate_sorted")
+            assert ex["status"].tolist() == [0, T * M, 0, 0]
+            # the registered torch op is the same call
+            for a, b in zip(torch.ops.terrace.k2_pack(hidden.to(DEV), ed, gates.to(DEV), world, E, rpn, M), got):
+                assert torch.equal(a, b)
+
+
+def test_plan_and_wire_functions_match_oracle(literals):
+    from terrace import ta2a
+    from terrace.ta2a_fwd import _pack_quota_wire
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        announce("plan", (world, rpn, E, T, k, M))
+        ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+        e, hidden, gates = _k2_case(world, rpn, E, T, k, M, "bf16", False, 900)
+        ed = torch.from_numpy(e).to(DEV)
+        got = ta2a.plan_ta2a(ed, world, E, rpn, groups_m=M)
+        want = orc.plan_ta2a(e, world, E, rpn, M)
+        for name, a, b in zip(("u_src", "u_node", "counts", "inverse"), got, want):
+            same(a, b, name)
+        slots = (E // world) * rpn
+        payload = hidden.to(DEV)[got[0]]
+        st, gt = _pack_quota_wire(ed, gates.to(DEV), got[3], payload, T * M, slots, k // M, E)
+        ws, wg = orc.pack_quota_wire(e, to_np(gates), want[3], T * M, slots, k // M)
+        same(st, ws, "slot_tab"), same(gt, wg, "gate_tab")
+        with pytest.raises(RuntimeError, match="dtype"):
+            _pack_quota_wire(ed, gates.float().to(DEV), got[3], payload, T * M, slots, k // M, E)
+        stats = ta2a.dispatch_stats(ed, world, E, rpn, groups_m=M)
+        assert stats["rows_ta2a"] == T * M and stats["rows_baseline"] == T * k
+
+
+def test_plan_guard_literal_cases(literals):
+    from terrace import ta2a
+    lit = literals["plan_quota_guard"]
+    geo = lit["geometry"]
+    for case in lit["cases"]:
+        announce("guard", case["name"])
+        ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+        idx = torch.tensor([case["expert_idx_row"]] * case["repeat"], device=DEV)
+        if case["raises"]:
+            with pytest.raises(ValueError, match=case["raises"]):
+                ta2a.plan_ta2a(idx, geo["world"], geo["n_experts"], geo["rpn"], groups_m=case["groups_m"])
+        else:
+            u_src, _, counts, _ = ta2a.plan_ta2a(idx, geo["world"], geo["n_experts"], geo["rpn"],
+                                                 groups_m=case["groups_m"])
+            assert u_src.numel() == case["n_rows"] and int(counts.sum()) == case["counts_sum"]
+    # group_limited routing has exact fan-out without quota: refused, not corrupted
+    import terrace
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    g = torch.Generator().manual_seed(5)
+    aff = torch.rand(256, 8, generator=g).to(DEV)
+    cfg = terrace.TRouteConfig(8, 2, 4, 2)
+    e, _, _ = terrace.t_route(aff, torch.zeros(8, device=DEV), cfg, mode="group_limited")
+    with pytest.raises(ValueError):
+        ta2a.plan_ta2a(e, 4, 8, 2, groups_m=2)
+    # and the guard sleeps between its periodic checks, as documented
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    good = torch.tensor([[0, 2, 4, 6]] * 4, device=DEV)
+    ta2a.plan_ta2a(good, 4, 8, 2, groups_m=2)
+    bad = torch.tensor([[0, 2, 3, 5]] * 4, device=DEV)
+    ta2a.plan_ta2a(bad, 4, 8, 2, groups_m=2)              # call 2 of this shape: unchecked
+    ta2a._VERIFY_COUNT[(4, 4, 2, 2)] = 256
+    with pytest.raises(ValueError, match="quota"):
+        ta2a.plan_ta2a(bad, 4, 8, 2, groups_m=2)
+
+
+def test_hopa_send_splits_literal(literals):
+    import terrace.ops as tops
+    lit = literals["hopa_counts"]
+    send = tops.hopa_send_splits(torch.tensor(lit["node_counts"], device=DEV), lit["world"], lit["rpn"],
+                                 lit["my_local"])
+    assert send.dtype == torch.int64 and send.tolist() == lit["send"]
+
+
+# ------------------------------------------------------------------------------- arrival
+
+@pytest.mark.parametrize("fmt", ["f32", "bf16", "f16"])
+def test_k1_arrival_reference_geometries(literals, fmt):
+    import terrace.ops as tops
+    for R, q, epr, rpn, H in literals["k1_geometries"]["rows"]:
+        for seed in (100, 101):
+            announce("k1", (R, q, epr, rpn, H), fmt, seed)
+            rslot = arrival_plane(R, q, epr, rpn, seed)
+            g = torch.Generator().manual_seed(seed)
+            rx = rows_of(torch.randn(R, H, generator=g), fmt)
+            rgate = rows_of(torch.rand(R, q, generator=g), fmt)
+            want = orc.k1_arrival(to_np(rx), rslot, to_np(rgate), q, epr, rpn)
+            got = tops.k1_arrival_raw(rx.to(DEV), torch.from_numpy(rslot).to(DEV), rgate.to(DEV), q, epr, rpn, 0,
+                                      want_pair_pos=True)
+            for name, a, b in zip(("send_buf", "gate_pairs", "r_idx", "slot_idx", "i_send"), got, want):
+                same(a, b, name)
+            same(got[5], orc.arrival_positions(rslot, epr, rpn), "pair_pos")
+            for a, b in zip(torch.ops.terrace.k1_arrival(rx.to(DEV), torch.from_numpy(rslot).to(DEV),
+                                                         rgate.to(DEV), q, epr, rpn, 0), got):
+                assert torch.equal(a, b)
+
+
+def test_k1_arrival_degenerate_empty_and_large(literals):
+    import terrace.ops as tops
+    d = literals["k1_degenerate"]["all_zero_slot_rows"]
+    announce("k1 degenerate")
+    rslot = arrival_plane(d["R"], d["quota"], d["epr"], d["rpn"], 5, degenerate=True)
+    g = torch.Generator().manual_seed(5)
+    rx, rgate = torch.randn(d["R"], d["H"], generator=g), torch.rand(d["R"], d["quota"], generator=g)
+    want = orc.k1_arrival(rx.numpy(), rslot, rgate.numpy(), d["quota"], d["epr"], d["rpn"])
+    got = tops.k1_arrival(rx.to(DEV), torch.from_numpy(rslot).to(DEV), rgate.to(DEV), d["quota"], d["epr"], d["rpn"])
+    for name, a, b in zip(("send_buf", "gate_pairs", "r_idx", "slot_idx", "i_send"), got, want):
+        same(a, b, name)
+    z = literals["k1_degenerate"]["empty_arrival"]
+    announce("k1 empty")
+    got = tops.k1_arrival(torch.zeros(0, z["H"], device=DEV), torch.zeros(0, z["quota"], dtype=torch.int64, device=DEV),
+                          torch.zeros(0, z["quota"], device=DEV), z["quota"], z["epr"], z["rpn"])
+    assert got[0].shape == (0, z["H"]) and got[4].shape == (z["rpn"],) and int(got[4].sum()) == z["i_send_sum"]
+    announce("k1 large, many units")
+    R, q, epr, rpn, H = 150001, 2, 4, 8, 64
+    rslot = arrival_plane(R, q, epr, rpn, 9)
+    rx = torch.randn(R, H, generator=g).bfloat16()
+    rgate = torch.rand(R, q, generator=g).bfloat16()
+    want = orc.k1_arrival(to_np(rx), rslot, to_np(rgate), q, epr, rpn)
+    got = tops.k1_arrival(rx.to(DEV), torch.from_numpy(rslot).to(DEV), rgate.to(DEV), q, epr, rpn)
+    for name, a, b in zip(("send_buf", "gate_pairs", "r_idx", "slot_idx", "i_send"), got, want):
+        same(a, b, name)
+
+
+def test_k1_out_of_range_slot_is_contained_and_reported():
+    import terrace.ops as tops
+    from terrace import _hip
+    announce("k1 bad slot")
+    rslot = torch.tensor([[0, 3], [1, 99], [2, 5]], device=DEV)
+    st = _hip.new_status(DEV)
+    out = tops.k1_arrival_raw(torch.randn(3, 8, device=DEV), rslot, torch.rand(3, 2, device=DEV), 2, 2, 4, 0,
+                              status_out=st)
+    assert st.tolist()[0] & _hip.FAULT_ID_RANGE
+    assert int(out[4].sum()) == 6 and sorted(out[2].tolist()) == [0, 0, 1, 1, 2, 2]
+
+
+def test_k1_backward_is_the_gather_adjoint():
+    import terrace.ops as tops
+    announce("k1 backward")
+    R, q, epr, rpn, H = 12, 2, 2, 4, 8
+    rslot = arrival_plane(R, q, epr, rpn, 9)
+    g = torch.Generator().manual_seed(1)
+    rx0, rg0 = torch.randn(R, H, generator=g), torch.rand(R, q, generator=g)
+    gs, gg = torch.randn(R * q, H, generator=g), torch.randn(R * q, generator=g)
+    _, _, r_idx, _, _ = orc.k1_arrival(rx0.numpy(), rslot, rg0.numpy(), q, epr, rpn)
+    pos = orc.arrival_positions(rslot, epr, rpn)
+    want_rx = orc.gather_reduce(gs.numpy(), pos.reshape(R, q), None)
+    want_rg = gg.numpy()[pos].reshape(R, q)
+    for fn in (tops.k1_arrival, tops.k1_arrival_segment):
+        rx, rg = rx0.to(DEV).requires_grad_(True), rg0.to(DEV).requires_grad_(True)
+        s, p, *_ = fn(rx, torch.from_numpy(rslot).to(DEV), rg, q, epr, rpn)
+        ((s * gs.to(DEV)).sum() + (p * gg.to(DEV)).sum()).backward()
+        same(rx.grad, want_rx, "grad_rx"), same(rg.grad, want_rg, "grad_rgate")
+
+
+# ------------------------------------------------------------------------------- regroup
+
+@pytest.mark.parametrize("P,epr,my_local,H,fmt", [(7, 4, 1, 3, "f32"), (1000, 4, 0, 16, "bf16"), (30000, 32, 0, 64, "bf16"),
+                                                  (513, 1, 5, 8, "f16"), (4097, 63, 2, 24, "f32")])
+def test_regroup_dropless_and_capacity(P, epr, my_local, H, fmt):
+    import terrace.ops as tops
+    announce("regroup", P, epr, my_local, H, fmt)
+    rng = np.random.default_rng(P)
+    my_slot = (rng.integers(0, epr, P) + my_local * epr).astype(np.int64)
+    if P == 7:
+        my_slot = np.array([5, 4, 5, 5, 4, 7, 5], dtype=np.int64)
+    g = torch.Generator().manual_seed(P)
+    rows = rows_of(torch.randn(P, H, generator=g), fmt)
+    gate = rows_of(torch.rand(P, generator=g), fmt)
+    sd = torch.from_numpy(my_slot).to(DEV)
+    permuted, order, tpe, pgate = tops.regroup(rows.to(DEV), sd, epr, my_local, my_gate=gate.to(DEV))
+    wp, wo, wt = orc.regroup(to_np(rows), my_slot, epr, my_local)
+    same(permuted, wp, "permuted"), same(order, wo, "order"), same(tpe, wt, "tokens_per_expert")
+    same(pgate, to_np(gate)[wo], "permuted_gate")
+    mean = max(P // epr, 1)
+    for cap in (0, 1, mean, int(mean * 1.25) + 1, P + 3):
+        padded, dest, kept, tpe, kpe, pg = tops.regroup(rows.to(DEV), sd, epr, my_local, capacity=cap,
+                                                        my_gate=gate.to(DEV))
+        wpad, wdest, wkept, wt, wk = orc.regroup(to_np(rows), my_slot, epr, my_local, capacity=cap)
+        same(padded, wpad, f"padded cap={cap}"), same(dest, wdest, "dest"), same(kept, wkept, "kept")
+        same(tpe, wt, "tokens_per_expert"), same(kpe, wk, "kept_per_expert")
+        wg = np.zeros(epr * cap, dtype=to_np(gate).dtype)
+        wg[wdest[wkept]] = to_np(gate)[wkept]
+        same(pg, wg, "padded_gate")
+
+
+def test_regroup_empty():
+    import terrace.ops as tops
+    announce("regroup empty")
+    permuted, order, tpe = tops.regroup(torch.zeros(0, 8, device=DEV), torch.zeros(0, dtype=torch.int64, device=DEV), 4)
+    assert permuted.shape == (0, 8) and order.numel() == 0 and tpe.tolist() == [0, 0, 0, 0]
+    padded, dest, kept, tpe, kpe = tops.regroup(torch.zeros(0, 8, device=DEV),
+                                                torch.zeros(0, dtype=torch.int64, device=DEV), 4, capacity=3)
+    assert padded.shape == (12, 8) and not padded.any() and kpe.tolist() == [0, 0, 0, 0]
+
+
+# ------------------------------------------------------------------------------- combine
+
+@pytest.mark.parametrize("src_fmt,out_fmt,H", [("f32", "f32", 1024), ("bf16", "bf16", 7168), ("bf16", "f32", 512),
+                                               ("f16", "f16", 256), ("f32", "bf16", 64), ("bf16", "bf16", 24),
+                                               ("f32", "f32", 6), ("f16", "f32", 13)])
+@pytest.mark.parametrize("fan", [1, 2, 3, 4, 8, 11])
+def test_combine_bit_exact_and_within_tolerance(src_fmt, out_fmt, H, fan):
+    import terrace.ops as tops
+    announce("combine", src_fmt, out_fmt, H, fan)
+    n_src, n_out = 300, 97
+    g = torch.Generator().manual_seed(H + fan)
+    src = rows_of(torch.randn(n_src, H, generator=g), src_fmt)
+    idx = torch.randint(0, n_src, (n_out, fan), generator=g)
+    idx[5, 0] = -1
+    idx[6, :] = -1
+    for wfmt in (None, "f32", src_fmt):
+        w = None if wfmt is None else rows_of(torch.rand(n_out, fan, generator=g), wfmt)
+        got = tops.combine(src.to(DEV), idx.to(DEV), None if w is None else w.to(DEV), out_dtype=DT[out_fmt])
+        wf = None if w is None else orc.decode_rows(to_np(w), wfmt)
+        want = orc.combine(to_np(src), idx.numpy(), wf, src_fmt, out_fmt)
+        same(got, want, f"combine w={wfmt}")
+        # the stated tolerance, against float64
+        ok = idx.numpy() >= 0
+        s64 = orc.decode_rows(to_np(src), src_fmt).astype(np.float64)
+        w64 = np.ones((n_out, fan)) if wf is None else wf.astype(np.float64)
+        ref = sum(np.where(ok[:, j:j + 1], s64[np.where(ok[:, j], idx.numpy()[:, j], 0)] * w64[:, j:j + 1], 0.0)
+                  for j in range(fan))
+        tol = 1e-5 if out_fmt == "f32" else 1e-2
+        scale = np.abs(ref).max() + 1e-30
+        assert np.abs(orc.decode_rows(to_np(got), out_fmt) - ref).max() <= tol * scale * (2 if out_fmt == "f16" else 1)
+
+
+def test_combine_fp8_rows():
+    import terrace.ops as tops
+    announce("combine fp8")
+    for H in (512, 7168, 384):
+        g = torch.Generator().manual_seed(H)
+        x = torch.randn(64, H, generator=g) * 3
+        rows = orc.fp8_quantise_rows(x.numpy())
+        idx = torch.randint(0, 64, (33, 8), generator=g)
+        w = torch.rand(33, 8, generator=g)
+        for out_fmt in ("bf16", "f32"):
+            got = tops.combine(torch.from_numpy(rows).to(DEV), idx.to(DEV), w.to(DEV), out_dtype=DT[out_fmt],
+                               fp8_hidden=H)
+            want = orc.combine(rows, idx.numpy(), w.numpy(), "fp8", out_fmt, hidden=H)
+            same(got, want, f"fp8 H={H} {out_fmt}")
+    # every e4m3 code decodes as the table says
+    codes = np.arange(256, dtype=np.uint8)
+    codes = codes[~np.isnan(orc.E4M3)]
+    row = np.zeros((1, 256 + 8), dtype=np.uint8)
+    row[0, :codes.size] = codes
+    row[0, 256:] = np.array([1.0, 1.0], dtype=np.float32).view(np.uint8)
+    got = tops.combine(torch.from_numpy(row).to(DEV), torch.zeros(1, 1, dtype=torch.int64, device=DEV), None,
+                       out_dtype=torch.float32, fp8_hidden=256)
+    assert np.array_equal(to_np(got)[0, :codes.size], orc.E4M3[codes])
+
+
+def test_gather_rows_and_index_chain():
+    import terrace.ops as tops
+    announce("gather/index_chain")
+    g = torch.Generator().manual_seed(4)
+    for H, dt in [(7168, torch.bfloat16), (1024, torch.float32), (7392, torch.uint8), (5, torch.float16), (3, torch.uint8)]:
+        src = torch.randint(0, 255, (50, H), generator=g, dtype=torch.uint8) if dt == torch.uint8 else \
+            torch.randn(50, H, generator=g).to(dt)
+        idx = torch.randint(0, 50, (200,), generator=g)
+        idx[3] = -1
+        out = tops.gather_rows(src.to(DEV), idx.to(DEV)).cpu()
+        want = src[idx.clamp(min=0)]
+        want[3] = 0
+        assert torch.equal(out, want)
+    table = torch.randint(-1, 100, (100,), generator=g)
+    idx = torch.randint(-1, 100, (4, 7), generator=g)
+    want = torch.where(idx < 0, torch.full_like(idx, -1), table[idx.clamp(min=0)])
+    assert torch.equal(tops.index_chain(table.to(DEV), idx.to(DEV)).cpu(), want)
