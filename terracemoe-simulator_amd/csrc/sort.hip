@@ -609,13 +609,13 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
         (gate_bytes != 2 && gate_bytes != 4) || P >= (int64_t)1 << 31 ||
         (capacity >= 0 && (int64_t)epr * capacity >= (int64_t)1 << 31))
         return TERRACE_EINVAL;
-    if ((node_rx && !permuted) || (my_gate && !permuted_gate)) return TERRACE_EINVAL;
     const int64_t places = capacity >= 0 ? (int64_t)epr * capacity : P;
+    if (places > 0 && ((node_rx && !permuted) || (my_gate && !permuted_gate))) return TERRACE_EINVAL;
     if (P == 0) {
         int rc = empty_outputs(tokens_per_expert, nullptr, kept_per_expert, epr, status, s);
         if (rc != TERRACE_OK || places == 0) return rc;
-        if (node_rx && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
-        if (my_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
+        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        if (permuted_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
         return check_launch();
     }
     if (!my_slot || !ws) return TERRACE_EINVAL;
