@@ -172,6 +172,12 @@ TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, con
 TERRACE_API int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes,
                         void *out, terrace_stream_t stream);
 
+/* dst[pos[r*fan + f]] = src[r] for r < n_src, f < fan (pos < 0 skips that copy): a source row
+ * is read once and written fan times.  The mover behind terrace_k2_pack (pos = token_rows)
+ * and terrace_k1_arrival (pos = pair_pos); exposed so it can be driven and timed on its own. */
+TERRACE_API int terrace_scatter_rows(const void *src, const int64_t *pos, int64_t n_src, int fan,
+                                     int64_t row_bytes, void *dst, terrace_stream_t stream);
+
 /* out[i] = table[idx[i]] over int64 planes; idx < 0 or table value < 0 gives -1. */
 TERRACE_API int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out,
                         terrace_stream_t stream);

@@ -8,6 +8,9 @@ int launch_combine(const void *src, int src_dtype, const int64_t *idx, const voi
 int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
 int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s);
 template <typename I>
+int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
+                        hipStream_t s);
+template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
 int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
                 int k, int M, int pool, int mode, int64_t *expert_idx, float *gates, int64_t *group_idx,
@@ -133,6 +136,13 @@ int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int6
     if (n_out < 0 || row_bytes < 0) return TERRACE_EINVAL;
     if (n_out && row_bytes && (!src || !idx || !out)) return TERRACE_EINVAL;
     return launch_gather_rows<int64_t>(src, out, idx, n_out, row_bytes, (hipStream_t)stream);
+}
+
+int terrace_scatter_rows(const void *src, const int64_t *pos, int64_t n_src, int fan, int64_t row_bytes, void *dst,
+                         terrace_stream_t stream) {
+    if (n_src < 0 || fan <= 0 || row_bytes < 0) return TERRACE_EINVAL;
+    if (n_src && row_bytes && (!src || !pos || !dst)) return TERRACE_EINVAL;
+    return launch_scatter_rows<int64_t>(src, dst, pos, n_src, fan, row_bytes, (hipStream_t)stream);
 }
 
 int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream) {

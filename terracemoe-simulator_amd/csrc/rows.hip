@@ -50,9 +50,9 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V
 // ---------------------------------------------------------------------------------------------
 // scatter: one read, fan writes
 // ---------------------------------------------------------------------------------------------
-template <typename V, int VPT>
+template <typename V, int VPT, typename I>
 __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restrict__ src, V *__restrict__ dst,
-                                                              const int32_t *__restrict__ pos, int64_t n_src,
+                                                              const I *__restrict__ pos, int64_t n_src,
                                                               int fan, int64_t row_vecs, int tpr_log2) {
     const int tpr = 1 << tpr_log2;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restric
     for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_src;
          row += (int64_t)gridDim.x * rows_per_iter) {
         const V *s = src + row * row_vecs;
-        const int32_t *p = pos + row * fan;
+        const I *p = pos + row * fan;
         for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
             V v[VPT];
 #pragma unroll
@@ -342,32 +342,35 @@ static int vec_bytes_for(int64_t row_bytes, const void *a, const void *b) {
     return 1;
 }
 
-template <typename V>
-static void launch_scatter_t(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan,
+template <typename V, typename I>
+static void launch_scatter_t(const void *src, void *dst, const I *pos, int64_t n_src, int fan,
                              int64_t row_vecs, hipStream_t s) {
     const int l = tpr_log2_for(row_vecs);
     const int rpi = kBlock >> l;
     const int grid = grid_for(n_src, rpi);
     if (row_vecs > ((int64_t)2 << l))
-        scatter_rows_kernel<V, 4><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
     else if (row_vecs > ((int64_t)1 << l))
-        scatter_rows_kernel<V, 2><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
     else
-        scatter_rows_kernel<V, 1><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
 }
 
-int launch_scatter_rows(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan, int64_t row_bytes,
+template <typename I>
+int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
                         hipStream_t s) {
     if (n_src <= 0 || row_bytes <= 0 || fan <= 0) return TERRACE_OK;
     switch (vec_bytes_for(row_bytes, src, dst)) {
-        case 16: launch_scatter_t<u32x4>(src, dst, pos, n_src, fan, row_bytes / 16, s); break;
-        case 8: launch_scatter_t<u32x2>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
-        case 4: launch_scatter_t<uint32_t>(src, dst, pos, n_src, fan, row_bytes / 4, s); break;
-        case 2: launch_scatter_t<uint16_t>(src, dst, pos, n_src, fan, row_bytes / 2, s); break;
-        default: launch_scatter_t<uint8_t>(src, dst, pos, n_src, fan, row_bytes, s); break;
+        case 16: launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, row_bytes / 16, s); break;
+        case 8: launch_scatter_t<u32x2, I>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
+        case 4: launch_scatter_t<uint32_t, I>(src, dst, pos, n_src, fan, row_bytes / 4, s); break;
+        case 2: launch_scatter_t<uint16_t, I>(src, dst, pos, n_src, fan, row_bytes / 2, s); break;
+        default: launch_scatter_t<uint8_t, I>(src, dst, pos, n_src, fan, row_bytes, s); break;
     }
     return check_launch();
 }
+template int launch_scatter_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int, int64_t, hipStream_t);
+template int launch_scatter_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int, int64_t, hipStream_t);
 
 template <typename V, typename I>
 static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_vecs,

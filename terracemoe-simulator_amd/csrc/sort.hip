@@ -510,7 +510,8 @@ __global__ __launch_bounds__(kBlock) void pack_quota_wire_kernel(const int64_t *
 // ---------------------------------------------------------------------------------------------
 // host drivers
 // ---------------------------------------------------------------------------------------------
-int launch_scatter_rows(const void *src, void *dst, const int32_t *pos, int64_t n_src, int fan, int64_t row_bytes,
+template <typename I>
+int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
                         hipStream_t s);
 template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
@@ -590,7 +591,7 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
     EmitArrival emit{rslot, rgate, gate_bytes, quota, gate_pairs, r_idx, slot_idx, pair_pos, pos32};
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, 1, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
-    return launch_scatter_rows(rx, send_buf, pos32, R, quota, row_bytes, s);
+    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
 }
 
 // ---- expert-order regroup ---------------------------------------------------------------------
@@ -692,7 +693,7 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
                         pos32};
     int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, 1, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
-    return launch_scatter_rows(hidden, payload, pos32, T, groups_m, row_bytes, s);
+    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
 }
 
 int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,

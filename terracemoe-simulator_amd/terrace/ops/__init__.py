@@ -294,6 +294,24 @@ def gather_rows(src, idx):
     return out
 
 
+def scatter_rows(src, pos, n_dst):
+    """``dst[pos[r, f]] = src[r]``: each source row is read once and written ``pos.shape[1]``
+    times (negative places are skipped).  ``dst`` has ``n_dst`` rows; rows no place names are
+    left uninitialised."""
+    _require()
+    _hip.need_device(src, pos)
+    src, pos = src.contiguous(), pos.contiguous()
+    if pos.dtype != torch.int64 or pos.dim() != 2 or pos.shape[0] != src.shape[0]:
+        raise RuntimeError("scatter_rows: pos must be int64 [n_src, fan]")
+    dst = torch.empty((n_dst,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+    row_bytes = src.element_size()
+    for d in src.shape[1:]:
+        row_bytes *= int(d)
+    _hip.call("terrace_scatter_rows", _hip.ptr(src), _hip.ptr(pos), src.shape[0], pos.shape[1], row_bytes,
+              _hip.ptr(dst), _hip.stream(src.device))
+    return dst
+
+
 def index_chain(table, idx):
     """``table[idx]`` over int64 planes (negative entries propagate as -1)."""
     _require()
@@ -545,5 +563,5 @@ def k2_pack(hidden, expert_idx, gates, world: int, n_experts: int, rpn: int, gro
 __all__ = [
     "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
-    "regroup", "combine", "gather_rows", "index_chain", "hist", "argsort_small", "hopa_send_splits",
+    "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "hist", "argsort_small", "hopa_send_splits",
 ]
