@@ -57,27 +57,25 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restric
     const int tpr = 1 << tpr_log2;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
     const int lane = threadIdx.x & (tpr - 1);
-    const int rows_per_iter = kBlock >> tpr_log2;
-    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_src;
-         row += (int64_t)gridDim.x * rows_per_iter) {
-        const V *s = src + row * row_vecs;
-        const I *p = pos + row * fan;
-        for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
-            V v[VPT];
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> tpr_log2) + sub;
+    if (row >= n_src) return;
+    const V *s = src + row * row_vecs;
+    const I *p = pos + row * fan;
+    for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
+        V v[VPT];
+#pragma unroll
+        for (int u = 0; u < VPT; ++u) {
+            const int64_t i = base + (int64_t)u * tpr;
+            if (i < row_vecs) v[u] = ld_stream(s + i);
+        }
+        for (int f = 0; f < fan; ++f) {
+            const int64_t d = p[f];
+            if (d < 0) continue;
+            V *o = dst + d * row_vecs;
 #pragma unroll
             for (int u = 0; u < VPT; ++u) {
                 const int64_t i = base + (int64_t)u * tpr;
-                if (i < row_vecs) v[u] = ld_stream(s + i);
-            }
-            for (int f = 0; f < fan; ++f) {
-                const int64_t d = p[f];
-                if (d < 0) continue;
-                V *o = dst + d * row_vecs;
-#pragma unroll
-                for (int u = 0; u < VPT; ++u) {
-                    const int64_t i = base + (int64_t)u * tpr;
-                    if (i < row_vecs) st_stream(o + i, v[u]);
-                }
+                if (i < row_vecs) st_stream(o + i, v[u]);
             }
         }
     }
@@ -93,28 +91,26 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict
     const int tpr = 1 << tpr_log2;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
     const int lane = threadIdx.x & (tpr - 1);
-    const int rows_per_iter = kBlock >> tpr_log2;
-    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_out;
-         row += (int64_t)gridDim.x * rows_per_iter) {
-        const int64_t from = (int64_t)idx[row];
-        V *o = out + row * row_vecs;
-        if (from < 0) {
-            for (int64_t i = lane; i < row_vecs; i += tpr) st_stream(o + i, zero_of<V>());
-            continue;
+    const int64_t row = (int64_t)blockIdx.x * (kBlock >> tpr_log2) + sub;
+    if (row >= n_out) return;
+    const int64_t from = (int64_t)idx[row];
+    V *o = out + row * row_vecs;
+    if (from < 0) {
+        for (int64_t i = lane; i < row_vecs; i += tpr) st_stream(o + i, zero_of<V>());
+        return;
+    }
+    const V *s = src + from * row_vecs;
+    for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
+        V v[VPT];
+#pragma unroll
+        for (int u = 0; u < VPT; ++u) {
+            const int64_t i = base + (int64_t)u * tpr;
+            if (i < row_vecs) v[u] = ld_stream(s + i);
         }
-        const V *s = src + from * row_vecs;
-        for (int64_t base = lane; base < row_vecs; base += (int64_t)tpr * VPT) {
-            V v[VPT];
 #pragma unroll
-            for (int u = 0; u < VPT; ++u) {
-                const int64_t i = base + (int64_t)u * tpr;
-                if (i < row_vecs) v[u] = ld_stream(s + i);
-            }
-#pragma unroll
-            for (int u = 0; u < VPT; ++u) {
-                const int64_t i = base + (int64_t)u * tpr;
-                if (i < row_vecs) st_stream(o + i, v[u]);
-            }
+        for (int u = 0; u < VPT; ++u) {
+            const int64_t i = base + (int64_t)u * tpr;
+            if (i < row_vecs) st_stream(o + i, v[u]);
         }
     }
 }
@@ -203,65 +199,58 @@ __device__ __forceinline__ void store_chunk(void *out_row, int64_t first_elem, c
     }
 }
 
-// Vector path: rows are 16-byte aligned multiples of 16 bytes.
+// Vector path: rows are 16-byte aligned multiples of 16 bytes.  One thread owns one 16-byte
+// chunk of one output row: blockIdx.x = row * slices + slice, chunk = slice*256 + threadIdx.x.
 template <int SRC, int OUT, int FANC>
 __global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restrict__ src, int64_t src_row_bytes,
                                                          const int64_t *__restrict__ idx, const void *__restrict__ w,
                                                          int w_dtype, int64_t n_out, int fan, int64_t hidden,
                                                          uint8_t *__restrict__ out, int64_t out_row_bytes,
-                                                         int tpr_log2) {
+                                                         int slices) {
     constexpr int N = Chunk<SRC>::N;
-    const int tpr = 1 << tpr_log2;
-    const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
-    const int lane = threadIdx.x & (tpr - 1);
-    const int rows_per_iter = kBlock >> tpr_log2;
-    const int64_t chunks = hidden / N;
-    for (int64_t row = (int64_t)blockIdx.x * rows_per_iter + sub; row < n_out;
-         row += (int64_t)gridDim.x * rows_per_iter) {
-        uint8_t *out_row = out + row * out_row_bytes;
-        for (int64_t c = lane; c < chunks; c += tpr) {
-            float acc[N];
+    const int64_t row = blockIdx.x / slices;
+    const int64_t c = (int64_t)(blockIdx.x - row * slices) * kBlock + threadIdx.x;
+    if (c >= hidden / N) return;
+    float acc[N];
 #pragma unroll
-            for (int i = 0; i < N; ++i) acc[i] = 0.0f;
-            for (int j0 = 0; j0 < fan; j0 += FANC) {
-                u32x4 raw[FANC];
-                float wj[FANC], sc[FANC];
-                bool live[FANC];
+    for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+    for (int j0 = 0; j0 < fan; j0 += FANC) {
+        u32x4 raw[FANC];
+        float wj[FANC], sc[FANC];
+        bool live[FANC];
 #pragma unroll
-                for (int jj = 0; jj < FANC; ++jj) {
-                    const int j = j0 + jj;
-                    live[jj] = false;
-                    wj[jj] = 1.0f;
-                    sc[jj] = 1.0f;
-                    if (j < fan) {
-                        const int64_t from = idx[row * fan + j];
-                        if (from >= 0) {
-                            live[jj] = true;
-                            const uint8_t *s = src + from * src_row_bytes;
-                            raw[jj] = ld_stream((const u32x4 *)s + c);
-                            if constexpr (SRC == TERRACE_FP8_E4M3_B128)
-                                sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
-                            if (w) wj[jj] = load_weight(w, w_dtype, row * fan + j);
-                        }
-                    }
-                }
-#pragma unroll
-                for (int jj = 0; jj < FANC; ++jj) {
-                    if (!live[jj]) continue;
-                    float f[N];
-                    decode_chunk<SRC>(raw[jj], f);
-#pragma unroll
-                    for (int i = 0; i < N; ++i) {
-                        float x = f[i];
-                        if constexpr (SRC == TERRACE_FP8_E4M3_B128) x = __fmul_rn(x, sc[jj]);
-                        if (w) x = __fmul_rn(x, wj[jj]);
-                        acc[i] = __fadd_rn(acc[i], x);
-                    }
+        for (int jj = 0; jj < FANC; ++jj) {
+            const int j = j0 + jj;
+            live[jj] = false;
+            wj[jj] = 1.0f;
+            sc[jj] = 1.0f;
+            if (j < fan) {
+                const int64_t from = idx[row * fan + j];
+                if (from >= 0) {
+                    live[jj] = true;
+                    const uint8_t *s = src + from * src_row_bytes;
+                    raw[jj] = ld_stream((const u32x4 *)s + c);
+                    if constexpr (SRC == TERRACE_FP8_E4M3_B128)
+                        sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
+                    if (w) wj[jj] = load_weight(w, w_dtype, row * fan + j);
                 }
             }
-            store_chunk<OUT, N>(out_row, c * N, acc);
+        }
+#pragma unroll
+        for (int jj = 0; jj < FANC; ++jj) {
+            if (!live[jj]) continue;
+            float f[N];
+            decode_chunk<SRC>(raw[jj], f);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                float x = f[i];
+                if constexpr (SRC == TERRACE_FP8_E4M3_B128) x = __fmul_rn(x, sc[jj]);
+                if (w) x = __fmul_rn(x, wj[jj]);
+                acc[i] = __fadd_rn(acc[i], x);
+            }
         }
     }
+    store_chunk<OUT, N>(out + row * out_row_bytes, c * N, acc);
 }
 
 // Element path: any hidden, any alignment.
@@ -320,10 +309,13 @@ __global__ void send_splits_kernel(const int64_t *__restrict__ node_counts, int 
 // ---------------------------------------------------------------------------------------------
 // host-side launch helpers
 // ---------------------------------------------------------------------------------------------
-static int grid_for(int64_t n_rows, int rows_per_iter) {
-    const int64_t need = (n_rows + rows_per_iter - 1) / rows_per_iter;
-    const int64_t cap = 256 * 16;               // 256 CUs, up to 16 resident workgroups' worth of rows each
-    return (int)(need < 1 ? 1 : (need > cap ? cap : need));
+// One sub-group per row and no grid-stride loop: many short workgroups stream measurably
+// faster on this part than a resident grid walking the rows.
+constexpr int64_t kMaxGridRows = (int64_t)1 << 30;   // keeps every launch below HIP's 2^31 - 1 blocks
+
+static unsigned grid_for(int64_t n_rows, int rows_per_block) {
+    const int64_t need = (n_rows + rows_per_block - 1) / rows_per_block;
+    return (unsigned)(need < 1 ? 1 : need);
 }
 
 // Lanes per row: enough that a lane holds about 4 vectors, at least one wave, at most the block.
@@ -347,7 +339,7 @@ static void launch_scatter_t(const void *src, void *dst, const I *pos, int64_t n
                              int64_t row_vecs, hipStream_t s) {
     const int l = tpr_log2_for(row_vecs);
     const int rpi = kBlock >> l;
-    const int grid = grid_for(n_src, rpi);
+    const unsigned grid = grid_for(n_src, rpi);
     if (row_vecs > ((int64_t)2 << l))
         scatter_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
     else if (row_vecs > ((int64_t)1 << l))
@@ -360,6 +352,7 @@ template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
                         hipStream_t s) {
     if (n_src <= 0 || row_bytes <= 0 || fan <= 0) return TERRACE_OK;
+    if (n_src > kMaxGridRows) return TERRACE_EINVAL;
     switch (vec_bytes_for(row_bytes, src, dst)) {
         case 16: launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, row_bytes / 16, s); break;
         case 8: launch_scatter_t<u32x2, I>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
@@ -377,7 +370,7 @@ static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_
                             hipStream_t s) {
     const int l = tpr_log2_for(row_vecs);
     const int rpi = kBlock >> l;
-    const int grid = grid_for(n_out, rpi);
+    const unsigned grid = grid_for(n_out, rpi);
     if (row_vecs > ((int64_t)2 << l))
         gather_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
     else if (row_vecs > ((int64_t)1 << l))
@@ -389,6 +382,7 @@ static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_
 template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s) {
     if (n_out <= 0 || row_bytes <= 0) return TERRACE_OK;
+    if (n_out > kMaxGridRows) return TERRACE_EINVAL;
     switch (vec_bytes_for(row_bytes, src, out)) {
         case 16: launch_gather_t<u32x4, I>(src, out, idx, n_out, row_bytes / 16, s); break;
         case 8: launch_gather_t<u32x2, I>(src, out, idx, n_out, row_bytes / 8, s); break;
@@ -415,14 +409,12 @@ template <int SRC, int OUT>
 static void launch_combine_so(const void *src, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
                               int fan, int64_t hidden, void *out, hipStream_t s) {
     const int64_t chunks = hidden / Chunk<SRC>::N;
-    int l = 6;
-    while (l < 8 && ((int64_t)2 << l) < chunks) ++l;
-    const int rpi = kBlock >> l;
-    const int grid = grid_for(n_out, rpi);
+    const int slices = (int)((chunks + kBlock - 1) / kBlock);
+    const unsigned grid = (unsigned)(n_out * slices);
     const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
 #define TERRACE_COMBINE_LAUNCH(F)                                                                          \
     combine_kernel<SRC, OUT, F><<<grid, kBlock, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, \
-                                                        fan, hidden, (uint8_t *)out, orb, l)
+                                                        fan, hidden, (uint8_t *)out, orb, slices)
     if (fan >= 8) TERRACE_COMBINE_LAUNCH(8);
     else if (fan >= 4) TERRACE_COMBINE_LAUNCH(4);
     else if (fan >= 2) TERRACE_COMBINE_LAUNCH(2);
@@ -441,6 +433,7 @@ static void launch_combine_s(const void *src, const int64_t *idx, const void *w,
 int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
                    int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
     if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
+    if (n_out * ((hidden + 1023) / 1024 + 1) > kMaxGridRows) return TERRACE_EINVAL;
     const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
     const int n = src_dtype == TERRACE_F32 ? 4 : (src_dtype == TERRACE_FP8_E4M3_B128 ? 16 : 8);
     const bool vec = hidden % n == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
@@ -465,9 +458,8 @@ int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s) {
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)y | (uintptr_t)nbytes;
     if ((bits & 15) == 0) {
         const int64_t n = (int64_t)(nbytes / 16);
-        int64_t blocks = (n + kBlock * 4 - 1) / (kBlock * 4);
-        if (blocks > 256 * 16) blocks = 256 * 16;
-        copy_kernel<u32x4, 4><<<(int)blocks, kBlock, 0, s>>>((const u32x4 *)x, (u32x4 *)y, n);
+        const int64_t blocks = (n + kBlock - 1) / kBlock;
+        copy_kernel<u32x4, 1><<<(unsigned)blocks, kBlock, 0, s>>>((const u32x4 *)x, (u32x4 *)y, n);
     } else {
         const int64_t n = (int64_t)nbytes;
         int64_t blocks = (n + kBlock * 4 - 1) / (kBlock * 4);

@@ -21,7 +21,7 @@ constexpr int kScanThreads = 1024;
 
 struct Units {
     int64_t n_items;
-    int chunks;       // 64-item chunks per unit
+    int chunks;       // 64-item chunks per unit: 4, or 16 for more than a million items
     int n_units;
     int n_buckets;
 };
@@ -30,10 +30,8 @@ Units make_units(int64_t n_items, int n_buckets) {
     Units u;
     u.n_items = n_items;
     u.n_buckets = n_buckets;
-    int64_t ch = 4;
-    while ((n_items + 64 * ch - 1) / (64 * ch) > 4096) ch *= 2;
-    u.chunks = (int)ch;
-    u.n_units = (int)((n_items + 64 * ch - 1) / (64 * ch));
+    u.chunks = n_items > ((int64_t)1 << 20) ? 16 : 4;
+    u.n_units = (int)((n_items + 64 * u.chunks - 1) / (64 * u.chunks));
     if (u.n_units < 1) u.n_units = 1;
     return u;
 }
@@ -60,25 +58,34 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
     }
 };
 
-// A token's k expert ids, in registers when k <= KMAX (KMAX > 0), else re-read through L1.
+// A token's k expert ids and their nodes, in registers when k <= KMAX (KMAX > 0), else re-read
+// through L1.  Padding entries hold INT_MAX so they rank after every real id.
 template <int KMAX>
 struct RowIds {
     int v[KMAX > 0 ? KMAX : 1];
+    int nd[KMAX > 0 ? KMAX : 1];
     const int64_t *row;
-    int k;
-    __device__ __forceinline__ void load(const int64_t *r, int k_) {
+    int k, slots;
+    __device__ __forceinline__ void load(const int64_t *r, int k_, int slots_) {
         row = r;
         k = k_;
+        slots = slots_;
         if constexpr (KMAX > 0) {
 #pragma unroll
-            for (int j = 0; j < KMAX; ++j) v[j] = j < k ? (int)r[j] : 0x7FFFFFFF;
+            for (int j = 0; j < KMAX; ++j) {
+                v[j] = j < k ? (int)r[j] : 0x7FFFFFFF;
+                nd[j] = j < k ? v[j] / slots : 0x7FFFFFFF;
+            }
         }
     }
     __device__ __forceinline__ int at(int j) const {
         if constexpr (KMAX > 0) return v[j];
         else return (int)row[j];
     }
-    __device__ __forceinline__ int bound() const { return KMAX > 0 ? KMAX : k; }
+    __device__ __forceinline__ int node(int j) const {
+        if constexpr (KMAX > 0) return nd[j];
+        else return (int)row[j] / slots;
+    }
 };
 
 template <int KMAX>
@@ -94,19 +101,32 @@ __device__ __forceinline__ int rank_in_row(const RowIds<KMAX> &ids, int j) {
     return r;
 }
 
-// Expert id of the element whose ascending rank inside the row is `want` (-1 if none: duplicates).
+// Column of the element whose ascending rank inside the row is `want` (-1 if none: duplicates).
 template <int KMAX>
-__device__ __forceinline__ int id_with_rank(const RowIds<KMAX> &ids, int want) {
+__device__ __forceinline__ int column_with_rank(const RowIds<KMAX> &ids, int want) {
     int found = -1;
     if constexpr (KMAX > 0) {
 #pragma unroll
         for (int j = 0; j < KMAX; ++j)
-            if (j < ids.k && rank_in_row(ids, j) == want) found = ids.v[j];
+            if (j < ids.k && rank_in_row(ids, j) == want) found = j;
     } else {
         for (int j = 0; j < ids.k; ++j)
-            if (rank_in_row(ids, j) == want) found = ids.at(j);
+            if (rank_in_row(ids, j) == want) found = j;
     }
     return found;
+}
+
+template <int KMAX>
+__device__ __forceinline__ int node_of_column(const RowIds<KMAX> &ids, int col) {
+    int n = -1;
+    if constexpr (KMAX > 0) {
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j)
+            if (j == col) n = ids.nd[j];
+    } else {
+        if (col >= 0) n = ids.node(col);
+    }
+    return n;
 }
 
 template <int KMAX>
@@ -117,20 +137,21 @@ struct KeyRun {              // item = t*M + m  ->  node of the m-th run of toke
         const int64_t t = item / groups_m;
         const int m = (int)(item - t * groups_m);
         RowIds<KMAX> ids;
-        ids.load(expert_idx + t * k, k);
-        const int e = id_with_rank(ids, m * quota);
-        if (e < 0 || e / slots >= n_nodes) {
+        ids.load(expert_idx + t * k, k, slots);
+        const int col = column_with_rank(ids, m * quota);
+        const int n = node_of_column(ids, col);
+        if (col < 0 || n < 0 || n >= n_nodes) {
             *bad = true;
             return 0;
         }
-        return e / slots;
+        return n;
     }
 };
 
 // ---------------------------------------------------------------------------------------------
-// count
+// count: table is bucket-major, table[b * n_units + unit]
 // ---------------------------------------------------------------------------------------------
-template <typename KeyFn>
+template <typename KeyFn, int CH>
 __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, int32_t *__restrict__ table) {
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
@@ -138,83 +159,96 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
     volatile int32_t *hist = lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
+    const int64_t first = (int64_t)unit * CH * kWave;
+    int keys[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {       // all chunks' keys are fetched before any is consumed
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        bool bad = false;
+        keys[c] = item < u.n_items ? key_of(item, &bad) : -1;
+    }
     for (int b = lane; b < u.n_buckets; b += kWave) hist[b] = 0;
     __builtin_amdgcn_wave_barrier();
-    const int64_t first = (int64_t)unit * u.chunks * kWave;
-    for (int c = 0; c < u.chunks; ++c) {
-        const int64_t item = first + (int64_t)c * kWave + lane;
-        const bool valid = item < u.n_items;
-        bool bad = false;
-        const int key = valid ? key_of(item, &bad) : 0;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int key = keys[c];
+        const bool valid = key >= 0;
         uint64_t todo = __ballot(valid);
         while (todo) {
             const int leader = __builtin_ctzll(todo);
             const int kk = read_lane(key, leader);
-            const uint64_t peers = __ballot(valid && key == kk);
+            const uint64_t peers = __ballot(key == kk);
             if (lane == leader) hist[kk] = hist[kk] + __popcll(peers);
             todo &= ~peers;
         }
         __builtin_amdgcn_wave_barrier();
     }
-    for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)unit * u.n_buckets + b] = hist[b];
+    for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)b * u.n_units + unit] = hist[b];
 }
 
 // ---------------------------------------------------------------------------------------------
-// scan: table[unit][bucket] counts -> exclusive cursors in (bucket, unit) order, in place.
-// Also start[b] (int32, n_buckets+1 entries after the table), the caller's histogram and
-// offsets planes, and a zeroed status block.
+// scan: exclusive prefix over the bucket-major table, in place (staged through LDS when it
+// fits).  Also writes start[b] (n_buckets+1 int32 after the table), the caller's histogram and
+// offsets planes, and zeroes the status block.
 // ---------------------------------------------------------------------------------------------
+constexpr int kScanLds = 12288;
+
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table,
                                                             int64_t *__restrict__ hist_i64,
                                                             float *__restrict__ hist_f32,
                                                             int64_t *__restrict__ offsets_i64,
-                                                            int32_t *__restrict__ status, int divide_by) {
+                                                            int32_t *__restrict__ status) {
+    __shared__ int32_t buf[kScanLds];
     __shared__ int32_t wave_tot[kScanThreads / kWave];
     __shared__ int32_t grand_total;
-    int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
     const int tid = threadIdx.x;
     const int64_t n = (int64_t)u.n_units * u.n_buckets;
+    int32_t *start = table + n;
+    const bool staged = n <= kScanLds;
+    if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
+    if (staged) {
+        for (int64_t i = tid; i < n; i += kScanThreads) buf[i] = table[i];
+        __syncthreads();
+    }
+    int32_t *x = staged ? buf : table;
     const int64_t per = (n + kScanThreads - 1) / kScanThreads;
     const int64_t lo = tid * per, hi = lo + per < n ? lo + per : n;
-    if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
     int32_t sum = 0;
-    for (int64_t i = lo; i < hi; ++i) {
-        const int64_t b = i / u.n_units, un = i - b * u.n_units;
-        sum += table[un * u.n_buckets + b];
-    }
-    int32_t incl = wave_inclusive_scan(sum);
+    for (int64_t i = lo; i < hi; ++i) sum += x[i];
+    const int32_t incl = wave_inclusive_scan(sum);
     if (lane_id() == kWave - 1) wave_tot[tid >> 6] = incl;
     __syncthreads();
     if (tid < kWave) {
-        int32_t t = tid < kScanThreads / kWave ? wave_tot[tid] : 0;
-        int32_t ti = wave_inclusive_scan(t);
+        const int32_t t = tid < kScanThreads / kWave ? wave_tot[tid] : 0;
+        const int32_t ti = wave_inclusive_scan(t);
         if (tid < kScanThreads / kWave) wave_tot[tid] = ti - t;
         if (tid == kScanThreads / kWave - 1) grand_total = ti;
     }
     __syncthreads();
     int32_t run = wave_tot[tid >> 6] + incl - sum;
     for (int64_t i = lo; i < hi; ++i) {
-        const int64_t b = i / u.n_units, un = i - b * u.n_units;
-        const int32_t c = table[un * u.n_buckets + b];
-        table[un * u.n_buckets + b] = run;
-        if (un == 0) start[b] = run;
+        const int32_t c = x[i];
+        x[i] = run;
         run += c;
     }
-    if (tid == 0) start[u.n_buckets] = grand_total;
     __syncthreads();
-    for (int b = tid; b < u.n_buckets; b += kScanThreads) {
-        const int32_t s0 = start[b], s1 = start[b + 1];
-        const int32_t cnt = (s1 - s0) / divide_by;
-        if (hist_i64) hist_i64[b] = cnt;
-        if (hist_f32) hist_f32[b] = (float)cnt;
-        if (offsets_i64) offsets_i64[b] = s0 / divide_by;
+    if (staged)
+        for (int64_t i = tid; i < n; i += kScanThreads) table[i] = buf[i];
+    for (int b = tid; b <= u.n_buckets; b += kScanThreads) {
+        const int32_t s0 = b < u.n_buckets ? x[(int64_t)b * u.n_units] : grand_total;
+        start[b] = s0;
+        if (b == u.n_buckets) break;
+        const int32_t s1 = b + 1 < u.n_buckets ? x[(int64_t)(b + 1) * u.n_units] : grand_total;
+        if (hist_i64) hist_i64[b] = s1 - s0;
+        if (hist_f32) hist_f32[b] = (float)(s1 - s0);
+        if (offsets_i64) offsets_i64[b] = s0;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // rank
 // ---------------------------------------------------------------------------------------------
-template <typename KeyFn, typename EmitFn>
+template <typename KeyFn, typename EmitFn, int CH>
 __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit, Units u,
                                                       const int32_t *__restrict__ table,
                                                       int32_t *__restrict__ status) {
@@ -224,26 +258,33 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
     volatile int32_t *cursor = lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
-    for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)unit * u.n_buckets + b];
+    const int64_t first = (int64_t)unit * CH * kWave;
+    int fault = 0;
+    int keys[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        bool bad = false;
+        keys[c] = item < u.n_items ? key_of(item, &bad) : -1;
+        if (bad) fault |= TERRACE_FAULT_ID_RANGE;
+    }
+    for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)b * u.n_units + unit];
     __builtin_amdgcn_wave_barrier();
     const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
-    const int64_t first = (int64_t)unit * u.chunks * kWave;
-    int fault = 0;
     int tally[2] = {0, 0};
-    for (int c = 0; c < u.chunks; ++c) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
         const int64_t item = first + (int64_t)c * kWave + lane;
-        const bool valid = item < u.n_items;
-        bool bad = false;
-        const int key = valid ? key_of(item, &bad) : 0;
-        if (bad) fault |= TERRACE_FAULT_ID_RANGE;
+        const int key = keys[c];
+        const bool valid = key >= 0;
         int32_t dest = 0;
         uint64_t todo = __ballot(valid);
         while (todo) {
             const int leader = __builtin_ctzll(todo);
             const int kk = read_lane(key, leader);
-            const uint64_t peers = __ballot(valid && key == kk);
+            const uint64_t peers = __ballot(key == kk);
             const int32_t base = cursor[kk];
-            if (valid && key == kk) dest = base + __popcll(peers & lanes_below(lane));
+            if (key == kk) dest = base + __popcll(peers & lanes_below(lane));
             __builtin_amdgcn_wave_barrier();
             if (lane == leader) cursor[kk] = base + __popcll(peers);
             todo &= ~peers;
@@ -340,15 +381,15 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
         const int64_t t = item / groups_m;
         const int m = (int)(item - t * groups_m);
         RowIds<KMAX> ids;
-        ids.load(expert_idx + t * k, k);
+        ids.load(expert_idx + t * k, k, slots);
         int fault = 0;
         if (m == 0) {
             int occupied = 0, off_quota = 0;
             auto census = [&](int j) {
-                const int nj = ids.at(j) / slots;
+                const int nj = ids.node(j);
                 int same = 0, earlier = 0;
                 auto cmp = [&](int i) {
-                    const bool hit = (ids.at(i) / slots) == nj;
+                    const bool hit = ids.node(i) == nj;
                     same += hit ? 1 : 0;
                     earlier += (hit && i < j) ? 1 : 0;
                 };
@@ -387,7 +428,7 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
             if (r / quota != m) return;
             const int i = r - m * quota;
             const int64_t cell = (int64_t)row * quota + i;
-            mask[cell] = e >= 0 ? e % slots : 0;
+            mask[cell] = e >= 0 ? e - ids.node(j) * slots : 0;
             if (gates) {
                 if (gate_bytes == 4) {
                     const uint32_t gv = ((const uint32_t *)gates)[t * k + j];
@@ -468,7 +509,7 @@ __global__ __launch_bounds__(kBlock) void pack_quota_wire_kernel(const int64_t *
     const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (t >= T) return;
     RowIds<KMAX> ids;
-    ids.load(expert_idx + t * k, k);
+    ids.load(expert_idx + t * k, k, slots);
     bool bad = false;
     auto body = [&](int j) {
         const int e = ids.at(j);
@@ -521,10 +562,16 @@ static size_t lds_for(const Units &u) { return (size_t)kWavesPerBlock * u.n_buck
 
 template <typename KeyFn, typename EmitFn>
 static int run_sort(const KeyFn &key, const EmitFn &emit, const Units &u, int32_t *table, int64_t *hist,
-                    float *hist_f, int64_t *offsets, int32_t *status, int divide_by, bool do_rank, hipStream_t s) {
-    count_kernel<KeyFn><<<blocks_for_units(u), kBlock, lds_for(u), s>>>(key, u, table);
-    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist, hist_f, offsets, status, divide_by);
-    if (do_rank) rank_kernel<KeyFn, EmitFn><<<blocks_for_units(u), kBlock, lds_for(u), s>>>(key, emit, u, table, status);
+                    float *hist_f, int64_t *offsets, int32_t *status, bool do_rank, hipStream_t s) {
+    const int blocks = blocks_for_units(u);
+    const size_t lds = lds_for(u);
+    if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, kBlock, lds, s>>>(key, u, table);
+    else count_kernel<KeyFn, 16><<<blocks, kBlock, lds, s>>>(key, u, table);
+    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist, hist_f, offsets, status);
+    if (do_rank) {
+        if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
+        else rank_kernel<KeyFn, EmitFn, 16><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
+    }
     return check_launch();
 }
 
@@ -550,7 +597,7 @@ int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_flo
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyAffine key{idx, 0, 1, n_buckets};
     // the rank pass runs only to report out-of-range ids
-    return run_sort(key, EmitNothing{}, u, (int32_t *)ws, h, hf, nullptr, status, 1, status != nullptr, s);
+    return run_sort(key, EmitNothing{}, u, (int32_t *)ws, h, hf, nullptr, status, status != nullptr, s);
 }
 
 int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *order, int64_t *hist, int32_t *status,
@@ -561,7 +608,7 @@ int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *or
     const Units u = make_units(n, n_buckets);
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyAffine key{keyp, 0, 1, n_buckets};
-    return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, hist, nullptr, nullptr, status, 1, true, s);
+    return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, hist, nullptr, nullptr, status, true, s);
 }
 
 // ---- Hop-B arrival ----------------------------------------------------------------------------
@@ -589,7 +636,7 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
     int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
     KeyAffine key{rslot, 0, epr, rpn};
     EmitArrival emit{rslot, rgate, gate_bytes, quota, gate_pairs, r_idx, slot_idx, pair_pos, pos32};
-    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, 1, true, s);
+    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
 }
@@ -628,7 +675,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     int32_t *gidx = (int32_t *)((char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
     KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr};
     EmitRegroup emit{capacity, order, dest, kept, order32};
-    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, 1, true, s);
+    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *src_of_place = order32;
     const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
@@ -691,7 +738,7 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
     EmitPack<KMAX> emit{expert_idx, gates, gate_bytes, k, groups_m, quota, slots, n_experts,
                         mask, u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_rows, gate_sorted,
                         pos32};
-    int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, 1, true, s);
+    int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
 }
