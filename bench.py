@@ -208,7 +208,7 @@ def main():
 
     # ---- the row-moving kernels alone ----
     row = cfg.row_bytes
-    where = tops.index_chain(state.place, tops.index_chain(state.pair_pos, state.extras["pair_table"]))
+    where = tops.index_chain2(state.place, state.pair_pos, state.extras["pair_table"])
     w_sorted = state.extras["gate_sorted"]
     token_rows, pair_pos2 = state.extras["token_rows"], state.pair_pos.view(cfg.send_rows, quota)
     if cap is None:

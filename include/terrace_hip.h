@@ -182,6 +182,11 @@ TERRACE_API int terrace_scatter_rows(const void *src, const int64_t *pos, int64_
 TERRACE_API int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out,
                         terrace_stream_t stream);
 
+/* out[i] = outer[inner[idx[i]]], -1 propagating at either level (one launch for the two
+ * look-ups that turn a token's Hop-A pair ids into places of the expert-order buffer). */
+TERRACE_API int terrace_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n,
+                                     int64_t *out, terrace_stream_t stream);
+
 /* Gate-weighted combine (terrace/ta2a_fwd.py:658-670; one level: terrace/ep_dist.py:121-122):
  *   out[i,:] = sum_{j<fan} w[i,j] * decode(src[idx[i,j],:])      (idx < 0 contributes nothing)
  * accumulated in fp32 as acc = fl(acc + fl(w*x)) for j = 0..fan-1, rounded once to out_dtype.

@@ -6,6 +6,8 @@ int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
 int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
                    int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
 int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
+int launch_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
+                        hipStream_t s);
 int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s);
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
@@ -148,6 +150,12 @@ int terrace_scatter_rows(const void *src, const int64_t *pos, int64_t n_src, int
 int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream) {
     if (n < 0 || (n && (!table || !idx || !out))) return TERRACE_EINVAL;
     return launch_index_chain(table, idx, n, out, (hipStream_t)stream);
+}
+
+int terrace_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
+                         terrace_stream_t stream) {
+    if (n < 0 || (n && (!outer || !inner || !idx || !out))) return TERRACE_EINVAL;
+    return launch_index_chain2(outer, inner, idx, n, out, (hipStream_t)stream);
 }
 
 int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const void *weights, int w_dtype,

@@ -300,6 +300,17 @@ __global__ __launch_bounds__(kBlock) void index_chain_kernel(const int64_t *__re
     out[i] = a < 0 ? -1 : table[a];
 }
 
+__global__ __launch_bounds__(kBlock) void index_chain2_kernel(const int64_t *__restrict__ outer,
+                                                              const int64_t *__restrict__ inner,
+                                                              const int64_t *__restrict__ idx, int64_t n,
+                                                              int64_t *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    int64_t a = idx[i];
+    if (a >= 0) a = inner[a];
+    out[i] = a < 0 ? -1 : outer[a];
+}
+
 __global__ void send_splits_kernel(const int64_t *__restrict__ node_counts, int world, int rpn, int my_local,
                                    int64_t *__restrict__ send) {
     for (int i = threadIdx.x; i < world; i += blockDim.x)
@@ -472,6 +483,13 @@ int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s) {
 int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s) {
     if (n <= 0) return TERRACE_OK;
     index_chain_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(table, idx, n, out);
+    return check_launch();
+}
+
+int launch_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
+                        hipStream_t s) {
+    if (n <= 0) return TERRACE_OK;
+    index_chain2_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(outer, inner, idx, n, out);
     return check_launch();
 }
 

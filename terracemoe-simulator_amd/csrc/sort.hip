@@ -12,19 +12,9 @@
 //   scan   one workgroup turns the [unit][bucket] counts into exclusive cursors (bucket-major);
 //   rank   each wave replays its unit, ranks items with wave ballots, and emits the outputs.
 // The row payload itself is moved afterwards by the scatter/gather kernels of rows.hip.
-#include "common.hpp"
+#include "sort.hpp"
 
 namespace terrace {
-
-constexpr int kMaxBuckets = 2048;
-constexpr int kScanThreads = 1024;
-
-struct Units {
-    int64_t n_items;
-    int chunks;       // 64-item chunks per unit: 4, or 16 for more than a million items
-    int n_units;
-    int n_buckets;
-};
 
 Units make_units(int64_t n_items, int n_buckets) {
     Units u;
@@ -191,30 +181,33 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
 // fits).  Also writes start[b] (n_buckets+1 int32 after the table), the caller's histogram and
 // offsets planes, and zeroes the status block.
 // ---------------------------------------------------------------------------------------------
-constexpr int kScanLds = 12288;
+// Each of the 1024 threads owns a contiguous segment of `per` (a multiple of 4) entries and
+// moves it with 16-byte accesses, several in flight.
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table,
                                                             int64_t *__restrict__ hist_i64,
                                                             float *__restrict__ hist_f32,
                                                             int64_t *__restrict__ offsets_i64,
                                                             int32_t *__restrict__ status) {
-    __shared__ int32_t buf[kScanLds];
     __shared__ int32_t wave_tot[kScanThreads / kWave];
     __shared__ int32_t grand_total;
     const int tid = threadIdx.x;
     const int64_t n = (int64_t)u.n_units * u.n_buckets;
     int32_t *start = table + n;
-    const bool staged = n <= kScanLds;
     if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
-    if (staged) {
-        for (int64_t i = tid; i < n; i += kScanThreads) buf[i] = table[i];
-        __syncthreads();
-    }
-    int32_t *x = staged ? buf : table;
-    const int64_t per = (n + kScanThreads - 1) / kScanThreads;
+    const int64_t per = ((n + kScanThreads - 1) / kScanThreads + 3) / 4 * 4;
     const int64_t lo = tid * per, hi = lo + per < n ? lo + per : n;
+    const bool vec = (hi - lo) == per && (((uintptr_t)table) & 15) == 0;
     int32_t sum = 0;
-    for (int64_t i = lo; i < hi; ++i) sum += x[i];
+    if (vec) {
+        i32x4 acc = {0, 0, 0, 0};
+#pragma unroll 4
+        for (int64_t i = lo; i < hi; i += 4) acc += *(const i32x4 *)(table + i);
+        sum = acc[0] + acc[1] + acc[2] + acc[3];
+    } else {
+        for (int64_t i = lo; i < hi; ++i) sum += table[i];
+    }
     const int32_t incl = wave_inclusive_scan(sum);
     if (lane_id() == kWave - 1) wave_tot[tid >> 6] = incl;
     __syncthreads();
@@ -226,23 +219,40 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__
     }
     __syncthreads();
     int32_t run = wave_tot[tid >> 6] + incl - sum;
-    for (int64_t i = lo; i < hi; ++i) {
-        const int32_t c = x[i];
-        x[i] = run;
-        run += c;
+    if (vec) {
+#pragma unroll 4
+        for (int64_t i = lo; i < hi; i += 4) {
+            const i32x4 c = *(const i32x4 *)(table + i);
+            i32x4 o;
+            o[0] = run;
+            o[1] = o[0] + c[0];
+            o[2] = o[1] + c[1];
+            o[3] = o[2] + c[2];
+            run = o[3] + c[3];
+            *(i32x4 *)(table + i) = o;
+        }
+    } else {
+        for (int64_t i = lo; i < hi; ++i) {
+            const int32_t c = table[i];
+            table[i] = run;
+            run += c;
+        }
     }
     __syncthreads();
-    if (staged)
-        for (int64_t i = tid; i < n; i += kScanThreads) table[i] = buf[i];
     for (int b = tid; b <= u.n_buckets; b += kScanThreads) {
-        const int32_t s0 = b < u.n_buckets ? x[(int64_t)b * u.n_units] : grand_total;
+        const int32_t s0 = b < u.n_buckets ? table[(int64_t)b * u.n_units] : grand_total;
         start[b] = s0;
         if (b == u.n_buckets) break;
-        const int32_t s1 = b + 1 < u.n_buckets ? x[(int64_t)(b + 1) * u.n_units] : grand_total;
+        const int32_t s1 = b + 1 < u.n_buckets ? table[(int64_t)(b + 1) * u.n_units] : grand_total;
         if (hist_i64) hist_i64[b] = s1 - s0;
         if (hist_f32) hist_f32[b] = (float)(s1 - s0);
         if (offsets_i64) offsets_i64[b] = s0;
     }
+}
+
+void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
+                 int32_t *status, hipStream_t s) {
+    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -551,12 +561,6 @@ __global__ __launch_bounds__(kBlock) void pack_quota_wire_kernel(const int64_t *
 // ---------------------------------------------------------------------------------------------
 // host drivers
 // ---------------------------------------------------------------------------------------------
-template <typename I>
-int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
-                        hipStream_t s);
-template <typename I>
-int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
-
 static int blocks_for_units(const Units &u) { return (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock; }
 static size_t lds_for(const Units &u) { return (size_t)kWavesPerBlock * u.n_buckets * sizeof(int32_t); }
 
@@ -567,7 +571,7 @@ static int run_sort(const KeyFn &key, const EmitFn &emit, const Units &u, int32_
     const size_t lds = lds_for(u);
     if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, kBlock, lds, s>>>(key, u, table);
     else count_kernel<KeyFn, 16><<<blocks, kBlock, lds, s>>>(key, u, table);
-    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist, hist_f, offsets, status);
+    launch_scan(u, table, hist, hist_f, offsets, status, s);
     if (do_rank) {
         if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
         else rank_kernel<KeyFn, EmitFn, 16><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
@@ -723,7 +727,9 @@ int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int6
 size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m) {
     const int64_t S = T * groups_m;
     if (S <= 0 || n_nodes <= 0 || n_nodes > kMaxBuckets) return 256;
-    return units_table_bytes(make_units(S, n_nodes)) + align_up((size_t)S * sizeof(int32_t), 256);
+    const size_t item_path = units_table_bytes(make_units(S, n_nodes)) + align_up((size_t)S * sizeof(int32_t), 256);
+    const size_t token_path = k2_token_path_applies(k, n_nodes) ? k2_token_workspace(T, n_nodes, groups_m) : 0;
+    return item_path > token_path ? item_path : token_path;
 }
 
 template <int KMAX>
@@ -757,9 +763,13 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
     if (n_nodes > kMaxBuckets || T * k >= (int64_t)1 << 31 || S >= (int64_t)1 << 31) return TERRACE_EINVAL;
     if (S == 0) return empty_outputs(node_counts, nullptr, node_offsets, n_nodes, status, s);
     if (!expert_idx || !mask || !u_src || !ws || (hidden && !payload) || (gates && !gate_rows)) return TERRACE_EINVAL;
+    if (ws_bytes < k2_workspace(T, k, n_nodes, groups_m)) return TERRACE_ENOSPC;
+    if (k2_token_path_applies(k, n_nodes))
+        return run_k2_token(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts,
+                            groups_m, payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets,
+                            pair_table, sort_order, token_rows, gate_sorted, status, ws, s);
     const Units u = make_units(S, n_nodes);
     const size_t table_bytes = units_table_bytes(u);
-    if (ws_bytes < table_bytes + align_up((size_t)S * sizeof(int32_t), 256)) return TERRACE_ENOSPC;
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
 #define TERRACE_K2(KM)                                                                                        \

@@ -323,6 +323,17 @@ def index_chain(table, idx):
     return out
 
 
+def index_chain2(outer, inner, idx):
+    """``outer[inner[idx]]`` over int64 planes in one launch (negative entries propagate as -1)."""
+    _require()
+    _hip.need_device(outer, inner, idx)
+    outer, inner, idx = outer.contiguous(), inner.contiguous(), idx.contiguous()
+    out = torch.empty_like(idx)
+    _hip.call("terrace_index_chain2", _hip.ptr(outer), _hip.ptr(inner), _hip.ptr(idx), idx.numel(), _hip.ptr(out),
+              _hip.stream(idx.device))
+    return out
+
+
 def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
     """``out[i] = sum_j weights[i,j] * src[idx[i,j]]`` accumulated in fp32 in the order ``idx``
     lists the rows, rounded once to ``out_dtype`` (default: ``src.dtype``, or bf16 for fp8 rows).
@@ -563,5 +574,5 @@ def k2_pack(hidden, expert_idx, gates, world: int, n_experts: int, rpn: int, gro
 __all__ = [
     "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
-    "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "hist", "argsort_small", "hopa_send_splits",
+    "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
 ]

@@ -127,7 +127,7 @@ def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, wei
     node ascending across the token's rows -- which is the order the reference's two
     ``index_add`` levels add in (terrace/ta2a_fwd.py:661-670 there), accumulated in fp32.
     """
-    where = _ops.index_chain(st.place, _ops.index_chain(st.pair_pos, st.extras["pair_table"]))
+    where = _ops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
     w = st.extras["gate_sorted"] if weights is None else weights
     return _ops.combine(ye, where, w, out_dtype=out_dtype, fp8_hidden=fp8_hidden)
 

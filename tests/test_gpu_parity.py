@@ -157,11 +157,17 @@ def _k2_case(world, rpn, E, T, k, M, fmt, sort_rows, seed, H=16):
     return e, hidden, gates
 
 
+# beyond the reference's list: k in 9..16 (wider register row), more than 64 nodes and k > 16
+# (the (token, run)-item kernels), several units per launch, a single token per wave tail
+EXTRA_K2_GEOMS = [(8, 2, 64, 37, 12, 3), (80, 1, 160, 50, 4, 2), (8, 2, 64, 21, 24, 4), (64, 8, 256, 3000, 8, 4),
+                  (128, 8, 128, 1025, 8, 2), (64, 8, 64, 257, 4, 2)]
+
+
 @pytest.mark.parametrize("fmt", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("sort_rows", [True, False])
 def test_k2_pack_reference_geometries(literals, fmt, sort_rows):
     import terrace.ops as tops
-    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"] + EXTRA_K2_GEOMS:
         for seed in (500, 501):
             announce("k2", (world, rpn, E, T, k, M), fmt, sort_rows, seed)
             e, hidden, gates = _k2_case(world, rpn, E, T, k, M, fmt, sort_rows, seed)
@@ -240,6 +246,33 @@ def test_plan_guard_literal_cases(literals):
     ta2a._VERIFY_COUNT[(4, 4, 2, 2)] = 256
     with pytest.raises(ValueError, match="quota"):
         ta2a.plan_ta2a(bad, 4, 8, 2, groups_m=2)
+
+
+def test_malformed_routing_is_contained_and_counted():
+    """Unchecked calls on a routing that breaks the invariants must stay in range and report the
+    census the guard reads: occupied (token, node) pairs and pairs off the quota."""
+    import terrace.ops as tops
+    from terrace import _hip
+    announce("k2 malformed")
+    cases = {
+        "three_one": ([[0, 2, 3, 5]] * 6, 12, 12),          # 2 nodes each, both off the 2/2 quota
+        "fanout_one": ([[0, 1, 2, 3]] * 6, 6, 6),           # one node holding 4
+        "id_range": ([[0, 2, 4, 99]] * 6, 12, 6),           # one id outside [0, 8)
+    }
+    for name, (rows, occupied, off_quota) in cases.items():
+        e = torch.tensor(rows, device=DEV)
+        x = torch.randn(6, 16, device=DEV)
+        gts = torch.rand(6, 4, device=DEV)
+        (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e, gts, 4, 8, 2, 2, extras=True)
+        fault, occ, offq, _ = ex["status"].tolist()
+        assert fault != 0 and occ == occupied and offq == off_quota, (name, fault, occ, offq)
+        assert int(counts.sum()) <= 12 and (counts >= 0).all()
+        assert ((u_src >= 0) & (u_src < 6)).all() and ((mask >= 0) & (mask < 4)).all()
+        assert ((ex["pair_table"] >= -1) & (ex["pair_table"] < 24)).all()
+        assert ((ex["token_rows"] >= -1) & (ex["token_rows"] < 12)).all()
+        assert torch.isfinite(gate_rows).all()
+        if name == "id_range":
+            assert fault & _hip.FAULT_ID_RANGE
 
 
 def test_hopa_send_splits_literal(literals):
