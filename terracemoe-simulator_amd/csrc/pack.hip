@@ -16,7 +16,9 @@
 
 namespace terrace {
 
-constexpr int kTokChunks = 4;      // 256 tokens per wave
+// 64 tokens per wave while that keeps the count table small, 256 beyond a quarter million tokens:
+// the work per token is latency-bound, so more, shorter waves finish sooner.
+static int token_chunks(int64_t T) { return T <= ((int64_t)1 << 18) ? 1 : 4; }
 
 bool k2_token_path_applies(int k, int n_nodes) { return k <= 16 && n_nodes <= 64; }
 
@@ -24,8 +26,8 @@ static Units token_units(int64_t T, int n_nodes) {
     Units u;
     u.n_items = T;
     u.n_buckets = n_nodes;
-    u.chunks = kTokChunks;
-    u.n_units = (int)((T + 64 * kTokChunks - 1) / (64 * kTokChunks));
+    u.chunks = token_chunks(T);
+    u.n_units = (int)((T + 64 * u.chunks - 1) / (64 * u.chunks));
     if (u.n_units < 1) u.n_units = 1;
     return u;
 }
@@ -69,7 +71,7 @@ struct TokenRow {
     }
 };
 
-template <int KMAX>
+template <int KMAX, int kTokChunks>
 __global__ __launch_bounds__(kBlock) void k2_count_kernel(const int64_t *__restrict__ expert_idx, int64_t T, int k,
                                                           int slots, int n_nodes, int n_experts, int M, int n_units,
                                                           int32_t *__restrict__ table) {
@@ -102,7 +104,7 @@ __device__ __forceinline__ void put_gate(void *plane, int64_t at, const void *ga
     ((G *)plane)[at] = ((const G *)gates)[from];
 }
 
-template <int KMAX, typename G>
+template <int KMAX, typename G, int kTokChunks>
 __global__ __launch_bounds__(kBlock) void k2_place_kernel(
     const int64_t *__restrict__ expert_idx, const G *__restrict__ gates, int64_t T, int k, int slots, int n_nodes,
     int n_experts, int M, int quota, int n_units, const int32_t *__restrict__ table, int64_t *__restrict__ mask,
@@ -248,10 +250,14 @@ static void launch_place(const int64_t *expert_idx, const void *gates, int64_t T
                          int64_t *sort_order, int64_t *token_rows, void *gate_sorted, int32_t *pos32,
                          int32_t *status, hipStream_t s) {
     const int blocks = (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock;
-    k2_place_kernel<KMAX, G><<<blocks, kBlock, 0, s>>>(expert_idx, (const G *)gates, T, k, slots, n_nodes, n_experts,
-                                                       M, k / M, u.n_units, table, mask, (G *)gate_rows, u_src,
-                                                       u_node, inverse, pair_table, sort_order, token_rows,
-                                                       (G *)gate_sorted, pos32, status);
+    if (u.chunks == 1)
+        k2_place_kernel<KMAX, G, 1><<<blocks, kBlock, 0, s>>>(
+            expert_idx, (const G *)gates, T, k, slots, n_nodes, n_experts, M, k / M, u.n_units, table, mask,
+            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status);
+    else
+        k2_place_kernel<KMAX, G, 4><<<blocks, kBlock, 0, s>>>(
+            expert_idx, (const G *)gates, T, k, slots, n_nodes, n_experts, M, k / M, u.n_units, table, mask,
+            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status);
 }
 
 int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
@@ -263,10 +269,16 @@ int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gate
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + units_table_bytes(u));
     const int blocks = (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (k <= 8)
-        k2_count_kernel<8><<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, groups_m, u.n_units, table);
-    else
-        k2_count_kernel<16><<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, groups_m, u.n_units, table);
+#define TERRACE_COUNT(KM, CH) \
+    k2_count_kernel<KM, CH><<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, groups_m, u.n_units, table)
+    if (k <= 8) {
+        if (u.chunks == 1) TERRACE_COUNT(8, 1);
+        else TERRACE_COUNT(8, 4);
+    } else {
+        if (u.chunks == 1) TERRACE_COUNT(16, 1);
+        else TERRACE_COUNT(16, 4);
+    }
+#undef TERRACE_COUNT
     launch_scan(u, table, node_counts, nullptr, node_offsets, status, s);
 #define TERRACE_PLACE(KM, G)                                                                                       \
     launch_place<KM, G>(expert_idx, gates, T, k, slots, n_nodes, n_experts, groups_m, u, table, mask, gate_rows,   \

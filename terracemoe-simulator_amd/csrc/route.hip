@@ -365,8 +365,8 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
         return TERRACE_EINVAL;
     if (T == 0) return TERRACE_OK;
     if (!affinity || !bias || !expert_idx || !gates || !group_idx) return TERRACE_EINVAL;
-    int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 256 * 8) blocks = 256 * 8;
+    int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;      // one token per wave
+    if (blocks > ((int64_t)1 << 24)) blocks = (int64_t)1 << 24;
     int vpl = 1;
     while (vpl * kWave < E) vpl *= 2;
     const bool aligned = (((uintptr_t)affinity) & 15) == 0;

@@ -148,10 +148,16 @@ __device__ __forceinline__ void decode_chunk(u32x4 raw, float *f) {
             f[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(raw[i] >> 16)));
         }
     } else {
+        // gfx950's packed fp8 conversion reads OCP e4m3 ("fn": bias 7, no infinities)
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-#pragma unroll
-            for (int b = 0; b < 4; ++b) f[4 * i + b] = e4m3_to_f32((raw[i] >> (8 * b)) & 0xFFu);
+            const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)raw[i], false);
+            const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)raw[i], true);
+            f[4 * i] = lo[0];
+            f[4 * i + 1] = lo[1];
+            f[4 * i + 2] = hi[0];
+            f[4 * i + 3] = hi[1];
         }
     }
 }

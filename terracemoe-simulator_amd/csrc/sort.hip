@@ -20,7 +20,14 @@ Units make_units(int64_t n_items, int n_buckets) {
     Units u;
     u.n_items = n_items;
     u.n_buckets = n_buckets;
-    u.chunks = n_items > ((int64_t)1 << 20) ? 16 : 4;
+    // the smallest unit (most waves) whose count table stays within 16K entries
+    u.chunks = 16;
+    for (int ch : {1, 4}) {
+        if ((n_items + 64 * ch - 1) / (64 * ch) * n_buckets <= 16384) {
+            u.chunks = ch;
+            break;
+        }
+    }
     u.n_units = (int)((n_items + 64 * u.chunks - 1) / (64 * u.chunks));
     if (u.n_units < 1) u.n_units = 1;
     return u;
@@ -181,62 +188,66 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
 // fits).  Also writes start[b] (n_buckets+1 int32 after the table), the caller's histogram and
 // offsets planes, and zeroes the status block.
 // ---------------------------------------------------------------------------------------------
-// Each of the 1024 threads owns a contiguous segment of `per` (a multiple of 4) entries and
-// moves it with 16-byte accesses, several in flight.
+// Each of the 16 waves owns a contiguous span (a multiple of 256 entries) and walks it 256
+// entries at a time, 16 bytes per lane, so every access is a fully coalesced 1 KB.
 typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ i32x4 load4_guarded(const int32_t *t, int64_t i, int64_t n) {
+    if (i + 3 < n) return *(const i32x4 *)(t + i);
+    i32x4 v = {0, 0, 0, 0};
+    if (i < n) v[0] = t[i];
+    if (i + 1 < n) v[1] = t[i + 1];
+    if (i + 2 < n) v[2] = t[i + 2];
+    return v;
+}
 
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table,
                                                             int64_t *__restrict__ hist_i64,
                                                             float *__restrict__ hist_f32,
                                                             int64_t *__restrict__ offsets_i64,
                                                             int32_t *__restrict__ status) {
-    __shared__ int32_t wave_tot[kScanThreads / kWave];
+    constexpr int kWaves = kScanThreads / kWave;
+    __shared__ int32_t wave_tot[kWaves];
     __shared__ int32_t grand_total;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = lane_id(), w = tid >> 6;
     const int64_t n = (int64_t)u.n_units * u.n_buckets;
     int32_t *start = table + n;
     if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
-    const int64_t per = ((n + kScanThreads - 1) / kScanThreads + 3) / 4 * 4;
-    const int64_t lo = tid * per, hi = lo + per < n ? lo + per : n;
-    const bool vec = (hi - lo) == per && (((uintptr_t)table) & 15) == 0;
-    int32_t sum = 0;
-    if (vec) {
-        i32x4 acc = {0, 0, 0, 0};
-#pragma unroll 4
-        for (int64_t i = lo; i < hi; i += 4) acc += *(const i32x4 *)(table + i);
-        sum = acc[0] + acc[1] + acc[2] + acc[3];
-    } else {
-        for (int64_t i = lo; i < hi; ++i) sum += table[i];
-    }
-    const int32_t incl = wave_inclusive_scan(sum);
-    if (lane_id() == kWave - 1) wave_tot[tid >> 6] = incl;
+    const int64_t span = ((n + kWaves - 1) / kWaves + 255) / 256 * 256;
+    const int64_t lo = w * span, hi = lo + span < n ? lo + span : n;
+    i32x4 acc = {0, 0, 0, 0};
+    for (int64_t base = lo; base < hi; base += 256) acc += load4_guarded(table, base + lane * 4, hi);
+    int32_t sum = acc[0] + acc[1] + acc[2] + acc[3];
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+    if (lane == 0) wave_tot[w] = sum;
     __syncthreads();
     if (tid < kWave) {
-        const int32_t t = tid < kScanThreads / kWave ? wave_tot[tid] : 0;
+        const int32_t t = tid < kWaves ? wave_tot[tid] : 0;
         const int32_t ti = wave_inclusive_scan(t);
-        if (tid < kScanThreads / kWave) wave_tot[tid] = ti - t;
-        if (tid == kScanThreads / kWave - 1) grand_total = ti;
+        if (tid < kWaves) wave_tot[tid] = ti - t;
+        if (tid == kWaves - 1) grand_total = ti;
     }
     __syncthreads();
-    int32_t run = wave_tot[tid >> 6] + incl - sum;
-    if (vec) {
-#pragma unroll 4
-        for (int64_t i = lo; i < hi; i += 4) {
-            const i32x4 c = *(const i32x4 *)(table + i);
-            i32x4 o;
-            o[0] = run;
-            o[1] = o[0] + c[0];
-            o[2] = o[1] + c[1];
-            o[3] = o[2] + c[2];
-            run = o[3] + c[3];
+    int32_t carry = wave_tot[w];
+    for (int64_t base = lo; base < hi; base += 256) {
+        const int64_t i = base + lane * 4;
+        const i32x4 c = load4_guarded(table, i, hi);
+        const int32_t s4 = c[0] + c[1] + c[2] + c[3];
+        const int32_t incl = wave_inclusive_scan(s4);
+        i32x4 o;
+        o[0] = carry + incl - s4;
+        o[1] = o[0] + c[0];
+        o[2] = o[1] + c[1];
+        o[3] = o[2] + c[2];
+        if (i + 3 < hi) {
             *(i32x4 *)(table + i) = o;
+        } else {
+            if (i < hi) table[i] = o[0];
+            if (i + 1 < hi) table[i + 1] = o[1];
+            if (i + 2 < hi) table[i + 2] = o[2];
         }
-    } else {
-        for (int64_t i = lo; i < hi; ++i) {
-            const int32_t c = table[i];
-            table[i] = run;
-            run += c;
-        }
+        carry += __shfl(incl, kWave - 1, kWave);
     }
     __syncthreads();
     for (int b = tid; b <= u.n_buckets; b += kScanThreads) {
@@ -569,11 +580,13 @@ static int run_sort(const KeyFn &key, const EmitFn &emit, const Units &u, int32_
                     float *hist_f, int64_t *offsets, int32_t *status, bool do_rank, hipStream_t s) {
     const int blocks = blocks_for_units(u);
     const size_t lds = lds_for(u);
-    if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, kBlock, lds, s>>>(key, u, table);
+    if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, kBlock, lds, s>>>(key, u, table);
+    else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, kBlock, lds, s>>>(key, u, table);
     else count_kernel<KeyFn, 16><<<blocks, kBlock, lds, s>>>(key, u, table);
     launch_scan(u, table, hist, hist_f, offsets, status, s);
     if (do_rank) {
-        if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
+        if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
+        else if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
         else rank_kernel<KeyFn, EmitFn, 16><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
     }
     return check_launch();

@@ -11,7 +11,7 @@ constexpr int kScanThreads = 1024;
 // A "unit" is the contiguous run of items one wave owns: chunks * 64 of them.
 struct Units {
     int64_t n_items;
-    int chunks;       // 64-item chunks per unit: 4, or 16 for more than a million items
+    int chunks;       // 64-item chunks per unit: 1, 4 or 16, growing with the item count
     int n_units;
     int n_buckets;
 };
