@@ -1,0 +1,188 @@
+"""The five benchmark geometries end to end on the device.
+
+At a reduced token count every plane of every stage is compared bit for bit with the CPU
+oracle.  At the full size the index / count / offset planes are still compared with the oracle
+(they are small), while the moved rows are checked through size-independent properties: every
+row of a stage's output equals the input row its index plane names, and with identity experts
+the combine returns each token scaled by the sum of its kept gates (dispatch -> combine round
+trip) within the stated tolerance.
+"""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import terrace_oracle as orc
+from test_gpu_parity import DEV, announce, same, to_np
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f32": 1e-5, "bf16": 1e-2, "fp8": 1e-2}
+
+
+def _route(cfg, inp):
+    import terrace
+    rcfg = terrace.TRouteConfig(cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups)
+    ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(DEV)
+    e, g, grp = terrace.t_route(inp["logits"].to(DEV), inp["bias"].to(DEV), rcfg, gate_affinity=ga)
+    oga = None if inp["gate_affinity"] is None else inp["gate_affinity"].numpy()
+    oe, og, ogrp = orc.t_route(inp["logits"].numpy(), inp["bias"].numpy(), cfg.n_experts, cfg.n_groups, cfg.top_k,
+                               cfg.top_groups, gate_affinity=oga)
+    same(e, oe, "expert_idx"), same(g, og, "gates"), same(grp, ogrp, "group_idx")
+    return e, g, oe, og
+
+
+def _np_rows(x):
+    return to_np(x)
+
+
+def _expert_scale(cfg, u_node, r_idx, slot_idx, places, n_places):
+    """(global expert id + 1) / E for the row sitting at each place of the expert-order buffer."""
+    e = u_node[r_idx] * cfg.slots + slot_idx
+    scale = np.zeros(n_places, dtype=np.float32)
+    ok = places >= 0
+    scale[places[ok]] = ((e[ok] + 1).astype(np.float32) / np.float32(cfg.n_experts))
+    return scale
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_reduced_size_every_plane_matches_oracle(name):
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, twolevel_combine
+    cfg = configs.CONFIGS[name].scaled(1536)
+    announce("reduced", cfg.name, cfg.T)
+    inp = configs.make_inputs(cfg)
+    e, g32, oe, og = _route(cfg, inp)
+    gates = g32.to(cfg.gate_dtype)
+    ogates = to_np(gates)
+    x = inp["x"].to(DEV)
+    ox = _np_rows(inp["x"])
+    cap = cfg.capacity(cfg.slots)
+    st = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    # ---- send side
+    payload, mask, gate_rows, u_src, counts = orc.k2_pack(ox, oe, ogates, cfg.world, cfg.n_experts, cfg.rpn,
+                                                          cfg.top_groups)
+    same(st.payload, payload, "payload"), same(st.mask, mask, "mask"), same(st.gate_rows, gate_rows, "gate_rows")
+    same(st.u_src, u_src, "u_src"), same(st.node_counts, counts, "node_counts")
+    _, u_node, _, inverse = orc.plan_ta2a(oe, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups)
+    same(st.extras["u_node"], u_node, "u_node"), same(st.extras["inverse"], inverse, "inverse")
+    same(st.extras["node_offsets"], orc.send_offsets(counts), "node_offsets")
+    assert st.extras["status"].tolist() == [0, cfg.send_rows, 0, 0]
+    # ---- arrival
+    send, gp, r_idx, s_idx, i_send = orc.k1_arrival(payload, mask, gate_rows, cfg.quota, cfg.epr, cfg.rpn)
+    same(st.send_buf, send, "send_buf"), same(st.gate_pairs, gp, "gate_pairs"), same(st.r_idx, r_idx, "r_idx")
+    same(st.slot_idx, s_idx, "slot_idx"), same(st.i_send, i_send, "i_send")
+    pos = orc.arrival_positions(mask, cfg.epr, cfg.rpn)
+    same(st.pair_pos, pos, "pair_pos")
+    # ---- regroup (+ capacity)
+    if cap is None:
+        perm, order, tpe = orc.regroup(send, s_idx, cfg.slots)
+        place = np.empty_like(order)
+        place[order] = np.arange(order.size)
+    else:
+        perm, place, kept, tpe, kpe = orc.regroup(send, s_idx, cfg.slots, capacity=cap)
+        same(st.kept, kept, "kept")
+        assert 0 < kept.sum() < kept.size, "the skewed workload must overflow some expert but not all"
+    same(st.permuted, perm, "permuted"), same(st.place, place, "place"), same(st.tokens_per_expert, tpe, "tokens_per_expert")
+    # ---- experts: row * (expert id + 1) / E, or fresh fp8 rows for the fp8 workload
+    n_places = perm.shape[0]
+    if cfg.fmt == "fp8":
+        gq = torch.Generator().manual_seed(7)
+        ye_rows = orc.fp8_quantise_rows(torch.randn(n_places, cfg.hidden, generator=gq).numpy())
+        ye = torch.from_numpy(ye_rows).to(DEV)
+        fmt_in, hid = "fp8", cfg.hidden
+    else:
+        scale = _expert_scale(cfg, u_node, r_idx, s_idx, place, n_places)
+        dec = orc.decode_rows(perm, cfg.fmt)
+        ye_rows = orc.encode_rows((dec * scale[:, None]).astype(np.float32), cfg.fmt)
+        ye = (st.permuted.float() * torch.from_numpy(scale).to(DEV)[:, None]).to(st.permuted.dtype)
+        same(ye, ye_rows, "expert output")
+        fmt_in, hid = cfg.fmt, None
+    # ---- combine, fused
+    out_fmt = "f32" if cfg.fmt == "f32" else "bf16"
+    pair_tab, sort_order = orc.token_pair_table(oe, inverse, cfg.quota)
+    where = np.where(pos[pair_tab] >= 0, place[pos[pair_tab]], -1)
+    w_sorted = np.take_along_axis(ogates, sort_order, 1)
+    wf = orc.decode_rows(w_sorted, "f32" if cfg.fmt == "f32" else "bf16")
+    want = orc.combine(ye_rows, where, wf, fmt_in, out_fmt, hidden=cfg.hidden)
+    got = loopback_combine(ye, st, out_dtype=cfg.out_dtype, fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None)
+    same(got, want, "combine")
+    # ---- the stated tolerance against float64
+    src64 = orc.decode_rows(ye_rows, fmt_in, cfg.hidden).astype(np.float64)
+    ref = np.zeros((cfg.T, cfg.hidden))
+    for j in range(cfg.top_k):
+        ok = where[:, j] >= 0
+        ref += np.where(ok[:, None], src64[np.where(ok, where[:, j], 0)] * wf[:, j:j + 1].astype(np.float64), 0.0)
+    err = np.abs(orc.decode_rows(to_np(got), out_fmt) - ref).max() / (np.abs(ref).max() + 1e-30)
+    assert err <= TOL[cfg.fmt], err
+    # ---- the reference's two-level shape agrees with the fused one to the same tolerance
+    if cfg.fmt != "fp8":
+        two = twolevel_combine(ye, st, out_dtype=cfg.out_dtype)
+        err2 = np.abs(orc.decode_rows(to_np(two), out_fmt) - ref).max() / (np.abs(ref).max() + 1e-30)
+        assert err2 <= 2 * TOL[cfg.fmt], err2
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_full_size_index_planes_and_round_trip(name):
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    cfg = configs.CONFIGS[name]
+    announce("full", cfg.name, cfg.T)
+    inp = configs.make_inputs(cfg)
+    e, g32, oe, og = _route(cfg, inp)
+    gates = g32.to(cfg.gate_dtype)
+    x = inp["x"].to(DEV)
+    cap = cfg.capacity(cfg.slots)
+    st = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    u_src, u_node, counts, inverse = orc.plan_ta2a(oe, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups)
+    mask, gate_rows = orc.pack_quota_wire(oe, to_np(gates), inverse, cfg.send_rows, cfg.slots, cfg.quota)
+    same(st.u_src, u_src, "u_src"), same(st.node_counts, counts, "node_counts"), same(st.mask, mask, "mask")
+    same(st.gate_rows, gate_rows, "gate_rows"), same(st.extras["inverse"], inverse, "inverse")
+    assert int(counts.sum()) == cfg.send_rows and st.extras["status"].tolist() == [0, cfg.send_rows, 0, 0]
+    assert torch.equal(st.payload, x[st.u_src]), "payload rows are not the rows u_src names"
+    flat = mask.reshape(-1)
+    ordo = orc.stable_argsort_small(flat // cfg.epr, cfg.rpn)
+    same(st.r_idx, ordo // cfg.quota, "r_idx"), same(st.slot_idx, flat[ordo], "slot_idx")
+    same(st.i_send, orc.fixed_hist(flat // cfg.epr, cfg.rpn), "i_send")
+    same(st.gate_pairs, gate_rows.reshape(-1)[ordo], "gate_pairs")
+    assert torch.equal(st.send_buf, st.payload[st.r_idx]), "send_buf rows are not the rows r_idx names"
+    s_idx = flat[ordo]
+    tpe = orc.fixed_hist(s_idx, cfg.slots)
+    same(st.tokens_per_expert, tpe, "tokens_per_expert")
+    order = orc.stable_argsort_small(s_idx, cfg.slots)
+    if cap is None:
+        place = np.empty_like(order)
+        place[order] = np.arange(order.size)
+        same(st.place, place, "place")
+        assert torch.equal(st.permuted, st.send_buf[torch.from_numpy(order).to(DEV)])
+        kept_gate_sum = None
+    else:
+        start = orc.send_offsets(tpe)
+        rank = np.empty_like(order)
+        rank[order] = np.arange(order.size) - start[s_idx[order]]
+        kept = rank < cap
+        place = np.where(kept, s_idx * cap + rank, -1)
+        same(st.place, place, "place"), same(st.kept, kept, "kept")
+        dropped = int((~kept).sum())
+        assert 0 < dropped < kept.size
+        pk = torch.from_numpy(place[kept]).to(DEV)
+        assert torch.equal(st.permuted[pk], st.send_buf[torch.from_numpy(np.flatnonzero(kept)).to(DEV)])
+        used = torch.zeros(st.permuted.shape[0], dtype=torch.bool, device=DEV)
+        used[pk] = True
+        assert not st.permuted[~used].any(), "capacity padding rows must be zero"
+    # ---- round trip with identity experts: y[t] = x[t] * (sum of the token's kept gates)
+    got = loopback_combine(st.permuted, st, out_dtype=cfg.out_dtype,
+                           fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None).float()
+    pos = np.empty_like(ordo)
+    pos[ordo] = np.arange(ordo.size)
+    pair_tab, sort_order = orc.token_pair_table(oe, inverse, cfg.quota)
+    live = torch.from_numpy(place[pos[pair_tab]] >= 0).to(DEV)
+    gsum = (st.extras["gate_sorted"].float() * live).sum(-1, keepdim=True)
+    if cfg.fmt == "fp8":
+        xf = torch.from_numpy(orc.fp8_dequantise_rows(inp["x"][:4096].numpy(), cfg.hidden)).to(DEV)
+        got, gsum = got[:4096], gsum[:4096]
+    else:
+        xf = x.float()
+    err = ((got - xf * gsum).abs().max() / xf.abs().max()).item()
+    assert err <= 2 * TOL[cfg.fmt], err
