@@ -29,6 +29,10 @@ for _p in (ROOT, os.path.join(ROOT, "terracemoe-simulator_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of a workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE and scaled by the same counters' reading for the copy kernel (fetch x2.00,
+# write x1.00).  Only workloads that have been measured are listed; others report null.
+MEASURED_TRAFFIC_BYTES = {("c2", "gather_rows_kernel(regroup)"): 3.769e9}
 REFERENCE_TARGET_US_PER_ROW = 0.012     # the reference's fused-chain design target
 
 
@@ -39,7 +43,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=2048)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1 << 20,
+                    help="tokens of the workload the CPU baseline runs on (default: all of them)")
     return ap.parse_args()
 
 
@@ -57,62 +62,81 @@ def event_ms(fn, reps, torch):
 
 
 def cpu_baseline(cfg, sample_tokens):
-    """The CPU oracle (a numpy restatement of the reference chain) on `sample_tokens` tokens of
-    the same geometry; returns algorithmic GB/s over the same stage set and the stage seconds."""
+    """The CPU oracle timed on the host cores over `sample_tokens` tokens of the same geometry:
+    the OpenMP C restatement (oracle/terrace_oracle.c) when its library is built, else the numpy
+    one.  Best of three passes; algorithmic GB/s over the same stage set as the GPU figure."""
     import numpy as np
+    import torch
+    from oracle import c_oracle as corc
     from oracle import terrace_oracle as orc
     from terrace import configs
-    small = cfg.scaled(min(sample_tokens, cfg.T))
+    use_c = corc.available()
+    small = cfg.scaled(min(sample_tokens if use_c else min(sample_tokens, 1024), cfg.T))
     inp = configs.make_inputs(small)
     logits, bias = inp["logits"].numpy(), inp["bias"].numpy()
     ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].numpy()
     if small.fmt == "f32":
         x, gcast, fmt = inp["x"].numpy(), (lambda g: g), "f32"
     elif small.fmt == "bf16":
-        x, gcast, fmt = inp["x"].view(__import__("torch").int16).numpy().view(np.uint16), orc.f32_to_bf16, "bf16"
+        x, gcast, fmt = inp["x"].view(torch.int16).numpy().view(np.uint16), orc.f32_to_bf16, "bf16"
     else:
         x, gcast, fmt = inp["x"].numpy(), orc.f32_to_bf16, "fp8"
+    impl = corc if use_c else orc
     best = None
-    for _attempt in range(2):          # the second pass runs on warm pages
-        t = _oracle_pass(orc, np, small, logits, bias, ga, x, gcast, fmt)
+    for _attempt in range(3):          # later passes run on warm pages
+        t = _oracle_pass(impl, orc, np, small, logits, bias, ga, x, gcast, fmt, use_c)
         best = t if best is None else {k: min(best[k], t[k]) for k in t}
     t = best
     nbytes = sum(configs.algorithmic_bytes(small).values())
     total = sum(t.values())
-    return {"value": round(nbytes / total / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"numpy oracle, whole path on {small.T} of {cfg.T} tokens of {cfg.name} "
-                      f"({total:.2f} s: " + ", ".join(f"{k} {v:.2f}" for k, v in t.items()) + ")",
+    cores = corc.threads() if use_c else 1
+    what = f"OpenMP C oracle ({cores} threads)" if use_c else "numpy oracle (1 thread)"
+    return {"value": round(nbytes / total / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{what}, whole path on {small.T} of {cfg.T} tokens of {cfg.name}, best of 3 passes "
+                      f"({total:.3f} s: " + ", ".join(f"{k} {v:.3f}" for k, v in t.items()) + ")",
             "arrival_us_per_row": round(t["arrival"] * 1e6 / small.pairs, 4)}
 
 
-def _oracle_pass(orc, np, small, logits, bias, ga, x, gcast, fmt):
+def _oracle_pass(impl, orc, np, small, logits, bias, ga, x, gcast, fmt, use_c):
     t = {}
     t0 = time.perf_counter()
-    e, gates, _ = orc.t_route(logits, bias, small.n_experts, small.n_groups, small.top_k, small.top_groups,
-                              gate_affinity=ga)
+    if use_c:
+        e, gates, _ = impl.t_route(logits, bias, small.n_experts, small.n_groups, small.top_k, small.top_groups,
+                                   2, ga)
+    else:
+        e, gates, _ = impl.t_route(logits, bias, small.n_experts, small.n_groups, small.top_k, small.top_groups,
+                                   gate_affinity=ga)
     t["route"] = time.perf_counter() - t0
+    gq = gcast(gates)
     t0 = time.perf_counter()
-    payload, mask, gate_rows, u_src, counts = orc.k2_pack(x, e, gcast(gates), small.world, small.n_experts,
-                                                          small.rpn, small.top_groups)
+    packed = impl.k2_pack(x, e, gq, small.world, small.n_experts, small.rpn, small.top_groups)
+    payload, mask, gate_rows = packed[0], packed[1], packed[2]
     t["pack"] = time.perf_counter() - t0
     t0 = time.perf_counter()
-    send, gp, r_idx, s_idx, i_send = orc.k1_arrival(payload, mask, gate_rows, small.quota, small.epr, small.rpn)
+    arrived = impl.k1_arrival(payload, mask, gate_rows, small.quota, small.epr, small.rpn)
+    send, s_idx = arrived[0], arrived[3]
     t["arrival"] = time.perf_counter() - t0
     t0 = time.perf_counter()
     cap = small.capacity(small.slots)
-    if cap is None:
-        perm, order, tpe = orc.regroup(send, s_idx, small.slots)
+    if use_c:
+        perm, place, _kept, _tpe = impl.regroup(send, s_idx, small.slots, 0, cap)
+    elif cap is None:
+        perm, order, _tpe = impl.regroup(send, s_idx, small.slots)
         place = np.empty_like(order)
         place[order] = np.arange(order.size)
     else:
-        perm, place, kept, tpe, kpe = orc.regroup(send, s_idx, small.slots, capacity=cap)
+        perm, place, _kept, _tpe, _kpe = impl.regroup(send, s_idx, small.slots, capacity=cap)
     t["regroup"] = time.perf_counter() - t0
     t0 = time.perf_counter()
-    _, _, _, inverse = orc.plan_ta2a(e, small.world, small.n_experts, small.rpn, small.top_groups)
-    pair_tab, sort_order = orc.token_pair_table(e, inverse, small.quota)
-    where = place[orc.arrival_positions(mask, small.epr, small.rpn)[pair_tab]]
-    orc.combine(perm, where, np.take_along_axis(gates, sort_order, 1), fmt, "f32" if fmt == "f32" else "bf16",
-                hidden=small.hidden)
+    if use_c:
+        pair_tab, sort_order, pos = packed[5]["pair_table"], packed[5]["sort_order"], arrived[5]
+    else:
+        _, _, _, inverse = orc.plan_ta2a(e, small.world, small.n_experts, small.rpn, small.top_groups)
+        pair_tab, sort_order = orc.token_pair_table(e, inverse, small.quota)
+        pos = orc.arrival_positions(mask, small.epr, small.rpn)
+    where = place[pos[pair_tab]]
+    w_sorted = np.take_along_axis(gates, sort_order, 1)
+    impl.combine(perm, where, w_sorted, fmt, "f32" if fmt == "f32" else "bf16", hidden=small.hidden)
     t["combine"] = time.perf_counter() - t0
     return t
 
@@ -238,7 +262,8 @@ def main():
     dominant = max((k for k in kern if not k.startswith("copy")), key=lambda k: kern[k]["ms"])
     achieved = kern[dominant]["GBps"]
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)),
                 "avg_launch_ms": kern[dominant]["ms"], "algorithmic_bytes_per_launch": kern[dominant]["algorithmic_bytes"]}
 
     total_bytes = sum(nbytes.values())
