@@ -197,6 +197,22 @@ TERRACE_API int terrace_combine(const void *src, int src_dtype, const int64_t *i
                     int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
                     terrace_stream_t stream);
 
+/* Wire containers (terrace/ta2a_pack.py:319-336 hopa_pack, :398-414 hopa_pack_small, :474-497
+ * hopb_pack_meta): each out row of row_bytes is plane a's row, then b's, then c's, then zeros.
+ * A NULL plane is absent (its width counts as 0).  Pure byte moves.
+ *   Hop-A full:  a = ids [n, id_w] i64, b = payload [n, H], c = gates [n, gw]; row = W*8 bytes
+ *   Hop-A small: a = ids, b = gates;  Hop-B meta: a = slot ids [P] i64, b = gates [P]; row = 16 */
+TERRACE_API int terrace_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c,
+                                    int64_t c_bytes, int64_t n_rows, int64_t row_bytes, void *out,
+                                    terrace_stream_t stream);
+
+/* The inverse (hopa_unpack :339-356, hopa_unpack_small :417-423, hopb_unpack_meta :500-503): row
+ * bytes [0, a_bytes) go to a, the next b_bytes to b, the next c_bytes to c; each destination is a
+ * dense plane of its own (never a view of the container); a NULL destination is skipped. */
+TERRACE_API int terrace_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, void *a,
+                                      int64_t a_bytes, void *b, int64_t b_bytes, void *c, int64_t c_bytes,
+                                      terrace_stream_t stream);
+
 /* Hop-A counts exchange buffer (terrace/ta2a_dispatch.py:197-211): send [world] i64 is zero
  * except send[n*rpn + my_local] = node_counts[n]. */
 TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local,

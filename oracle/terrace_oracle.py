@@ -495,3 +495,49 @@ def token_pair_table(expert_idx, inverse, quota):
     order = np.argsort(e, axis=1, kind="stable")
     rows = np.take_along_axis(np.asarray(inverse).reshape(T, k), order, 1)
     return rows * quota + (np.arange(k)[None, :] % quota), order
+
+
+# --------------------------------------------------------------------------------------
+# wire containers -- terrace/ta2a_pack.py:276-506
+# --------------------------------------------------------------------------------------
+
+
+def container_words(id_w, hidden, gate_w, itemsize):
+    """Row width in int64 words: the id plane, then just enough words for hidden+gate_w
+    elements (terrace/ta2a_pack.py:287-288; hidden = 0 gives the small layout, :380-381)."""
+    per_word = 8 // itemsize
+    return id_w + -(-(hidden + gate_w) // per_word)
+
+
+def pack_planes(planes, n_rows, row_bytes):
+    """Byte-level container: each row is the planes' rows back to back, then zeros.
+    hopa_pack (:319-336) = (ids, payload, gates); hopa_pack_small (:398-414) = (ids, gates);
+    hopb_pack_meta (:474-497) = (slot ids, gates) with row_bytes = 16."""
+    out = np.zeros((n_rows, row_bytes), dtype=np.uint8)
+    at = 0
+    for p in planes:
+        b = np.ascontiguousarray(p).reshape(n_rows, -1).view(np.uint8) if n_rows else np.zeros((0, 0), np.uint8)
+        if n_rows:
+            out[:, at:at + b.shape[1]] = b
+            at += b.shape[1]
+    return out.view(np.int64) if row_bytes % 8 == 0 else out
+
+
+def unpack_planes(buf, specs):
+    """Inverse: specs = [(dtype, elements per row), ...] consecutive from the row head
+    (hopa_unpack :339-356, hopa_unpack_small :417-423, hopb_unpack_meta :500-503)."""
+    raw = np.ascontiguousarray(buf).view(np.uint8).reshape(buf.shape[0], -1)
+    out, at = [], 0
+    for dtype, width in specs:
+        nbytes = np.dtype(dtype).itemsize * width
+        out.append(np.ascontiguousarray(raw[:, at:at + nbytes]).view(dtype).reshape(buf.shape[0], width))
+        at += nbytes
+    return out
+
+
+def hopa_send_splits(node_counts, world, rpn, my_local):
+    """terrace/ta2a_dispatch.py:197-211 -- length-`world` send counts, node n's rows go to its
+    designated peer n*rpn + my_local, every other entry is zero."""
+    send = np.zeros(world, dtype=np.int64)
+    send[np.arange(world // rpn) * rpn + my_local] = np.asarray(node_counts, dtype=np.int64)
+    return send

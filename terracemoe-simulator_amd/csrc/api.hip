@@ -8,6 +8,10 @@ int launch_combine(const void *src, int src_dtype, const int64_t *idx, const voi
 int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
 int launch_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
                         hipStream_t s);
+int launch_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,
+                       int64_t n_rows, int64_t row_bytes, void *out, hipStream_t s);
+int launch_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, void *a, int64_t a_bytes, void *b,
+                         int64_t b_bytes, void *c, int64_t c_bytes, hipStream_t s);
 int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s);
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
@@ -167,6 +171,24 @@ int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const vo
     if (n_out && hidden && (!src || !idx || !out)) return TERRACE_EINVAL;
     return launch_combine(src, src_dtype, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
                           (hipStream_t)stream);
+}
+
+int terrace_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,
+                        int64_t n_rows, int64_t row_bytes, void *out, terrace_stream_t stream) {
+    if (n_rows < 0 || a_bytes < 0 || b_bytes < 0 || c_bytes < 0) return TERRACE_EINVAL;
+    const int64_t used = (a ? a_bytes : 0) + (b ? b_bytes : 0) + (c ? c_bytes : 0);
+    if (row_bytes < used || (n_rows && row_bytes && !out)) return TERRACE_EINVAL;
+    // an absent plane must not leave a hole in front of a present one
+    if ((!a && a_bytes && (b || c)) || (!b && b_bytes && c)) return TERRACE_EINVAL;
+    return launch_pack_planes(a, a_bytes, b, b_bytes, c, c_bytes, n_rows, row_bytes, out, (hipStream_t)stream);
+}
+
+int terrace_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, void *a, int64_t a_bytes, void *b,
+                          int64_t b_bytes, void *c, int64_t c_bytes, terrace_stream_t stream) {
+    if (n_rows < 0 || a_bytes < 0 || b_bytes < 0 || c_bytes < 0 || row_bytes < a_bytes + b_bytes + c_bytes)
+        return TERRACE_EINVAL;
+    if (n_rows && row_bytes && !packed) return TERRACE_EINVAL;
+    return launch_unpack_planes(packed, row_bytes, n_rows, a, a_bytes, b, b_bytes, c, c_bytes, (hipStream_t)stream);
 }
 
 int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send,

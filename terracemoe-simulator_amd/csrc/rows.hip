@@ -297,6 +297,73 @@ __global__ __launch_bounds__(kBlock) void combine_elem_kernel(const uint8_t *__r
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// wire containers: out row = a | b | c | zero pad, and the inverse split
+// (the int64-word rows of the reference's terrace/ta2a_pack.py:319-336,398-414,474-497)
+// ---------------------------------------------------------------------------------------------
+struct Planes {
+    const uint8_t *src[3];
+    uint8_t *dst[3];
+    int64_t bytes[3];       // per-row width of each plane (0 = absent)
+};
+
+template <typename V, bool PACK>
+__global__ __launch_bounds__(kBlock) void planes_kernel(Planes pl, uint8_t *__restrict__ packed, int64_t row_bytes,
+                                                        int64_t n_rows) {
+    const int64_t vecs = row_bytes / (int64_t)sizeof(V);
+    const int64_t a = pl.bytes[0], ab = a + pl.bytes[1], abc = ab + pl.bytes[2];
+    for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < n_rows * vecs;
+         g += (int64_t)gridDim.x * kBlock) {
+        const int64_t row = g / vecs, off = (g - row * vecs) * (int64_t)sizeof(V);
+        V *cell = (V *)(packed + row * row_bytes + off);
+        int which = -1;
+        int64_t inner = 0;
+        if (off < a) { which = 0; inner = off; }
+        else if (off < ab) { which = 1; inner = off - a; }
+        else if (off < abc) { which = 2; inner = off - ab; }
+        if constexpr (PACK) {
+            *cell = which < 0 ? zero_of<V>() : *(const V *)(pl.src[which] + row * pl.bytes[which] + inner);
+        } else {
+            if (which >= 0 && pl.dst[which]) *(V *)(pl.dst[which] + row * pl.bytes[which] + inner) = *cell;
+        }
+    }
+}
+
+template <bool PACK>
+static int launch_planes(const Planes &pl, void *packed, int64_t row_bytes, int64_t n_rows, hipStream_t s) {
+    if (n_rows <= 0 || row_bytes <= 0) return TERRACE_OK;
+    uintptr_t bits = (uintptr_t)packed | (uintptr_t)row_bytes;
+    for (int i = 0; i < 3; ++i) {
+        if (!pl.bytes[i]) continue;
+        bits |= (uintptr_t)pl.bytes[i] | (uintptr_t)(PACK ? (const void *)pl.src[i] : (const void *)pl.dst[i]);
+    }
+    int64_t blocks;
+#define TERRACE_PLANES(V)                                                          \
+    blocks = (n_rows * (row_bytes / (int64_t)sizeof(V)) + kBlock - 1) / kBlock;    \
+    if (blocks > ((int64_t)1 << 22)) blocks = (int64_t)1 << 22;                    \
+    planes_kernel<V, PACK><<<(unsigned)blocks, kBlock, 0, s>>>(pl, (uint8_t *)packed, row_bytes, n_rows)
+    if ((bits & 15) == 0) { TERRACE_PLANES(u32x4); }
+    else if ((bits & 7) == 0) { TERRACE_PLANES(u32x2); }
+    else if ((bits & 3) == 0) { TERRACE_PLANES(uint32_t); }
+    else if ((bits & 1) == 0) { TERRACE_PLANES(uint16_t); }
+    else { TERRACE_PLANES(uint8_t); }
+#undef TERRACE_PLANES
+    return check_launch();
+}
+
+int launch_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,
+                       int64_t n_rows, int64_t row_bytes, void *out, hipStream_t s) {
+    Planes pl{{(const uint8_t *)a, (const uint8_t *)b, (const uint8_t *)c}, {nullptr, nullptr, nullptr},
+              {a ? a_bytes : 0, b ? b_bytes : 0, c ? c_bytes : 0}};
+    return launch_planes<true>(pl, out, row_bytes, n_rows, s);
+}
+
+int launch_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, void *a, int64_t a_bytes, void *b,
+                         int64_t b_bytes, void *c, int64_t c_bytes, hipStream_t s) {
+    Planes pl{{nullptr, nullptr, nullptr}, {(uint8_t *)a, (uint8_t *)b, (uint8_t *)c}, {a_bytes, b_bytes, c_bytes}};
+    return launch_planes<false>(pl, (void *)packed, row_bytes, n_rows, s);
+}
+
 __global__ __launch_bounds__(kBlock) void index_chain_kernel(const int64_t *__restrict__ table,
                                                              const int64_t *__restrict__ idx, int64_t n,
                                                              int64_t *__restrict__ out) {

@@ -51,6 +51,8 @@ SIGNATURES = {
     "terrace_index_chain": (_I, [_P, _P, _L, _P, _P]),
     "terrace_index_chain2": (_I, [_P, _P, _P, _L, _P, _P]),
     "terrace_combine": (_I, [_P, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
+    "terrace_pack_planes": (_I, [_P, _L, _P, _L, _P, _L, _L, _L, _P, _P]),
+    "terrace_unpack_planes": (_I, [_P, _L, _L, _P, _L, _P, _L, _P, _L, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
 }
 

@@ -479,3 +479,61 @@ def test_gather_rows_and_index_chain():
     idx = torch.randint(-1, 100, (4, 7), generator=g)
     want = torch.where(idx < 0, torch.full_like(idx, -1), table[idx.clamp(min=0)])
     assert torch.equal(tops.index_chain(table.to(DEV), idx.to(DEV)).cpu(), want)
+
+
+# ------------------------------------------------------------------------------- wire containers
+
+HOPA_GEOMS = [(5, 6, 2, 2), (5, 6, 4, 1), (1, 7, 3, 3), (17, 2048, 3, 3), (4, 5, 1, 1), (3, 24, 24, 1),
+              (9, 2048, 24, 1), (0, 16, 2, 2), (1000, 7168, 2, 2)]
+
+
+@pytest.mark.parametrize("geom", HOPA_GEOMS, ids=lambda g: "n%dh%dg%di%d" % g)
+@pytest.mark.parametrize("fmt", ["f32", "bf16"])
+def test_hopa_containers_round_trip_bitwise(geom, fmt):
+    from terrace import ta2a_pack as pk
+    n, hidden, gate_w, id_w = geom
+    announce("hopa container", geom, fmt)
+    g = torch.Generator().manual_seed(1000 + n * 31 + hidden + id_w)
+    payload = rows_of(torch.randn(n, hidden, generator=g), fmt)
+    gate = rows_of(torch.rand(n, gate_w, generator=g), fmt)
+    ids = torch.randint(0, 1 << 40, (n,), generator=g) if id_w == 1 else torch.randint(0, 24, (n, id_w), generator=g)
+    es = payload.element_size()
+    buf, lay = pk.hopa_pack(payload.to(DEV), gate.to(DEV), ids.to(DEV))
+    assert buf.shape == (n, lay.words) and buf.dtype == torch.int64 and buf.is_contiguous()
+    assert lay.id_w == id_w and lay.id_1d is (ids.dim() == 1) and lay.words == orc.container_words(id_w, hidden, gate_w, es)
+    want = orc.pack_planes([ids.numpy().reshape(n, id_w), to_np(payload), to_np(gate)], n, lay.words * 8)
+    same(buf, want.reshape(n, lay.words), "hopa container")
+    p2, g2, i2 = pk.hopa_unpack(buf, lay)
+    assert torch.equal(p2.cpu(), payload) and torch.equal(g2.cpu(), gate) and torch.equal(i2.cpu(), ids)
+    assert p2.is_contiguous() and g2.is_contiguous() and i2.is_contiguous() and i2.shape == ids.shape
+    pk.assert_not_aliased(buf, p2, g2, i2)
+    sbuf, slay = pk.hopa_pack_small(gate.to(DEV), ids.to(DEV))
+    assert slay.words == orc.container_words(id_w, 0, gate_w, es)
+    same(sbuf, orc.pack_planes([ids.numpy().reshape(n, id_w), to_np(gate)], n, slay.words * 8).reshape(n, slay.words),
+         "hopa small container")
+    g3, i3 = pk.hopa_unpack_small(sbuf, slay)
+    assert torch.equal(g3.cpu(), gate) and torch.equal(i3.cpu(), ids)
+
+
+def test_hopb_meta_and_container_errors():
+    from terrace import ta2a_pack as pk
+    announce("hopb meta")
+    g = torch.Generator().manual_seed(3)
+    for P in (0, 1, 7, 24576):
+        for fmt in ("f32", "bf16"):
+            slot = torch.randint(0, 63, (P,), generator=g)
+            gate = rows_of(torch.rand(P, generator=g), fmt)
+            buf = pk.hopb_pack_meta(slot.to(DEV), gate.to(DEV))
+            assert buf.shape == (P, 2) and buf.dtype == torch.int64 and pk.hopb_meta_words() == 2
+            same(buf, orc.pack_planes([slot.numpy(), to_np(gate)], P, 16).reshape(P, 2), "hopb meta")
+            s2, g2 = pk.hopb_unpack_meta(buf, gate.dtype)
+            assert torch.equal(s2.cpu(), slot) and torch.equal(g2.cpu(), gate)
+    ids = torch.tensor([0, 1, (1 << 62) + 12345, -1, (1 << 63) - 1], device=DEV)
+    buf, lay = pk.hopa_pack(torch.randn(5, 6, device=DEV).bfloat16(), torch.rand(5, 3, device=DEV).bfloat16(), ids)
+    assert torch.equal(pk.hopa_unpack(buf, lay)[2], ids)
+    with pytest.raises(RuntimeError, match="dtype"):
+        pk.hopa_pack(torch.zeros(2, 4, device=DEV), torch.zeros(2, 2, device=DEV).bfloat16(), ids[:2])
+    with pytest.raises(RuntimeError, match="int64"):
+        pk.hopa_pack_small(torch.zeros(2, 2, device=DEV), ids[:2].int())
+    with pytest.raises(RuntimeError, match="shape"):
+        pk.hopb_pack_meta(ids[:2], torch.zeros(3, device=DEV))

@@ -184,3 +184,24 @@ def test_plan_guard_messages_from_status_words():
     with pytest.raises(ValueError, match="out of range"):
         ta2a._raise_from_status(st, 4, 4, 2)
     ta2a._raise_from_status(torch.tensor([0, 8, 0, 0], dtype=torch.int32), 4, 4, 2)
+
+
+def test_pack_mode_switch(monkeypatch):
+    from terrace import ta2a_pack as pk
+    monkeypatch.delenv("TERRACE_TA2A_PACK", raising=False)
+    pk.reset()
+    assert pk.pack_mode() == "small" and pk.pack_enabled()
+    for raw, mode in [("0", "off"), ("1", "small"), ("full", "full"), ("2", "full"), ("meta", "small")]:
+        monkeypatch.setenv("TERRACE_TA2A_PACK", raw)
+        pk.reset()
+        assert pk.pack_mode() == mode
+    monkeypatch.setenv("TERRACE_TA2A_PACK", "ful")
+    pk.reset()
+    with pytest.raises(RuntimeError, match="not a valid mode"):
+        pk.pack_mode()
+    monkeypatch.delenv("TERRACE_TA2A_PACK")
+    pk.reset()
+    monkeypatch.setattr(pk, "pack_enabled", lambda: False)
+    assert pk.pack_mode() == "off"
+    lay = pk.HopALayout(2048, 3, 3, False, torch.bfloat16)
+    assert lay.words == 516 and pk.HopASmallLayout(3, 3, False, torch.bfloat16).words == 4

@@ -446,3 +446,43 @@ def test_combine_formats():
     got8 = orc.combine(rows8, idx, w, "fp8", "f32", hidden=256)
     assert np.allclose(got8, ref, rtol=0.15, atol=0.15)
     assert np.array_equal(orc.combine(src, idx, w), ref)
+
+
+# ----------------------------------------------------------------------------- containers
+
+def test_container_widths_match_reference_literals():
+    # verdict geometry of the reference: H=2048 bf16, quota 3 -> 516 words full, 4 words small, 2 words Hop B
+    assert orc.container_words(3, 2048, 3, 2) == 516
+    assert orc.container_words(3, 0, 3, 2) == 4
+    assert orc.container_words(1, 0, 1, 2) == 2 and orc.container_words(1, 0, 1, 4) == 2
+
+
+def test_container_layout_and_round_trip():
+    rng = np.random.default_rng(9)
+    for n, hidden, gate_w, id_w in [(5, 6, 2, 2), (5, 6, 4, 1), (1, 7, 3, 3), (17, 2048, 3, 3), (4, 5, 1, 1),
+                                    (3, 24, 24, 1), (9, 2048, 24, 1)]:            # tests/test_ta2a_pack_bitparity.py:100-101
+        for dt in (np.float32, np.uint16):
+            es = np.dtype(dt).itemsize
+            payload = rng.integers(0, 60000, (n, hidden)).astype(dt)
+            gate = rng.integers(0, 60000, (n, gate_w)).astype(dt)
+            ids = rng.integers(0, 1 << 40, (n, id_w)).astype(np.int64)
+            words = orc.container_words(id_w, hidden, gate_w, es)
+            buf = orc.pack_planes([ids, payload, gate], n, words * 8)
+            assert buf.shape == (n, words) and buf.dtype == np.int64
+            assert np.array_equal(buf[:, :id_w], ids)                       # id plane leads the row
+            flat = buf.view(dt)
+            base = id_w * (8 // es)
+            assert np.array_equal(flat[:, base:base + hidden], payload)
+            assert np.array_equal(flat[:, base + hidden:base + hidden + gate_w], gate)
+            assert not flat[:, base + hidden + gate_w:].any()               # zero pad
+            got = orc.unpack_planes(buf, [(np.int64, id_w), (dt, hidden), (dt, gate_w)])
+            assert all(np.array_equal(a, b) for a, b in zip(got, (ids, payload, gate)))
+    wide = np.array([0, 1, (1 << 62) + 12345, -1, (1 << 63) - 1], dtype=np.int64)   # :143-152 full int64 range
+    buf = orc.pack_planes([wide, np.zeros((5, 3), np.uint16)], 5, 16)
+    assert np.array_equal(orc.unpack_planes(buf, [(np.int64, 1)])[0][:, 0], wide)
+
+
+def test_hopa_send_splits_literal(literals):
+    lit = literals["hopa_counts"]
+    send = orc.hopa_send_splits(lit["node_counts"], lit["world"], lit["rpn"], lit["my_local"])
+    assert send.tolist() == lit["send"] and send.dtype == np.int64
