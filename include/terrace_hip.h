@@ -213,6 +213,75 @@ TERRACE_API int terrace_unpack_planes(const void *packed, int64_t row_bytes, int
                                       int64_t a_bytes, void *b, int64_t b_bytes, void *c, int64_t c_bytes,
                                       terrace_stream_t stream);
 
+/* ---- the general (data-dependent fan-out) branch and the seam's entry helper ---- */
+
+/* plan_ta2a without groups_m (terrace/ta2a.py:70-275, general branch): one send row per occupied
+ * (node, token) pair in (node asc, token asc) order, for n_nodes <= 64.  u_src / u_node must hold
+ * T*min(k, n_nodes) entries; the number actually written is sum(counts), which the caller reads
+ * back (the reference pays the same synchronisation at terrace/ta2a.py:148). */
+TERRACE_API size_t terrace_plan_general_workspace(int64_t T, int n_nodes);
+TERRACE_API int terrace_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn,
+                                     int64_t *u_src, int64_t *u_node, int64_t *counts, int64_t *inverse,
+                                     int32_t *status, void *workspace, size_t workspace_bytes,
+                                     terrace_stream_t stream);
+
+/* build_expansion (terrace/ta2a_fwd.py:348-442): mask[inverse[i]] |= 1 << (expert_idx[i] % slots) for
+ * i < n = T*k.  mask [n_rows] i64 must be zero-filled by the caller; slots <= 63. */
+TERRACE_API int terrace_build_mask(const int64_t *expert_idx, const int64_t *inverse, int64_t n, int slots,
+                                   int64_t n_rows, int64_t *mask, int32_t *status, terrace_stream_t stream);
+
+/* out[rows[i]*width + c] = vals[i] (elements of elem_bytes = 2 or 4) with c = cols[i], or cols[i] % col_mod
+ * when col_mod > 0: the sparse gate plane gate_rows[inverse, expert % slots] = gates of
+ * terrace/ta2a_fwd.py:498-500.  out is pre-filled by the caller; cells outside it are skipped. */
+TERRACE_API int terrace_scatter_elems(const void *vals, int elem_bytes, const int64_t *rows, const int64_t *cols,
+                                      int col_mod, int64_t n, int64_t n_rows, int width, void *out,
+                                      terrace_stream_t stream);
+
+/* _expand_arrival (terrace/ta2a_fwd.py:120-174).  With a quota: per row its `quota` lowest set bits
+ * ascending, then, if it has fewer, its unset columns ascending; r_idx / slot_idx hold R*quota.
+ * Without: every set bit, row-major with columns ascending; _count leaves the exclusive offsets in
+ * the workspace and the pair total in n_pairs (device int64, read back by the caller), _fill then
+ * writes the n_pairs entries. */
+TERRACE_API int terrace_expand_mask_quota(const int64_t *rmask, int64_t R, int slots, int quota, int64_t *r_idx,
+                                          int64_t *slot_idx, terrace_stream_t stream);
+TERRACE_API size_t terrace_expand_mask_workspace(int64_t R);
+TERRACE_API int terrace_expand_mask_count(const int64_t *rmask, int64_t R, int slots, int64_t *n_pairs,
+                                          void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+TERRACE_API int terrace_expand_mask_fill(const int64_t *rmask, int64_t R, int slots, int64_t *r_idx,
+                                         int64_t *slot_idx, const void *workspace, terrace_stream_t stream);
+
+/* The arrival chain of the general branch (terrace/ta2a_fwd.py:605-628): the P pairs (r_in[p], slot_in[p])
+ * that terrace_expand_mask_* listed are placed in stable ascending order of slot/epr.  Writes r_idx [P],
+ * slot_idx [P], i_send [rpn], ordo [P] (the source pair of each place; may be NULL), send_buf [P,row_bytes]
+ * = rx[r_idx] (rx NULL: index planes only) and gate_pairs [P] = rgate[r_idx, slot_idx] looked up in the
+ * sparse plane rgate [R, gate_width] (NULL: skipped). */
+TERRACE_API size_t terrace_arrival_pairs_workspace(int64_t P, int rpn);
+TERRACE_API int terrace_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_in, const void *rgate,
+                                      int64_t R, int64_t P, int64_t row_bytes, int gate_bytes, int gate_width, int epr,
+                                      int rpn, void *send_buf, void *gate_pairs, int64_t *r_idx, int64_t *slot_idx,
+                                      int64_t *i_send, int64_t *ordo, int32_t *status, void *workspace,
+                                      size_t workspace_bytes, terrace_stream_t stream);
+
+/* The read side of an index_add (red.index_add_(0, r_idx, ret) and y.index_add(0, u_src, back),
+ * terrace/ta2a_dispatch.py:483-494) when the number of contributions per target varies: table
+ * [n_seg, width] i64 lists, for each target s, the items i < n with seg[i] == s in ascending i, padded
+ * with -1 (width <= 64).  terrace_combine over that table is then the reduction, adding in the same
+ * ascending order.  A target with more than `width` items raises TERRACE_FAULT_FANOUT in status word 0. */
+TERRACE_API size_t terrace_segment_table_workspace(int64_t n_seg);
+TERRACE_API int terrace_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table,
+                                      int32_t *status, void *workspace, size_t workspace_bytes,
+                                      terrace_stream_t stream);
+
+/* routing_map_to_topk (terrace/ta2a_dispatch.py:224-260): routing_map [T,E] bytes (non-zero = chosen).
+ * _count writes row_stats = {min, max} of the per-token counts (int32[2]); after the caller has
+ * checked min == max == k, _topk writes the k chosen expert ids ascending and their probs
+ * (elem_bytes-wide elements of probs [T,E]). */
+TERRACE_API int terrace_routing_map_count(const void *routing_map, int64_t T, int n_experts, int32_t *row_stats,
+                                          terrace_stream_t stream);
+TERRACE_API int terrace_routing_map_topk(const void *routing_map, const void *probs, int elem_bytes, int64_t T,
+                                         int n_experts, int k, int64_t *expert_idx, void *gates,
+                                         terrace_stream_t stream);
+
 /* Hop-A counts exchange buffer (terrace/ta2a_dispatch.py:197-211): send [world] i64 is zero
  * except send[n*rpn + my_local] = node_counts[n]. */
 TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local,

@@ -498,6 +498,91 @@ def token_pair_table(expert_idx, inverse, quota):
 
 
 # --------------------------------------------------------------------------------------
+# general (data-dependent fan-out) branch -- terrace/ta2a_fwd.py:120-174, :348-442, :496-500
+# and the seam's entry helper -- terrace/ta2a_dispatch.py:224-260
+# --------------------------------------------------------------------------------------
+
+
+def build_expansion(expert_idx, inverse, n_rows, world, n_experts, rpn=8):
+    """mask [n_rows] i64: bit j of row r is set iff node-local slot j wants the row.
+
+    terrace/ta2a_fwd.py:348-442.  The reference sums distinct powers of two per row (:440-441,
+    and the structured path :425-438 sums the same set); for distinct experts per token that
+    is the bitwise OR restated here.  ``slots > 63`` raises as at :372-373.
+    """
+    e = np.asarray(expert_idx, dtype=np.int64)
+    slots = (n_experts // world) * rpn
+    if slots > 63:
+        raise ValueError(f"{slots} expert slots per node exceeds the int64 mask")
+    mask = np.zeros(n_rows, dtype=np.int64)
+    np.bitwise_or.at(mask, np.asarray(inverse, dtype=np.int64).reshape(-1),
+                     np.int64(1) << (e.reshape(-1) % slots))
+    return mask
+
+
+def sparse_gate_plane(expert_idx, gates, inverse, n_rows, slots):
+    """gate_rows [n_rows, slots], zero except [inverse[t,j], expert % slots] = gates[t,j]
+    (terrace/ta2a_fwd.py:498-500)."""
+    e = np.asarray(expert_idx, dtype=np.int64).reshape(-1)
+    g = np.asarray(gates)
+    out = np.zeros((n_rows, slots), dtype=g.dtype)
+    out[np.asarray(inverse, dtype=np.int64).reshape(-1), e % slots] = g.reshape(-1)
+    return out
+
+
+def expand_arrival(rmask, slots, quota=None):
+    """(r_idx, slot_idx) demand pairs of the arrived bitmasks (terrace/ta2a_fwd.py:120-174).
+
+    ``quota`` None: every set bit, rows ascending and columns ascending inside a row
+    (``nonzero`` order, :174).  With a quota: exactly ``quota`` columns per row, chosen by the
+    distinct key ``bit*slots + (slots-1-col)`` descending (:165-169), i.e. the set columns
+    ascending first, then -- for a row with fewer -- its unset columns ascending.
+    """
+    rmask = np.asarray(rmask, dtype=np.int64)
+    R = rmask.shape[0]
+    bits = (rmask[:, None] >> np.arange(slots, dtype=np.int64)[None, :]) & 1     # [R, slots]
+    if quota is None:
+        r, c = np.nonzero(bits)
+        return r.astype(np.int64), c.astype(np.int64)
+    key = bits * slots + (slots - 1 - np.arange(slots, dtype=np.int64))[None, :]
+    cols = np.argsort(-key, axis=1, kind="stable")[:, :quota]
+    r_idx = np.repeat(np.arange(R, dtype=np.int64), quota)
+    return r_idx, cols.reshape(-1).astype(np.int64)
+
+
+def arrival_pairs(rx, r_idx, slot_idx, rgate, epr, rpn):
+    """The arrival chain of the general branch (terrace/ta2a_fwd.py:605-628): pairs in stable
+    ascending owner-card order; the gate of a pair is looked up in the sparse plane
+    ``rgate[r, slot]`` after the reorder (:626-627).
+    Returns (send_buf, gate_pairs, r_idx, slot_idx, i_send, ordo)."""
+    r_idx = np.asarray(r_idx, dtype=np.int64)
+    slot_idx = np.asarray(slot_idx, dtype=np.int64)
+    owner = slot_idx // epr
+    ordo = stable_argsort_small(owner, rpn)
+    r2, s2 = r_idx[ordo], slot_idx[ordo]
+    i_send = fixed_hist(owner, rpn)
+    return rx[r2], np.asarray(rgate)[r2, s2], r2, s2, i_send, ordo
+
+
+def routing_map_to_topk(routing_map, probs):
+    """(expert_idx [T,k] i64 ascending per row, gates [T,k] = probs at those columns).
+
+    terrace/ta2a_dispatch.py:224-260: every row must hold the same non-zero number k of set
+    entries, else RuntimeError.
+    """
+    rm = np.asarray(routing_map) != 0
+    counts = rm.sum(1)
+    if counts.size and counts.min() != counts.max():
+        raise RuntimeError("T-A2A requires exactly k experts per token (drop-less); observed per-row "
+                           "expert counts differ")
+    k = int(counts[0]) if counts.size else 0
+    if k == 0:
+        raise RuntimeError("T-A2A got an all-empty routing_map (k=0); impossible under drop-less routing")
+    expert_idx = np.nonzero(rm)[1].reshape(rm.shape[0], k).astype(np.int64)
+    return expert_idx, np.take_along_axis(np.asarray(probs), expert_idx, 1)
+
+
+# --------------------------------------------------------------------------------------
 # wire containers -- terrace/ta2a_pack.py:276-506
 # --------------------------------------------------------------------------------------
 

@@ -45,6 +45,32 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
 int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
                         int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
                         int32_t *status, hipStream_t s);
+size_t plan_general_workspace(int64_t T, int n_nodes);
+int run_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn, int64_t *u_src,
+                     int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status, void *ws, size_t ws_bytes,
+                     hipStream_t s);
+int run_build_mask(const int64_t *expert_idx, const int64_t *inverse, int64_t n, int slots, int64_t n_rows,
+                   int64_t *mask, int32_t *status, hipStream_t s);
+int run_scatter_elems(const void *vals, int elem_bytes, const int64_t *rows, const int64_t *cols, int col_mod,
+                      int64_t n, int64_t n_rows, int width, void *out, hipStream_t s);
+int run_expand_quota(const int64_t *rmask, int64_t R, int slots, int quota, int64_t *r_idx, int64_t *slot_idx,
+                     hipStream_t s);
+size_t expand_workspace(int64_t R);
+int run_expand_count(const int64_t *rmask, int64_t R, int slots, int64_t *n_pairs, void *ws, size_t ws_bytes,
+                     hipStream_t s);
+int run_expand_fill(const int64_t *rmask, int64_t R, int slots, int64_t *r_idx, int64_t *slot_idx, const void *ws,
+                    hipStream_t s);
+size_t arrival_pairs_workspace(int64_t P, int rpn);
+int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_in, const void *rgate, int64_t R,
+                      int64_t P, int64_t row_bytes, int gate_bytes, int gate_width, int epr, int rpn, void *send_buf,
+                      void *gate_pairs, int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *ordo,
+                      int32_t *status, void *ws, size_t ws_bytes, hipStream_t s);
+size_t segment_table_workspace(int64_t n_seg);
+int run_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table, int32_t *status,
+                      void *ws, size_t ws_bytes, hipStream_t s);
+int run_map_count(const void *map, int64_t T, int E, int32_t *row_stats, hipStream_t s);
+int run_map_topk(const void *map, const void *probs, int elem_bytes, int64_t T, int E, int k, int64_t *expert_idx,
+                 void *gates, hipStream_t s);
 }  // namespace terrace
 
 using namespace terrace;
@@ -189,6 +215,71 @@ int terrace_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows,
         return TERRACE_EINVAL;
     if (n_rows && row_bytes && !packed) return TERRACE_EINVAL;
     return launch_unpack_planes(packed, row_bytes, n_rows, a, a_bytes, b, b_bytes, c, c_bytes, (hipStream_t)stream);
+}
+
+size_t terrace_plan_general_workspace(int64_t T, int n_nodes) { return plan_general_workspace(T, n_nodes); }
+
+int terrace_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn,
+                         int64_t *u_src, int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status,
+                         void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_plan_general(expert_idx, T, k, world, n_experts, rpn, u_src, u_node, counts, inverse, status,
+                            workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_build_mask(const int64_t *expert_idx, const int64_t *inverse, int64_t n, int slots, int64_t n_rows,
+                       int64_t *mask, int32_t *status, terrace_stream_t stream) {
+    return run_build_mask(expert_idx, inverse, n, slots, n_rows, mask, status, (hipStream_t)stream);
+}
+
+int terrace_scatter_elems(const void *vals, int elem_bytes, const int64_t *rows, const int64_t *cols, int col_mod,
+                          int64_t n, int64_t n_rows, int width, void *out, terrace_stream_t stream) {
+    return run_scatter_elems(vals, elem_bytes, rows, cols, col_mod, n, n_rows, width, out, (hipStream_t)stream);
+}
+
+int terrace_expand_mask_quota(const int64_t *rmask, int64_t R, int slots, int quota, int64_t *r_idx,
+                              int64_t *slot_idx, terrace_stream_t stream) {
+    return run_expand_quota(rmask, R, slots, quota, r_idx, slot_idx, (hipStream_t)stream);
+}
+
+size_t terrace_expand_mask_workspace(int64_t R) { return expand_workspace(R); }
+
+int terrace_expand_mask_count(const int64_t *rmask, int64_t R, int slots, int64_t *n_pairs, void *workspace,
+                              size_t workspace_bytes, terrace_stream_t stream) {
+    return run_expand_count(rmask, R, slots, n_pairs, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_expand_mask_fill(const int64_t *rmask, int64_t R, int slots, int64_t *r_idx, int64_t *slot_idx,
+                             const void *workspace, terrace_stream_t stream) {
+    return run_expand_fill(rmask, R, slots, r_idx, slot_idx, workspace, (hipStream_t)stream);
+}
+
+size_t terrace_arrival_pairs_workspace(int64_t P, int rpn) { return arrival_pairs_workspace(P, rpn); }
+
+int terrace_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_in, const void *rgate, int64_t R,
+                          int64_t P, int64_t row_bytes, int gate_bytes, int gate_width, int epr, int rpn,
+                          void *send_buf, void *gate_pairs, int64_t *r_idx, int64_t *slot_idx, int64_t *i_send,
+                          int64_t *ordo, int32_t *status, void *workspace, size_t workspace_bytes,
+                          terrace_stream_t stream) {
+    return run_arrival_pairs(rx, r_in, slot_in, rgate, R, P, row_bytes, gate_bytes, gate_width, epr, rpn, send_buf,
+                             gate_pairs, r_idx, slot_idx, i_send, ordo, status, workspace, workspace_bytes,
+                             (hipStream_t)stream);
+}
+
+size_t terrace_segment_table_workspace(int64_t n_seg) { return segment_table_workspace(n_seg); }
+
+int terrace_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table, int32_t *status,
+                          void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_segment_table(seg, n, n_seg, width, table, status, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_routing_map_count(const void *routing_map, int64_t T, int n_experts, int32_t *row_stats,
+                              terrace_stream_t stream) {
+    return run_map_count(routing_map, T, n_experts, row_stats, (hipStream_t)stream);
+}
+
+int terrace_routing_map_topk(const void *routing_map, const void *probs, int elem_bytes, int64_t T, int n_experts,
+                             int k, int64_t *expert_idx, void *gates, terrace_stream_t stream) {
+    return run_map_topk(routing_map, probs, elem_bytes, T, n_experts, k, expert_idx, gates, (hipStream_t)stream);
 }
 
 int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send,

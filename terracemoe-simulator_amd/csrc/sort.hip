@@ -364,6 +364,32 @@ struct EmitArrival {         // terrace/ops/__init__.py:287-299
     }
 };
 
+struct EmitPairs {           // terrace/ta2a_fwd.py:605-628, general branch: pairs come as (row, slot) lists
+    const int64_t *r_in, *slot_in;
+    const void *rgate;       // sparse plane [R, gate_width]
+    int gate_bytes, gate_width;
+    int64_t R;
+    void *gate_pairs;
+    int64_t *r_idx, *slot_idx, *ordo;
+    int32_t *src32;          // source row of each output place (-1: row id out of range)
+    static constexpr bool kTallies = false;
+    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, const int32_t *, int *) const {
+        const int64_t r = r_in[p], sl = slot_in[p];
+        const bool ok = r >= 0 && r < R;
+        r_idx[dest] = r;
+        slot_idx[dest] = sl;
+        if (ordo) ordo[dest] = p;
+        src32[dest] = ok ? (int32_t)r : -1;
+        if (rgate) {
+            const bool gok = ok && sl >= 0 && sl < gate_width;
+            const int64_t cell = r * gate_width + sl;
+            if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = gok ? ((const uint32_t *)rgate)[cell] : 0u;
+            else ((uint16_t *)gate_pairs)[dest] = gok ? ((const uint16_t *)rgate)[cell] : (uint16_t)0;
+        }
+        return ok ? 0 : TERRACE_FAULT_ID_RANGE;
+    }
+};
+
 struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
     int64_t capacity;        // < 0: drop-less
     int64_t *order, *dest_out;
@@ -656,6 +682,34 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
+}
+
+// ---- Hop-B arrival, general branch (pairs listed explicitly) -------------------------------------
+size_t arrival_pairs_workspace(int64_t P, int rpn) {
+    if (P <= 0 || rpn <= 0 || rpn > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(P, rpn)) + align_up((size_t)P * sizeof(int32_t), 256);
+}
+
+int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_in, const void *rgate, int64_t R,
+                      int64_t P, int64_t row_bytes, int gate_bytes, int gate_width, int epr, int rpn, void *send_buf,
+                      void *gate_pairs, int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *ordo,
+                      int32_t *status, void *ws, size_t ws_bytes, hipStream_t s) {
+    if (R < 0 || P < 0 || epr <= 0 || rpn <= 0 || rpn > kMaxBuckets || !i_send || row_bytes < 0 ||
+        (gate_bytes != 2 && gate_bytes != 4) || gate_width < 0 || P >= (int64_t)1 << 31 || R >= (int64_t)1 << 31)
+        return TERRACE_EINVAL;
+    if (P == 0) return empty_outputs(i_send, nullptr, nullptr, rpn, status, s);
+    if (!r_in || !slot_in || !r_idx || !slot_idx || !ws || (rx && !send_buf) || (rgate && !gate_pairs))
+        return TERRACE_EINVAL;
+    const Units u = make_units(P, rpn);
+    const size_t table_bytes = units_table_bytes(u);
+    if (ws_bytes < table_bytes + align_up((size_t)P * sizeof(int32_t), 256)) return TERRACE_ENOSPC;
+    int32_t *table = (int32_t *)ws;
+    int32_t *src32 = (int32_t *)((char *)ws + table_bytes);
+    KeyAffine key{slot_in, 0, epr, rpn};
+    EmitPairs emit{r_in, slot_in, rgate, gate_bytes, gate_width, R, gate_pairs, r_idx, slot_idx, ordo, src32};
+    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
+    if (rc != TERRACE_OK || !rx) return rc;
+    return launch_gather_rows<int32_t>(rx, send_buf, src32, P, row_bytes, s);
 }
 
 // ---- expert-order regroup ---------------------------------------------------------------------

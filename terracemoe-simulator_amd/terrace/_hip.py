@@ -53,6 +53,20 @@ SIGNATURES = {
     "terrace_combine": (_I, [_P, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
     "terrace_pack_planes": (_I, [_P, _L, _P, _L, _P, _L, _L, _L, _P, _P]),
     "terrace_unpack_planes": (_I, [_P, _L, _L, _P, _L, _P, _L, _P, _L, _P]),
+    "terrace_plan_general_workspace": (_Z, [_L, _I]),
+    "terrace_plan_general": (_I, [_P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_build_mask": (_I, [_P, _P, _L, _I, _L, _P, _P, _P]),
+    "terrace_scatter_elems": (_I, [_P, _I, _P, _P, _I, _L, _L, _I, _P, _P]),
+    "terrace_expand_mask_quota": (_I, [_P, _L, _I, _I, _P, _P, _P]),
+    "terrace_expand_mask_workspace": (_Z, [_L]),
+    "terrace_expand_mask_count": (_I, [_P, _L, _I, _P, _P, _Z, _P]),
+    "terrace_expand_mask_fill": (_I, [_P, _L, _I, _P, _P, _P, _P]),
+    "terrace_arrival_pairs_workspace": (_Z, [_L, _I]),
+    "terrace_arrival_pairs": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_segment_table_workspace": (_Z, [_L]),
+    "terrace_segment_table": (_I, [_P, _L, _L, _I, _P, _P, _P, _Z, _P]),
+    "terrace_routing_map_count": (_I, [_P, _L, _I, _P, _P]),
+    "terrace_routing_map_topk": (_I, [_P, _P, _I, _L, _I, _I, _P, _P, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
 }
 

@@ -399,6 +399,182 @@ def argsort_small(key, n_buckets):
     return order, st
 
 
+def plan_general(expert_idx, world, n_experts, rpn):
+    """plan_ta2a with a data-dependent fan-out: (u_src [S], u_node [S], counts, inverse [T*k]);
+    S = counts.sum() is read back (the one synchronisation the reference pays too)."""
+    _require()
+    _hip.need_device(expert_idx)
+    expert_idx = expert_idx.contiguous()
+    dev = expert_idx.device
+    T, k = expert_idx.shape
+    n_nodes = world // rpn
+    if n_nodes > 64:
+        raise ValueError(f"plan_ta2a: the general plan handles at most 64 destination nodes, got {n_nodes}")
+    cap = T * min(k, n_nodes)
+    u_src = torch.empty((cap,), dtype=torch.int64, device=dev)
+    u_node = torch.empty((cap,), dtype=torch.int64, device=dev)
+    inverse = torch.empty((T * k,), dtype=torch.int64, device=dev)
+    counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_plan_general_workspace", T, n_nodes), dev)
+    _hip.call("terrace_plan_general", _hip.ptr(expert_idx), T, k, world, n_experts, rpn, _hip.ptr(u_src),
+              _hip.ptr(u_node), _hip.ptr(counts), _hip.ptr(inverse), _hip.ptr(st), _hip.ptr(ws), ws.numel(),
+              _hip.stream(dev))
+    both = torch.cat([counts.sum().reshape(1), st[:1].to(torch.int64)]).tolist()
+    if both[1] & _hip.FAULT_ID_RANGE:
+        raise ValueError("plan_ta2a: expert id out of range")
+    n_rows = int(both[0])
+    return u_src[:n_rows], u_node[:n_rows], counts, inverse
+
+
+def build_mask(expert_idx, inverse, n_rows, slots):
+    """Per-send-row int64 bitmask: bit j of row r set iff node-local slot j wants the row."""
+    _require()
+    _hip.need_device(expert_idx, inverse)
+    e, inv = expert_idx.contiguous().reshape(-1), inverse.contiguous().reshape(-1)
+    if e.dtype != torch.int64 or inv.dtype != torch.int64 or e.numel() != inv.numel():
+        raise RuntimeError("build_mask: expert_idx and inverse must be int64 planes of equal size")
+    dev = e.device
+    mask = torch.zeros((n_rows,), dtype=torch.int64, device=dev)
+    st = torch.zeros(_hip.STATUS_WORDS, dtype=torch.int32, device=dev)
+    _hip.call("terrace_build_mask", _hip.ptr(e), _hip.ptr(inv), e.numel(), slots, n_rows, _hip.ptr(mask),
+              _hip.ptr(st), _hip.stream(dev))
+    return mask, st
+
+
+def scatter_elems(vals, rows, cols, out, col_mod=0):
+    """``out[rows[i], c] = vals[i]`` in place on a dense 2-D ``out`` with ``c = cols[i]``, or
+    ``cols[i] % col_mod`` when ``col_mod > 0``; returns ``out``."""
+    _require()
+    _hip.need_device(vals, rows, cols, out)
+    vals, rows, cols = vals.contiguous().reshape(-1), rows.contiguous().reshape(-1), cols.contiguous().reshape(-1)
+    if vals.dtype != out.dtype or not out.is_contiguous() or out.dim() != 2:
+        raise RuntimeError("scatter_elems: out must be a dense 2-D plane of the values' dtype")
+    if rows.dtype != torch.int64 or cols.dtype != torch.int64 or not (vals.numel() == rows.numel() == cols.numel()):
+        raise RuntimeError("scatter_elems: rows/cols must be int64 planes as long as vals")
+    _hip.call("terrace_scatter_elems", _hip.ptr(vals), vals.element_size(), _hip.ptr(rows), _hip.ptr(cols),
+              int(col_mod), vals.numel(), out.shape[0], out.shape[1], _hip.ptr(out), _hip.stream(out.device))
+    return out
+
+
+def expand_mask(rmask, slots, quota=None):
+    """(r_idx, slot_idx) demand pairs of arrived bitmasks; without a quota the pair count is
+    read back from the device (the data-dependent shape ``nonzero`` has in the reference)."""
+    _require()
+    _hip.need_device(rmask)
+    rmask = rmask.contiguous().reshape(-1)
+    if rmask.dtype != torch.int64:
+        raise RuntimeError("expand_mask: rmask must be int64")
+    dev = rmask.device
+    R = rmask.numel()
+    if quota is not None:
+        r_idx = torch.empty((R * quota,), dtype=torch.int64, device=dev)
+        slot_idx = torch.empty((R * quota,), dtype=torch.int64, device=dev)
+        _hip.call("terrace_expand_mask_quota", _hip.ptr(rmask), R, slots, quota, _hip.ptr(r_idx), _hip.ptr(slot_idx),
+                  _hip.stream(dev))
+        return r_idx, slot_idx
+    n_pairs = torch.empty((1,), dtype=torch.int64, device=dev)
+    ws = _hip.workspace(_hip.query("terrace_expand_mask_workspace", R), dev)
+    _hip.call("terrace_expand_mask_count", _hip.ptr(rmask), R, slots, _hip.ptr(n_pairs), _hip.ptr(ws), ws.numel(),
+              _hip.stream(dev))
+    P = int(n_pairs.item())
+    r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    if P == 0:
+        return r_idx, slot_idx
+    _hip.call("terrace_expand_mask_fill", _hip.ptr(rmask), R, slots, _hip.ptr(r_idx), _hip.ptr(slot_idx),
+              _hip.ptr(ws), _hip.stream(dev))
+    return r_idx, slot_idx
+
+
+def arrival_pairs(rx, r_in, slot_in, rgate, epr, rpn):
+    """Arrival chain over an explicit pair list (the general branch):
+    (send_buf, gate_pairs, r_idx, slot_idx, i_send, ordo) with pairs in stable owner-card order
+    and ``gate_pairs = rgate[r_idx, slot_idx]`` looked up in the sparse [R, width] plane."""
+    _require()
+    _hip.need_device(rx, r_in, slot_in, rgate)
+    rx, r_in, slot_in = rx.contiguous(), r_in.contiguous().reshape(-1), slot_in.contiguous().reshape(-1)
+    if r_in.dtype != torch.int64 or slot_in.dtype != torch.int64 or r_in.numel() != slot_in.numel():
+        raise RuntimeError("arrival_pairs: r_idx/slot_idx must be int64 planes of equal length")
+    if rx.dim() != 2:
+        raise RuntimeError("arrival_pairs: rx must be 2-D")
+    dev = rx.device
+    R, H = rx.shape
+    P = r_in.numel()
+    gate_bytes, width, gate_pairs = 4, 0, None
+    if rgate is not None:
+        rgate = rgate.contiguous()
+        if rgate.dim() != 2 or rgate.shape[0] != R or rgate.element_size() not in (2, 4):
+            raise RuntimeError("arrival_pairs: rgate must be a [R, width] plane of 2- or 4-byte elements")
+        gate_bytes, width = rgate.element_size(), rgate.shape[1]
+        gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
+    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev)
+    r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    ordo = torch.empty((P,), dtype=torch.int64, device=dev)
+    i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_arrival_pairs_workspace", P, rpn), dev)
+    _hip.call("terrace_arrival_pairs", _hip.ptr(rx), _hip.ptr(r_in), _hip.ptr(slot_in), _hip.ptr(rgate), R, P,
+              H * rx.element_size(), gate_bytes, width, epr, rpn, _hip.ptr(send_buf), _hip.ptr(gate_pairs),
+              _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(ordo), _hip.ptr(st), _hip.ptr(ws),
+              ws.numel(), _hip.stream(dev))
+    return send_buf, gate_pairs, r_idx, slot_idx, i_send, ordo
+
+
+def segment_table(seg, n_seg, width):
+    """[n_seg, width] int64 table listing, per target s, the positions i with ``seg[i] == s`` in
+    ascending order, padded with -1: ``combine(src, table)`` is then ``index_add`` by ``seg``."""
+    _require()
+    _hip.need_device(seg)
+    seg = seg.contiguous().reshape(-1)
+    if seg.dtype != torch.int64:
+        raise RuntimeError("segment_table: seg must be int64")
+    dev = seg.device
+    table = torch.empty((n_seg, width), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_segment_table_workspace", n_seg), dev)
+    _hip.call("terrace_segment_table", _hip.ptr(seg), seg.numel(), n_seg, width, _hip.ptr(table), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return table, st
+
+
+def routing_map_topk(routing_map, probs):
+    """Dense [T,E] routing map -> ([T,k] ascending expert ids, [T,k] their probs).  One
+    synchronisation (the per-row count's min and max), as in the reference; raises
+    RuntimeError when rows do not all hold the same non-zero count."""
+    _require()
+    _hip.need_device(routing_map, probs)
+    if routing_map.dim() != 2 or probs.shape != routing_map.shape:
+        raise RuntimeError("routing_map_to_topk: routing_map and probs must both be [T, E]")
+    rm = routing_map.contiguous()
+    if rm.dtype == torch.bool:
+        rm = rm.view(torch.uint8)
+    elif rm.element_size() != 1:
+        rm = (rm != 0).view(torch.uint8)
+    probs = probs.contiguous()
+    if probs.element_size() not in (2, 4):
+        raise RuntimeError(f"routing_map_to_topk: unsupported probs dtype {probs.dtype}")
+    dev = rm.device
+    T, E = rm.shape
+    stats = torch.empty((2,), dtype=torch.int32, device=dev)
+    _hip.call("terrace_routing_map_count", _hip.ptr(rm), T, E, _hip.ptr(stats), _hip.stream(dev))
+    mn, mx = stats.tolist()
+    if T == 0:
+        mn = mx = 0
+    if mn != mx:
+        raise RuntimeError("T-A2A requires exactly k experts per token (drop-less); observed per-row expert "
+                           "counts differ")
+    k = int(mn)
+    if k == 0:
+        raise RuntimeError("T-A2A got an all-empty routing_map (k=0); impossible under drop-less routing")
+    expert_idx = torch.empty((T, k), dtype=torch.int64, device=dev)
+    gates = torch.empty((T, k), dtype=probs.dtype, device=dev)
+    _hip.call("terrace_routing_map_topk", _hip.ptr(rm), _hip.ptr(probs), probs.element_size(), T, E, k,
+              _hip.ptr(expert_idx), _hip.ptr(gates), _hip.stream(dev))
+    return expert_idx, gates
+
+
 def hopa_send_splits(node_counts, world, rpn, my_local):
     """Hop-A counts-exchange send buffer (terrace/ta2a_dispatch.py:197-211 of the reference)."""
     _require()
@@ -575,4 +751,5 @@ __all__ = [
     "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
     "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
+    "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table",
 ]

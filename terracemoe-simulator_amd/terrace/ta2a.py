@@ -57,22 +57,27 @@ def plan_ta2a(expert_idx: torch.Tensor, world: int, n_experts: int, rpn: int = 8
       inverse [T*k] for each (token, expert) slot, the send row that carries it
     Rows are ordered (node ascending, token ascending).
 
-    ``groups_m`` must be given (equal-quota routing, every token on exactly M nodes with k/M
-    experts on each); the data-dependent fan-out of the reference's ``groups_m=None`` branch
-    is not part of this build.
+    Without ``groups_m`` the fan-out is data dependent: S is read back from the device (one
+    sync, as in the reference) and nothing is verified.  With it, S = T*groups_m is known up
+    front and the equal-quota guard applies.
     """
     _hip.need_device(expert_idx)
     if expert_idx.dim() != 2:
         raise ValueError("plan_ta2a: expert_idx must be [T, k]")
     T, k = expert_idx.shape
     n_nodes = world // rpn
+    if n_nodes * T >= (1 << 24):
+        raise ValueError(
+            f"plan_ta2a float32 key range exceeded: n_nodes*T = {n_nodes * T} >= 2^24; "
+            f"shard tokens below {(1 << 24) // max(n_nodes, 1)} per rank or extend the "
+            f"plan to int64 keys first")
+    if world % rpn or n_experts % world:
+        raise ValueError(f"plan_ta2a: world={world} rpn={rpn} n_experts={n_experts} not divisible")
     if groups_m is None:
-        raise NotImplementedError("plan_ta2a: this build implements the equal-quota plan (pass groups_m)")
+        return _ops.plan_general(expert_idx.to(torch.int64), world, n_experts, rpn)
     if k % groups_m:
         raise ValueError(f"groups_m={groups_m} does not divide k={k}: the structured path's per-node quota "
                          f"k/M is not an integer. Leave groups_m None.")
-    if world % rpn or n_experts % world:
-        raise ValueError(f"plan_ta2a: world={world} rpn={rpn} n_experts={n_experts} not divisible")
     u_src, u_node, counts, inverse, _mask, status = _ops.plan_raw(
         expert_idx.to(torch.int64), world, n_experts, rpn, groups_m)
     _guard(status, T, k, n_nodes, groups_m)

@@ -60,6 +60,47 @@ def _expand_arrival_quota(rslot: torch.Tensor):
     return r_idx, rslot.reshape(-1)
 
 
+def _expand_arrival(rmask: torch.Tensor, slots: int, quota):
+    """Arrival-side (row, slot) demand pairs from shipped bitmasks, before the owner reorder.
+
+    ``quota`` None: every set bit, row-major with columns ascending (a data-dependent count,
+    read back from the device).  Otherwise exactly ``quota`` columns per row: its set columns
+    ascending, then -- only for a row holding fewer -- its unset columns ascending, which is
+    the order the reference's distinct-key top-k gives."""
+    return _ops.expand_mask(rmask, slots, quota)
+
+
+def build_expansion(expert_idx, inverse, n_rows: int, world: int, n_experts: int, rpn: int = 8,
+                    groups_m: int | None = None, *, sorted_rows: bool = False, slot_flat=None):
+    """Per-send-row int64 bitmask of the destination node's expert slots that want the token:
+    bit j of row r is set iff node-local slot j is one of the token's experts.  Requires
+    ``epr*rpn <= 63``.  ``groups_m`` / ``sorted_rows`` / ``slot_flat`` only select cheaper
+    formulations in the reference and never change a bit; one kernel serves all of them."""
+    slots = (n_experts // world) * rpn
+    if slots > 63:
+        raise ValueError(f"{slots} expert slots per node exceeds the int64 mask")
+    mask, _ = _ops.build_mask(expert_idx, inverse, n_rows, slots)
+    return mask
+
+
+def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8):
+    """Send side of the general (non-quota) branch: (payload, mask, gate_rows, u_src,
+    node_counts, inverse) with ``mask`` the [n_rows] int64 bitmask plane and ``gate_rows`` the
+    sparse [n_rows, slots] plane in the payload dtype."""
+    from .ta2a import plan_ta2a
+    slots = (n_experts // world) * rpn
+    if gates.dtype != x.dtype:
+        raise RuntimeError(f"Index put requires the source and destination dtypes match, got {x.dtype} "
+                           f"for the destination and {gates.dtype} for the source.")
+    u_src, _u_node, node_counts, inverse = plan_ta2a(expert_idx, world, n_experts, rpn, groups_m=None)
+    n_rows = u_src.numel()
+    payload = _ops.gather_rows(x, u_src)
+    mask = build_expansion(expert_idx, inverse, n_rows, world, n_experts, rpn)
+    gate_rows = torch.zeros((n_rows, slots), dtype=x.dtype, device=x.device)
+    _ops.scatter_elems(gates, inverse, expert_idx, gate_rows, col_mod=slots)
+    return payload, mask, gate_rows, u_src, node_counts, inverse
+
+
 @dataclass
 class LoopbackState:
     """What the combine needs from the dispatch, and what a caller may want to inspect."""
@@ -102,8 +143,9 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
                          slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
 
 
-def _regroup_with_place(node_rx, my_slot, epr):
-    """Drop-less regroup that also returns each input row's place (the inverse of ``order``)."""
+def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
+    """Drop-less regroup that also returns each input row's place (the inverse of ``order``):
+    (permuted, order, tokens_per_expert, place[, permuted_gate])."""
     _ops._require()
     node_rx, my_slot = node_rx.contiguous(), my_slot.contiguous().reshape(-1)
     dev = my_slot.device
@@ -112,12 +154,19 @@ def _regroup_with_place(node_rx, my_slot, epr):
     order = torch.empty((P,), dtype=torch.int64, device=dev)
     place = torch.empty((P,), dtype=torch.int64, device=dev)
     tpe = torch.empty((epr,), dtype=torch.int64, device=dev)
+    pgate, gate_bytes = None, 4
+    if my_gate is not None:
+        my_gate = my_gate.contiguous().reshape(-1)
+        gate_bytes = my_gate.element_size()
+        pgate = torch.empty((P,), dtype=my_gate.dtype, device=dev)
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, -1), dev)
-    _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), None, P, H * node_rx.element_size(), 4, epr,
-              0, -1, _hip.ptr(permuted), None, _hip.ptr(order), _hip.ptr(place), None, _hip.ptr(tpe), None,
-              _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
-    return permuted, order, tpe, place
+    _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), _hip.ptr(my_gate), P,
+              H * node_rx.element_size(), gate_bytes, epr, my_local, -1, _hip.ptr(permuted), _hip.ptr(pgate),
+              _hip.ptr(order), _hip.ptr(place), None, _hip.ptr(tpe), None, _hip.ptr(st), _hip.ptr(ws), ws.numel(),
+              _hip.stream(dev))
+    out = (permuted, order, tpe, place)
+    return out + (pgate,) if my_gate is not None else out
 
 
 def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, weights=None):

@@ -1,0 +1,276 @@
+"""HIP path vs the CPU oracle for the general (data-dependent fan-out) branch and the two seam
+halves -- through the C ABI only.  Index planes and moved rows bit-exact; the two-level combine
+bit-exact against the oracle's fp32 definition and within tolerance of float64."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import equal_quota_routing
+from oracle import terrace_oracle as orc
+from test_gpu_parity import DEV, DT, announce, same, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _ops_loaded():
+    import terrace.ops as tops
+    tops.reset()
+    assert tops.status().loaded, tops.status().reason
+    yield
+
+
+def _free_routing(T, k, E, seed):
+    rng = np.random.default_rng(seed)
+    return np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int64)
+
+
+GEOMS = [(4, 2, 8, 9, 3), (32, 8, 64, 40, 4), (16, 8, 32, 17, 5), (64, 8, 128, 333, 6), (8, 4, 8, 1, 2),
+         (64, 8, 256, 3000, 8), (512, 8, 512, 700, 12)]
+
+
+@pytest.mark.parametrize("world,rpn,E,T,k", GEOMS)
+@pytest.mark.parametrize("fmt", ["f32", "bf16"])
+def test_general_send_side_planes(world, rpn, E, T, k, fmt):
+    from terrace import ta2a
+    from terrace.ta2a_fwd import build_expansion, general_hopa_planes
+    announce("general send", (world, rpn, E, T, k), fmt)
+    e = _free_routing(T, k, E, 21)
+    slots = (E // world) * rpn
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, 24, generator=g).to(DT[fmt])
+    gates = torch.rand(T, k, generator=g).to(DT[fmt])
+    ed = torch.from_numpy(e).to(DEV)
+    got = ta2a.plan_ta2a(ed, world, E, rpn)
+    want = orc.plan_ta2a(e, world, E, rpn)
+    for name, a, b in zip(("u_src", "u_node", "counts", "inverse"), got, want):
+        same(a, b, name)
+    payload, mask, gate_rows, u_src, counts, inverse = general_hopa_planes(x.to(DEV), ed, gates.to(DEV), world, E, rpn)
+    same(payload, to_np(x)[want[0]], "payload")
+    same(mask, orc.build_expansion(e, want[3], want[0].size, world, E, rpn), "mask")
+    same(gate_rows, orc.sparse_gate_plane(e, to_np(gates), want[3], want[0].size, slots), "gate_rows")
+    same(u_src, want[0], "u_src"), same(counts, want[2], "counts"), same(inverse, want[3], "inverse")
+    # the reference's cheaper formulations give the same bits
+    m2 = build_expansion(ed, got[3], got[0].numel(), world, E, rpn, groups_m=None, sorted_rows=True,
+                         slot_flat=ed.reshape(-1) % slots)
+    assert torch.equal(m2, mask)
+    stats = ta2a.dispatch_stats(ed, world, E, rpn)
+    assert stats == orc.dispatch_stats(e, world, E, rpn)
+
+
+def test_general_plan_errors_and_empty():
+    from terrace import ta2a
+    from terrace.ta2a_fwd import build_expansion
+    announce("general plan errors")
+    bad = torch.tensor([[0, 2, 99]] * 5, device=DEV)
+    with pytest.raises(ValueError, match="out of range"):
+        ta2a.plan_ta2a(bad, 4, 8, 2)
+    with pytest.raises(ValueError, match="2\\^24"):
+        ta2a.plan_ta2a(torch.zeros((1 << 21, 1), dtype=torch.int64, device=DEV), 64, 64, 8)
+    with pytest.raises(ValueError, match="exceeds the int64 mask"):
+        build_expansion(torch.zeros((2, 2), dtype=torch.int64, device=DEV), torch.zeros(4, dtype=torch.int64, device=DEV),
+                        2, 2, 128, 2)
+    u_src, u_node, counts, inverse = ta2a.plan_ta2a(torch.zeros((0, 4), dtype=torch.int64, device=DEV), 4, 8, 2)
+    assert u_src.numel() == 0 and inverse.numel() == 0 and counts.tolist() == [0, 0]
+
+
+@pytest.mark.parametrize("slots", [1, 5, 16, 24, 25, 40, 63])
+def test_expand_arrival_both_forms(slots):
+    from terrace.ta2a_fwd import _expand_arrival
+    announce("expand", slots)
+    rng = np.random.default_rng(slots)
+    for R in (0, 1, 70, 5000):
+        rmask = rng.integers(0, 1 << slots, size=R, dtype=np.int64)
+        if R > 3:
+            rmask[3] = 0
+        md = torch.from_numpy(rmask).to(DEV)
+        r, c = _expand_arrival(md, slots, None)
+        wr, wc = orc.expand_arrival(rmask, slots, None)
+        same(r, wr, "r_idx"), same(c, wc, "slot_idx")
+        for quota in {1, min(2, slots), min(4, slots), slots}:
+            r, c = _expand_arrival(md, slots, quota)
+            wr, wc = orc.expand_arrival(rmask, slots, quota)
+            same(r, wr, f"r_idx q={quota}"), same(c, wc, f"slot_idx q={quota}")
+
+
+@pytest.mark.parametrize("R,slots,epr,rpn,H,fmt", [(30, 12, 3, 4, 5, "f32"), (700, 32, 4, 8, 64, "bf16"),
+                                                    (1, 8, 1, 8, 16, "f16"), (4096, 16, 2, 8, 512, "bf16")])
+def test_arrival_pairs_general(R, slots, epr, rpn, H, fmt):
+    import terrace.ops as tops
+    announce("arrival_pairs", R, slots, epr, rpn, H, fmt)
+    rng = np.random.default_rng(R + slots)
+    rmask = rng.integers(0, 1 << slots, size=R, dtype=np.int64)
+    r, c = orc.expand_arrival(rmask, slots, None)
+    g = torch.Generator().manual_seed(R)
+    rx = torch.randn(R, H, generator=g).to(DT[fmt])
+    rgate = torch.randn(R, slots, generator=g).to(DT[fmt])
+    got = tops.arrival_pairs(rx.to(DEV), torch.from_numpy(r).to(DEV), torch.from_numpy(c).to(DEV), rgate.to(DEV),
+                             epr, rpn)
+    want = orc.arrival_pairs(to_np(rx), r, c, to_np(rgate), epr, rpn)
+    for name, a, b in zip(("send_buf", "gate_pairs", "r_idx", "slot_idx", "i_send", "ordo"), got, want):
+        same(a, b, name)
+    # no pairs at all
+    z = torch.zeros(0, dtype=torch.int64, device=DEV)
+    out = tops.arrival_pairs(rx.to(DEV), z, z, rgate.to(DEV), epr, rpn)
+    assert out[0].shape == (0, H) and out[4].tolist() == [0] * rpn
+
+
+def test_segment_table_lists_items_in_ascending_order():
+    import terrace.ops as tops
+    announce("segment_table")
+    rng = np.random.default_rng(8)
+    for n, n_seg, width in [(0, 5, 3), (40, 7, 40), (5000, 300, 64), (9, 9, 1)]:
+        seg = np.sort(rng.integers(0, n_seg, size=n)) if width == 1 and n else rng.integers(0, n_seg, size=n)
+        if width == 1:
+            seg = rng.permutation(n_seg)[:n]
+        table, st = tops.segment_table(torch.from_numpy(seg.astype(np.int64)).to(DEV), n_seg, width)
+        want = np.full((n_seg, width), -1, dtype=np.int64)
+        for s in range(n_seg):
+            items = np.flatnonzero(seg == s)
+            want[s, :items.size] = items
+        same(table, want, f"table {n},{n_seg},{width}")
+        assert st.tolist()[0] == 0
+    # overflow and range faults are reported, never written out of bounds
+    from terrace import _hip
+    seg = torch.tensor([0, 0, 0, 5, -1], device=DEV)
+    table, st = tops.segment_table(seg, 2, 2)
+    assert st.tolist()[0] == (_hip.FAULT_ID_RANGE | _hip.FAULT_FANOUT)
+    assert table.tolist()[1] == [-1, -1] and sorted(table.tolist()[0])[0] >= 0
+
+
+def test_routing_map_to_topk_and_refusals():
+    from terrace.ta2a_dispatch import routing_map_to_topk
+    announce("routing_map_to_topk")
+    rng = np.random.default_rng(2)
+    for T, E, k, dt in [(19, 24, 5, torch.float32), (1000, 256, 8, torch.bfloat16), (64, 64, 64, torch.float16),
+                        (3, 300, 2, torch.float32)]:
+        e = np.sort(np.stack([rng.permutation(E)[:k] for _ in range(T)]), 1)
+        rm = np.zeros((T, E), dtype=bool)
+        rm[np.arange(T)[:, None], e] = True
+        probs = torch.from_numpy(rng.random((T, E)).astype(np.float32)).to(dt)
+        ge, gg = routing_map_to_topk(torch.from_numpy(rm).to(DEV), probs.to(DEV))
+        we, wg = orc.routing_map_to_topk(rm, to_np(probs))
+        same(ge, we, "expert_idx"), same(gg, wg, "gates")
+    bad = rm.copy()
+    bad[1, e[1, 0]] = False
+    with pytest.raises(RuntimeError, match="exactly k experts"):
+        routing_map_to_topk(torch.from_numpy(bad).to(DEV), probs.to(DEV))
+    with pytest.raises(RuntimeError, match="all-empty"):
+        routing_map_to_topk(torch.zeros(4, 8, dtype=torch.bool, device=DEV), torch.zeros(4, 8, device=DEV))
+
+
+def _seam_oracle(x_rows, e, gate_bits, world, E, rpn, M, fmt):
+    """Dispatch half by the oracle, loop-back: every slot of the node is a local expert."""
+    epr, slots = E // world, (E // world) * rpn
+    T, k = e.shape
+    if M:
+        payload, mask, gate_rows, u_src, counts = orc.k2_pack(x_rows, e, gate_bits, world, E, rpn, M)
+        send, gp, r_idx, slot_idx, i_send = orc.k1_arrival(payload, mask, gate_rows, k // M, epr, rpn)
+    else:
+        u_src, _, counts, inverse = orc.plan_ta2a(e, world, E, rpn)
+        payload = x_rows[u_src]
+        mask = orc.build_expansion(e, inverse, u_src.size, world, E, rpn)
+        plane = orc.sparse_gate_plane(e, gate_bits, inverse, u_src.size, slots)
+        r_in, s_in = orc.expand_arrival(mask, slots, None)
+        send, gp, r_idx, slot_idx, i_send, _ = orc.arrival_pairs(payload, r_in, s_in, plane, epr, rpn)
+    permuted, order, tpe = orc.regroup(send, slot_idx, slots)
+    return dict(permuted=permuted, tpe=tpe, pprobs=gp[order], u_src=u_src, r_idx=r_idx, order=order,
+                R=payload.shape[0])
+
+
+def _unpermute_oracle(out_rows, o, T, fmt, out_fmt):
+    """Two index_add levels as terrace/ta2a_dispatch.py:483-494 writes them, each level in fp32
+    with one rounding: a row sums its pairs in arrival order, a token its rows ascending."""
+    P = o["order"].size
+    place = np.empty(P, dtype=np.int64)
+    place[o["order"]] = np.arange(P)
+    R = o["R"]
+    fan1 = max(int(np.bincount(o["r_idx"], minlength=R).max()), 1) if P else 1
+    t1 = np.full((R, fan1), -1, dtype=np.int64)
+    fill = np.zeros(R, dtype=np.int64)
+    for j in range(P):
+        r = o["r_idx"][j]
+        t1[r, fill[r]] = place[j]
+        fill[r] += 1
+    red = orc.combine(out_rows, t1, None, fmt, fmt)
+    fan2 = max(int(np.bincount(o["u_src"], minlength=T).max()), 1)
+    t2 = np.full((T, fan2), -1, dtype=np.int64)
+    fill = np.zeros(T, dtype=np.int64)
+    for r in range(R):
+        t = o["u_src"][r]
+        t2[t, fill[t]] = r
+        fill[t] += 1
+    return orc.combine(red, t2, None, fmt, out_fmt), t1, t2
+
+
+SEAM = [(4, 2, 8, 8, 4, 2, 6), (32, 8, 64, 48, 4, 2, 32), (32, 8, 96, 32, 8, 4, 16), (16, 4, 16, 12, 4, 1, 24),
+        (64, 8, 256, 1500, 8, 4, 128), (64, 8, 128, 33, 6, 3, 8)]
+
+
+@pytest.mark.parametrize("world,rpn,E,T,k,M,H", SEAM)
+@pytest.mark.parametrize("fmt", ["f32", "bf16"])
+@pytest.mark.parametrize("branch", ["quota", "general"])
+@pytest.mark.parametrize("mode", ["small", "full", "off"])
+def test_seam_halves_loopback(world, rpn, E, T, k, M, H, fmt, branch, mode, monkeypatch):
+    from terrace import ta2a, ta2a_pack
+    from terrace.ta2a_dispatch import ta2a_permute, ta2a_unpermute
+    if (E // world) * rpn > 63 and branch == "general":
+        pytest.skip("bitmask branch needs <= 63 slots per node")
+    if mode != "small" and T > 100:
+        pytest.skip("container modes are covered on the small geometries")
+    announce("seam", (world, rpn, E, T, k, M, H), fmt, branch, mode)
+    monkeypatch.setenv("TERRACE_TA2A_PACK", mode)
+    ta2a_pack.reset()
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    e = equal_quota_routing(T, k, E, world // rpn, M, 31, sort_rows=True)
+    g = torch.Generator().manual_seed(T + H)
+    x = torch.randn(T, H, generator=g).to(DT[fmt])
+    probs = torch.rand(T, E, generator=g).to(DT[fmt])
+    rm = torch.zeros(T, E, dtype=torch.bool)
+    rm[torch.arange(T)[:, None], torch.from_numpy(e)] = True
+    try:
+        permuted, tpe, pprobs, st = ta2a_permute(x.to(DEV), probs.to(DEV), rm.to(DEV), world=world, rank=1, rpn=rpn,
+                                                 n_experts=E, groups_m=M if branch == "quota" else None)
+    finally:
+        ta2a_pack.reset()
+    gate_bits = np.take_along_axis(to_np(probs), e, 1)
+    o = _seam_oracle(to_np(x), e, gate_bits, world, E, rpn, M if branch == "quota" else None, fmt)
+    same(permuted, o["permuted"], "permuted"), same(tpe, o["tpe"], "tokens_per_expert")
+    same(pprobs, o["pprobs"], "permuted_probs")
+    same(st.u_src, o["u_src"], "u_src"), same(st.r_idx, o["r_idx"], "r_idx"), same(st.order, o["order"], "order")
+    assert (st.R, st.T, st.hidden, st.dtype) == (o["R"], T, H, DT[fmt])
+    # tokens_per_expert is forced by the routing alone: node-local slot histogram
+    assert np.array_equal(o["tpe"], np.bincount(e.reshape(-1) % ((E // world) * rpn), minlength=(E // world) * rpn))
+    # the vendor's expert layer: a per-row scale by the gate, then the combine half
+    slots = (E // world) * rpn
+    slot_sorted = torch.repeat_interleave(torch.arange(slots, device=DEV), tpe)
+    expert_out = (permuted.float() * ((slot_sorted + 1).float() / slots)[:, None] * pprobs.float()[:, None]).to(DT[fmt])
+    y = ta2a_unpermute(expert_out, st, x.to(DEV))
+    want, t1, t2 = _unpermute_oracle(to_np(expert_out), o, T, fmt, fmt)
+    same(y, want, "y")
+    e64 = orc.decode_rows(to_np(expert_out), fmt).astype(np.float64)
+    red64 = np.where((t1 >= 0)[:, :, None], e64[np.maximum(t1, 0)], 0.0).sum(1)
+    y64 = np.where((t2 >= 0)[:, :, None], red64[np.maximum(t2, 0)], 0.0).sum(1)
+    tol = 1e-5 if fmt == "f32" else 1e-2
+    assert np.abs(orc.decode_rows(to_np(y), fmt) - y64).max() <= tol * (np.abs(y64).max() + 1e-30)
+    # ... which is the one-level definition y[t] = sum_j gate[t,j] * f(x[t], e[t,j])
+    x64 = orc.decode_rows(to_np(x), fmt).astype(np.float64)
+    direct = np.zeros((T, H))
+    for j in range(k):
+        direct += x64 * ((e[:, j] % slots + 1) / slots)[:, None] * orc.decode_rows(gate_bits, fmt).astype(np.float64)[:, j:j + 1]
+    assert np.abs(y64 - direct).max() <= (2e-6 if fmt == "f32" else 2e-2) * (np.abs(direct).max() + 1e-30)
+
+
+def test_seam_refuses_process_groups_and_mismatched_probs():
+    from terrace.ta2a_dispatch import ta2a_permute
+    announce("seam refusals")
+    x = torch.randn(4, 8, device=DEV)
+    rm = torch.zeros(4, 8, dtype=torch.bool, device=DEV)
+    rm[:, [0, 2, 4, 6]] = True
+    with pytest.raises(NotImplementedError, match="loop-back"):
+        ta2a_permute(x, torch.rand(4, 8, device=DEV), rm, world=4, rank=0, rpn=2, n_experts=8, intra_group=object(),
+                     groups_m=2)
+    with pytest.raises(RuntimeError, match="dtypes match"):
+        ta2a_permute(x.bfloat16(), torch.rand(4, 8, device=DEV), rm, world=4, rank=0, rpn=2, n_experts=8, groups_m=2)
