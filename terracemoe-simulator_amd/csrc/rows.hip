@@ -115,37 +115,90 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict
     }
 }
 
-// Sliced form for 16-byte vectors: a workgroup of BT lanes owns BT consecutive vectors of one output
-// row (blockIdx.x = row * slices + slice) and every lane moves exactly one vector.  Many tiny
-// workgroups keep loads and stores of different rows interleaved in the memory pipeline, which
-// streams measurably faster than fewer workgroups that each load a whole row and then store it.
-template <int BT, typename I>
-__global__ __launch_bounds__(BT) void gather_rows_sliced_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ out,
-                                                                const I *__restrict__ idx, int64_t row_vecs,
-                                                                uint32_t slices) {
+// Sliced forms for 16-byte vectors: a workgroup is one wave, every lane moves exactly one vector, and
+// each wave's store covers one 1 KB-aligned kilobyte of the destination.  Many one-wave workgroups
+// keep loads and stores of different rows interleaved in the memory pipeline, which streams
+// measurably faster than fewer workgroups that load a whole row and then store it; and because
+// consecutive workgroups run on different XCDs (each with an L2 of its own), a store that ends inside
+// a 128-byte line would leave that line half-written in two L2s -- so chunks are cut on destination
+// kilobyte boundaries, not at multiples of 64 vectors from the row start.
+
+// Gather: the destination is one flat run of n_out*row_vecs vectors; `head` is the number of vectors
+// between the kilobyte boundary at or below `out` and `out` itself.
+template <typename I>
+__global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ out,
+                                                                 const I *__restrict__ idx, int64_t total_vecs,
+                                                                 int64_t row_vecs, int head) {
+    const int64_t first = (int64_t)blockIdx.x * kWave - head;            // wave-uniform, may be < 0 in block 0
+    const int64_t g = first + threadIdx.x;
+    if (g < 0 || g >= total_vecs) return;
+    int64_t row, i;
+    if (row_vecs >= kWave) {
+        const int64_t f0 = first < 0 ? 0 : first;
+        row = f0 / row_vecs;                                             // one division per wave
+        i = g - row * row_vecs;
+        if (i >= row_vecs) {                                             // at most one row boundary inside a wave
+            i -= row_vecs;
+            ++row;
+        }
+    } else {
+        row = g / row_vecs;
+        i = g - row * row_vecs;
+    }
+    const int64_t from = (int64_t)idx[row];
+    u32x4 v = zero_of<u32x4>();
+    if (from >= 0) v = ld_stream(src + from * row_vecs + i);
+    st_stream(out + g, v);
+}
+
+// Gather, rows that are whole kilobytes on a kilobyte-aligned destination: blockIdx.x = row * slices + slice.
+template <typename I>
+__global__ __launch_bounds__(kWave) void gather_rows_sliced_kernel(const u32x4 *__restrict__ src,
+                                                                   u32x4 *__restrict__ out, const I *__restrict__ idx,
+                                                                   int64_t row_vecs, uint32_t slices) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
-    const int64_t i = (int64_t)slice * BT + threadIdx.x;
-    if (i >= row_vecs) return;
+    const int64_t i = (int64_t)slice * kWave + threadIdx.x;
     const int64_t from = (int64_t)idx[row];
     u32x4 v = zero_of<u32x4>();
     if (from >= 0) v = ld_stream(src + from * row_vecs + i);
     st_stream(out + (int64_t)row * row_vecs + i, v);
 }
 
-template <int BT, typename I>
-__global__ __launch_bounds__(BT) void scatter_rows_sliced_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst,
-                                                                 const I *__restrict__ pos, int fan, int64_t row_vecs,
-                                                                 uint32_t slices) {
+// Scatter, rows that are whole kilobytes on a kilobyte-aligned destination: load once, store fan times.
+template <typename I>
+__global__ __launch_bounds__(kWave) void scatter_rows_sliced_kernel(const u32x4 *__restrict__ src,
+                                                                    u32x4 *__restrict__ dst, const I *__restrict__ pos,
+                                                                    int fan, int64_t row_vecs, uint32_t slices) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
-    const int64_t i = (int64_t)slice * BT + threadIdx.x;
-    if (i >= row_vecs) return;
+    const int64_t i = (int64_t)slice * kWave + threadIdx.x;
     const u32x4 v = ld_stream(src + (int64_t)row * row_vecs + i);
     const I *p = pos + (int64_t)row * fan;
     for (int f = 0; f < fan; ++f) {
         const int64_t d = p[f];
         if (d >= 0) st_stream(dst + d * row_vecs + i, v);
+    }
+}
+
+// Scatter, any other 16-byte-multiple row width: every copy is cut on its own destination's kilobyte
+// boundaries, so the window of source vectors a wave needs shifts from copy to copy and is loaded
+// again for each (the re-loads hit in cache: HBM still sees each source row once).
+template <typename I>
+__global__ __launch_bounds__(kWave) void scatter_rows_aligned_kernel(const u32x4 *__restrict__ src,
+                                                                     u32x4 *__restrict__ dst, const I *__restrict__ pos,
+                                                                     int fan, int64_t row_vecs, uint32_t chunks,
+                                                                     int head) {
+    const uint32_t row = blockIdx.x / chunks;
+    const int64_t c = blockIdx.x - row * chunks;
+    const u32x4 *s = src + (int64_t)row * row_vecs;
+    const I *p = pos + (int64_t)row * fan;
+    for (int f = 0; f < fan; ++f) {
+        const int64_t d = p[f];
+        if (d < 0) continue;
+        const int64_t base = d * row_vecs;
+        const int64_t i = c * kWave - ((base + head) & (kWave - 1)) + threadIdx.x;
+        if (i >= 0 && i < row_vecs) st_stream(dst + base + i, s[i]);
     }
 }
 
@@ -475,11 +528,18 @@ int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src,
     switch (vec_bytes_for(row_bytes, src, dst)) {
         case 16: {
             const int64_t rv = row_bytes / 16;
-            if (rv % 64 == 0 && n_src * (rv / 64) <= kMaxBlocks)
-                scatter_rows_sliced_kernel<64, I><<<(unsigned)(n_src * (rv / 64)), 64, 0, s>>>(
-                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)(rv / 64));
-            else
-                launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, rv, s);
+            const int head = (int)(((uintptr_t)dst >> 4) & (kWave - 1));
+            if (rv % kWave == 0 && head == 0 && n_src * (rv / kWave) <= kMaxBlocks) {
+                scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, 0, s>>>(
+                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)(rv / kWave));
+            } else {
+                const int64_t chunks = (rv + 2 * kWave - 2) / kWave;      // most kilobytes one copy can touch
+                if (n_src * chunks <= kMaxBlocks)
+                    scatter_rows_aligned_kernel<I><<<(unsigned)(n_src * chunks), kWave, 0, s>>>(
+                        (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)chunks, head);
+                else
+                    launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, rv, s);
+            }
             break;
         }
         case 8: launch_scatter_t<u32x2, I>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
@@ -506,18 +566,21 @@ static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_
         gather_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
 }
 
-// Rows that are whole kilobytes take the sliced form, one wave per workgroup.
 template <typename I>
 static bool launch_gather_sliced(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_vecs,
                                  hipStream_t s) {
-    if (row_vecs % 64 == 0) {
-        const int64_t slices = row_vecs / 64;
-        if (n_out * slices > kMaxBlocks) return false;
-        gather_rows_sliced_kernel<64, I><<<(unsigned)(n_out * slices), 64, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx,
-                                                                                  row_vecs, (uint32_t)slices);
+    const int head = (int)(((uintptr_t)out >> 4) & (kWave - 1));
+    const int64_t total = n_out * row_vecs;
+    const int64_t blocks = (total + head + kWave - 1) / kWave;
+    if (blocks > kMaxBlocks) return false;
+    if (row_vecs % kWave == 0 && head == 0) {
+        gather_rows_sliced_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, row_vecs,
+                                                                       (uint32_t)(row_vecs / kWave));
         return true;
     }
-    return false;
+    gather_rows_flat_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, total, row_vecs,
+                                                                 head);
+    return true;
 }
 
 template <typename I>
