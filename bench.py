@@ -10,8 +10,10 @@ part of the path; its output is a fixed synthetic tensor prepared before the tim
 The all-to-all exchanges are not executed (one GPU): the rank's Hop-A send buffer is looped
 back as its arrival buffer.
 
-Prints ONE JSON line: whole-step algorithmic GB/s as `value`, per-stage ms / GB/s / fraction
-of the 8 TB/s HBM peak and the arrival chain's us/row in `stages`, the roofline record of
+Prints ONE JSON line: whole-step algorithmic GB/s as `value` (each payload row counted once on the
+read side and once on the write side of every stage) and, beside it, the same step priced on the
+bytes that must cross HBM (`min_traffic`); per-stage ms / GB/s / fraction of the 8 TB/s HBM peak
+and the arrival chain's us/row in `stages`, the roofline record of
 the slowest row-moving kernel (timed alone with HIP events on the launch stream), and the CPU
 oracle timed on the host cores over a bounded sample of the same workload.
 """
@@ -32,7 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of a workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE and scaled by the same counters' reading for the copy kernel (fetch x2.00,
 # write x1.00).  Only workloads that have been measured are listed; others report null.
-MEASURED_TRAFFIC_BYTES = {("c2", "gather_rows_kernel(regroup)"): 3.769e9}
+MEASURED_TRAFFIC_BYTES = {("c2", "gather_rows_sliced_kernel(regroup)"): 3.767e9}
 REFERENCE_TARGET_US_PER_ROW = 0.012     # the reference's fused-chain design target
 
 
@@ -221,10 +223,13 @@ def main():
     stage_ms = {"route": event_ms(route, reps, torch), "pack": event_ms(pack, reps, torch),
                 "arrival": event_ms(arrival, reps, torch), "regroup": event_ms(regroup, reps, torch),
                 "combine": event_ms(combine, reps, torch)}
+    kept_pairs = int((state.place >= 0).sum()) if cap is not None else None
+    min_bytes = configs.minimum_traffic_bytes(cfg, kept_pairs, None if cap is None else cfg.slots * cap)
     stages = {}
     for name, ms in stage_ms.items():
         gbps = nbytes[name] / ms / 1e6
-        stages[name] = {"ms": round(ms, 4), "GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+        stages[name] = {"ms": round(ms, 4), "GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                        "min_traffic_GBps": round(min_bytes[name] / ms / 1e6, 1)}
     stages["arrival"]["us_per_row"] = round(stage_ms["arrival"] * 1e3 / cfg.pairs, 6)
     stages["arrival"]["reference_target_us_per_row"] = REFERENCE_TARGET_US_PER_ROW
     pc_bytes = nbytes["pack"] + nbytes["combine"]
@@ -243,13 +248,16 @@ def main():
         ok = state.place >= 0
         gather_idx[state.place[ok]] = torch.arange(cfg.pairs, device=dev)[ok]
     out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
+    # names of the kernels the library picks for this row width (whole kilobytes or not)
+    kb_rows = row % 1024 == 0
+    k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
+    k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
     kernels = {
-        "scatter_rows_kernel(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows),
-                                      2 * cfg.send_rows * row),
-        "scatter_rows_kernel(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
-                                         2 * cfg.pairs * row),
-        "gather_rows_kernel(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx),
-                                        2 * gather_idx.numel() * row),
+        f"{k_scatter}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), 2 * cfg.send_rows * row),
+        f"{k_scatter}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
+                                  2 * cfg.pairs * row),
+        f"{k_gather}(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx),
+                                 2 * gather_idx.numel() * row),
         "combine_kernel": (lambda: tops.combine(ye, where, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
                            cfg.pairs * row + cfg.pairs * 12 + cfg.T * out_row),
         "copy_kernel(passthrough)": (lambda: tops.passthrough(state.send_buf), 2 * state.send_buf.numel()
@@ -280,6 +288,10 @@ def main():
                    "exchange": "loop-back (no all-to-all on one GPU)",
                    "expert_outputs": "fixed synthetic tensor prepared before the timed region"},
         "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "min_traffic": {"GBps": round(sum(min_bytes.values()) / ms_per_step / 1e6, 1),
+                        "frac_hbm_peak": round(sum(min_bytes.values()) / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4),
+                        "note": "bytes that must cross HBM: a scatter reads each source row once however many "
+                                "copies it writes, a capacity layout reads only the rows it keeps"},
         "pack_plus_combine": {"GBps": round(pc_bytes / pc_ms / 1e6, 1),
                               "frac_hbm_peak": round(pc_bytes / pc_ms / 1e6 / HBM_PEAK_GBPS, 4)},
         "arrival_chain_us_per_row": stages["arrival"]["us_per_row"],

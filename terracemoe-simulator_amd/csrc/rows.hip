@@ -302,7 +302,7 @@ __global__ __launch_bounds__(BT) void combine_kernel(const uint8_t *__restrict__
                                                          int slices) {
     constexpr int N = Chunk<SRC>::N;
     const int64_t row = blockIdx.x / slices;
-    const int64_t c = (int64_t)(blockIdx.x - row * slices) * BT + threadIdx.x;
+    const int64_t c = (int64_t)(blockIdx.x - row * slices) * blockDim.x + threadIdx.x;
     if (c >= hidden / N) return;
     float acc[N];
 #pragma unroll
@@ -617,7 +617,9 @@ static void launch_combine_so(const void *src, const int64_t *idx, const void *w
                               int fan, int64_t hidden, void *out, hipStream_t s) {
     const int64_t chunks = hidden / Chunk<SRC>::N;
     const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
-    // one wave per workgroup when a row is a whole number of waves' worth of chunks
+    // one wave per workgroup when a row is a whole number of waves' worth of chunks (a workgroup
+    // spanning a whole misaligned row, which would keep split cache lines inside one L2, measured
+    // slower than this at the fp8 row shape)
     const bool one_wave = chunks % kWave == 0 && n_out * (chunks / kWave) <= kMaxBlocks;
     const int bt = one_wave ? kWave : kBlock;
     const int slices = (int)((chunks + bt - 1) / bt);

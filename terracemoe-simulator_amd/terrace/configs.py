@@ -146,3 +146,23 @@ def algorithmic_bytes(cfg: PathConfig, out_row_bytes: int | None = None) -> dict
         "regroup": 2 * P * row + P * 8 * 2,
         "combine": P * crow + P * 4 + P * 8 + T * orow,
     }
+
+
+def minimum_traffic_bytes(cfg: PathConfig, kept_pairs: int | None = None, places: int | None = None) -> dict:
+    """HBM bytes each stage cannot avoid: every distinct payload row read once and every output row
+    written once (a scatter reads a source row once however many copies it writes), plus the same
+    index and gate planes as ``algorithmic_bytes``.  ``kept_pairs`` / ``places`` describe a capacity
+    layout (rows that survive the cut, rows of the padded buffer); default: drop-less."""
+    T, k, q = cfg.T, cfg.top_k, cfg.quota
+    S, P, row = cfg.send_rows, cfg.pairs, cfg.row_bytes
+    kept = P if kept_pairs is None else kept_pairs
+    places = P if places is None else places
+    alg = algorithmic_bytes(cfg)
+    orow = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
+    return {
+        "route": alg["route"],
+        "pack": alg["pack"] - 2 * S * row + (T + S) * row,
+        "arrival": alg["arrival"] - 2 * P * row + (S + P) * row,
+        "regroup": alg["regroup"] - 2 * P * row + (kept + places) * row,
+        "combine": alg["combine"] - P * row + kept * row,
+    }
