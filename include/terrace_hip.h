@@ -272,6 +272,15 @@ TERRACE_API int terrace_segment_table(const int64_t *seg, int64_t n, int64_t n_s
                                       int32_t *status, void *workspace, size_t workspace_bytes,
                                       terrace_stream_t stream);
 
+/* The tables the adjoints of ta2a_permute / ta2a_unpermute read (terrace/ta2a_dispatch.py:263-498): for every
+ * place i < P of the expert-order buffer, behind it arrival row a = order[i], send row r = r_idx[a], token
+ * t = u_src[r] and expert e = u_node[r]*slots + slot_idx[a]:  token_of_place[i] = t (may be NULL) and
+ * where[t, j] = i for the column j with expert_idx[t, j] == e.  where [T,k] is first filled with -1. */
+TERRACE_API int terrace_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *slot_idx,
+                                    const int64_t *u_src, const int64_t *u_node, const int64_t *expert_idx, int64_t P,
+                                    int64_t T, int k, int slots, int64_t n_rows, int64_t *where,
+                                    int64_t *token_of_place, int32_t *status, terrace_stream_t stream);
+
 /* routing_map_to_topk (terrace/ta2a_dispatch.py:224-260): routing_map [T,E] bytes (non-zero = chosen).
  * _count writes row_stats = {min, max} of the per-token counts (int32[2]); after the caller has
  * checked min == max == k, _topk writes the k chosen expert ids ascending and their probs

@@ -582,6 +582,28 @@ def routing_map_to_topk(routing_map, probs):
     return expert_idx, np.take_along_axis(np.asarray(probs), expert_idx, 1)
 
 
+def pair_places(order, r_idx, slot_idx, u_src, u_node, expert_idx, slots):
+    """(where [T,k], token_of_place [P]) for the seam halves (terrace/ta2a_dispatch.py:263-498).
+
+    Place i of the expert-order buffer holds arrival row ``a = order[i]``, a copy of send row
+    ``r = r_idx[a]``, i.e. of token ``t = u_src[r]`` for expert ``u_node[r]*slots + slot_idx[a]``;
+    ``where[t, j] = i`` for the column j holding that expert.  So ``permuted[i] =
+    hidden[token_of_place[i]]`` and ``ta2a_unpermute`` computes ``y[t] = sum_j expert_out[where[t, j]]``;
+    the adjoints of both halves read these two tables.
+    """
+    e = np.asarray(expert_idx, dtype=np.int64)
+    T, k = e.shape
+    a = np.asarray(order, dtype=np.int64)
+    r = np.asarray(r_idx, dtype=np.int64)[a]
+    tok = np.asarray(u_src, dtype=np.int64)[r]
+    exp = np.asarray(u_node, dtype=np.int64)[r] * slots + np.asarray(slot_idx, dtype=np.int64)[a]
+    where = np.full((T, k), -1, dtype=np.int64)
+    hit = e[tok] == exp[:, None]                                  # [P, k]
+    rows, cols = np.nonzero(hit)
+    where[tok[rows], cols] = rows
+    return where, tok
+
+
 # --------------------------------------------------------------------------------------
 # wire containers -- terrace/ta2a_pack.py:276-506
 # --------------------------------------------------------------------------------------

@@ -68,6 +68,9 @@ int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_i
 size_t segment_table_workspace(int64_t n_seg);
 int run_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table, int32_t *status,
                       void *ws, size_t ws_bytes, hipStream_t s);
+int run_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *slot_idx, const int64_t *u_src,
+                    const int64_t *u_node, const int64_t *expert_idx, int64_t P, int64_t T, int k, int slots,
+                    int64_t n_rows, int64_t *where, int64_t *token_of_place, int32_t *status, hipStream_t s);
 int run_map_count(const void *map, int64_t T, int E, int32_t *row_stats, hipStream_t s);
 int run_map_topk(const void *map, const void *probs, int elem_bytes, int64_t T, int E, int k, int64_t *expert_idx,
                  void *gates, hipStream_t s);
@@ -270,6 +273,14 @@ size_t terrace_segment_table_workspace(int64_t n_seg) { return segment_table_wor
 int terrace_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table, int32_t *status,
                           void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
     return run_segment_table(seg, n, n_seg, width, table, status, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *slot_idx, const int64_t *u_src,
+                        const int64_t *u_node, const int64_t *expert_idx, int64_t P, int64_t T, int k, int slots,
+                        int64_t n_rows, int64_t *where, int64_t *token_of_place, int32_t *status,
+                        terrace_stream_t stream) {
+    return run_pair_places(order, r_idx, slot_idx, u_src, u_node, expert_idx, P, T, k, slots, n_rows, where,
+                           token_of_place, status, (hipStream_t)stream);
 }
 
 int terrace_routing_map_count(const void *routing_map, int64_t T, int n_experts, int32_t *row_stats,

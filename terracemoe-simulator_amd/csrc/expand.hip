@@ -305,6 +305,63 @@ int run_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, i
     return check_launch();
 }
 
+// ---- where each (token, expert) pair sits in the expert-order buffer --------------------------------
+// One lane per place i of the buffer: the arrival row behind it is a = order[i], its send row
+// r = r_idx[a], its token t = u_src[r] and its expert e = u_node[r]*slots + slot_idx[a]; the column j
+// with expert_idx[t, j] == e gets where[t, j] = i.  These are the tables the adjoints of the two seam
+// halves read (terrace/ta2a_dispatch.py:263-498): permuted[i] = hidden[token_of_place[i]] and
+// y[t] = sum_j expert_out[where[t, j]].
+__global__ __launch_bounds__(kBlock) void fill_i64_kernel(int64_t *__restrict__ p, int64_t n, int64_t v) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+__global__ __launch_bounds__(kBlock) void pair_places_kernel(
+    const int64_t *__restrict__ order, const int64_t *__restrict__ r_idx, const int64_t *__restrict__ slot_idx,
+    const int64_t *__restrict__ u_src, const int64_t *__restrict__ u_node, const int64_t *__restrict__ expert_idx,
+    int64_t P, int64_t T, int k, int slots, int64_t n_rows, int64_t *__restrict__ where,
+    int64_t *__restrict__ token_of_place, int32_t *__restrict__ status) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= P) return;
+    bool ok = false;
+    int64_t t = -1;
+    const int64_t a = order[i];
+    if (a >= 0 && a < P) {
+        const int64_t r = r_idx[a];
+        if (r >= 0 && r < n_rows) {
+            t = u_src[r];
+            if (t >= 0 && t < T) {
+                const int64_t e = u_node[r] * slots + slot_idx[a];
+                for (int j = 0; j < k; ++j) {
+                    if (expert_idx[t * k + j] == e) {
+                        where[t * k + j] = i;
+                        ok = true;
+                    }
+                }
+            }
+        }
+    }
+    if (token_of_place) token_of_place[i] = ok ? t : -1;
+    if (!ok && status) atomicOr(&status[0], TERRACE_FAULT_ID_RANGE);
+}
+
+int run_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *slot_idx, const int64_t *u_src,
+                    const int64_t *u_node, const int64_t *expert_idx, int64_t P, int64_t T, int k, int slots,
+                    int64_t n_rows, int64_t *where, int64_t *token_of_place, int32_t *status, hipStream_t s) {
+    if (P < 0 || T < 0 || k <= 0 || slots <= 0 || n_rows < 0) return TERRACE_EINVAL;
+    if (status) fill_i32_kernel<<<1, kBlock, 0, s>>>(status, TERRACE_STATUS_WORDS, 0);
+    if (T > 0) {
+        if (!where) return TERRACE_EINVAL;
+        fill_i64_kernel<<<(unsigned)((T * k + kBlock - 1) / kBlock), kBlock, 0, s>>>(where, T * k, -1);
+    }
+    if (P > 0) {
+        if (!order || !r_idx || !slot_idx || !u_src || !u_node || !expert_idx || !where) return TERRACE_EINVAL;
+        pair_places_kernel<<<(unsigned)((P + kBlock - 1) / kBlock), kBlock, 0, s>>>(
+            order, r_idx, slot_idx, u_src, u_node, expert_idx, P, T, k, slots, n_rows, where, token_of_place, status);
+    }
+    return check_launch();
+}
+
 // ---- routing_map -> top-k ---------------------------------------------------------------------------
 // one wave per token; row_stats = {min count, max count} over tokens (int32, pre-set by the first kernel's block 0
 // is not possible without ordering, so the caller provides them initialised to {INT_MAX, 0}).

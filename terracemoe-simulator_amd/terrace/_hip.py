@@ -65,6 +65,7 @@ SIGNATURES = {
     "terrace_arrival_pairs": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_segment_table_workspace": (_Z, [_L]),
     "terrace_segment_table": (_I, [_P, _L, _L, _I, _P, _P, _P, _Z, _P]),
+    "terrace_pair_places": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _L, _P, _P, _P, _P]),
     "terrace_routing_map_count": (_I, [_P, _L, _I, _P, _P]),
     "terrace_routing_map_topk": (_I, [_P, _P, _I, _L, _I, _I, _P, _P, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),

@@ -539,6 +539,28 @@ def segment_table(seg, n_seg, width):
     return table, st
 
 
+def pair_places(order, r_idx, slot_idx, u_src, u_node, expert_idx, slots):
+    """(where [T,k], token_of_place [P]): the place of every (token, expert) pair in the expert-order
+    buffer and the token behind every place."""
+    _require()
+    _hip.need_device(order, r_idx, slot_idx, u_src, u_node, expert_idx)
+    planes = [t.contiguous().reshape(-1) for t in (order, r_idx, slot_idx, u_src, u_node)]
+    expert_idx = expert_idx.contiguous()
+    if any(t.dtype != torch.int64 for t in planes) or expert_idx.dtype != torch.int64:
+        raise RuntimeError("pair_places: every plane must be int64")
+    order, r_idx, slot_idx, u_src, u_node = planes
+    dev = expert_idx.device
+    T, k = expert_idx.shape
+    P = order.numel()
+    where = torch.empty((T, k), dtype=torch.int64, device=dev)
+    tok = torch.empty((P,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    _hip.call("terrace_pair_places", _hip.ptr(order), _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(u_src),
+              _hip.ptr(u_node), _hip.ptr(expert_idx), P, T, k, slots, u_src.numel(), _hip.ptr(where), _hip.ptr(tok),
+              _hip.ptr(st), _hip.stream(dev))
+    return where, tok
+
+
 def routing_map_topk(routing_map, probs):
     """Dense [T,E] routing map -> ([T,k] ascending expert ids, [T,k] their probs).  One
     synchronisation (the per-row count's min and max), as in the reference; raises
@@ -751,5 +773,5 @@ __all__ = [
     "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
     "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
-    "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table",
+    "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table", "pair_places",
 ]

@@ -5,6 +5,10 @@ Same surface as the reference module (terrace/ta2a_dispatch.py there): ``routing
 them.  The dispatch half returns (rows in local-expert order, rows per local expert, the
 per-row gates, state); the gate is NOT multiplied here (the expert layer does that), and the
 combine half adds each returned row once per (row, slot) pair and once per (token, node).
+Both halves are differentiable: the float outputs hang on autograd edges whose backward passes
+are the adjoint row movers (a fixed-fan gather-reduce for ``hidden_states``, an element gather
+for ``probs``, a fan-k row scatter for ``expert_out``), so the router learns through
+``permuted_probs`` as it does in the reference.
 
 The reference runs four all-to-all exchanges inside these halves.  One GPU has no peers, so
 the exchanges are loop-back: the rank's own Hop-A send buffer is its arrival buffer and every
@@ -32,7 +36,7 @@ class TA2AState:
 
     __slots__ = ("u_src", "r_idx", "order", "R", "T", "hidden",
                  "send_l", "recv_l", "is_l", "ir_l", "intra", "inter", "dtype",
-                 "red_table", "tok_table")
+                 "red_table", "tok_table", "where", "token_of_place")
 
 
 def routing_map_to_topk(routing_map: torch.Tensor, probs: torch.Tensor):
@@ -40,6 +44,57 @@ def routing_map_to_topk(routing_map: torch.Tensor, probs: torch.Tensor):
     their gates.  Requires exactly k set entries in every row and raises RuntimeError otherwise;
     one host synchronisation (the min and max of the per-row counts)."""
     return _ops.routing_map_topk(routing_map, probs)
+
+
+class _PermutedEdge(torch.autograd.Function):
+    """permuted[i] = hidden[token_of_place[i]]; adjoint: a token sums the k places it was copied to."""
+
+    @staticmethod
+    def forward(ctx, hidden_states, where, permuted):
+        ctx.save_for_backward(where)
+        ctx.dtype = hidden_states.dtype
+        return permuted
+
+    @staticmethod
+    def backward(ctx, g):
+        (where,) = ctx.saved_tensors
+        return _ops.combine(g.contiguous(), where, None, out_dtype=ctx.dtype), None, None
+
+
+class _ProbsEdge(torch.autograd.Function):
+    """permuted_probs[where[t, j]] = probs[t, expert_idx[t, j]]; adjoint: the same two look-ups backwards."""
+
+    @staticmethod
+    def forward(ctx, probs, where, expert_idx, pprobs):
+        ctx.save_for_backward(where, expert_idx)
+        ctx.shape, ctx.dtype = probs.shape, probs.dtype
+        return pprobs
+
+    @staticmethod
+    def backward(ctx, g):
+        where, expert_idx = ctx.saved_tensors
+        T, k = expert_idx.shape
+        d_gates = _ops.gather_rows(g.contiguous().to(ctx.dtype).reshape(-1, 1), where.reshape(-1))
+        d_probs = torch.zeros(ctx.shape, dtype=ctx.dtype, device=g.device)
+        rows = torch.arange(T, device=g.device, dtype=torch.int64).unsqueeze(1).expand(T, k)
+        _ops.scatter_elems(d_gates, rows, expert_idx, d_probs)
+        return d_probs, None, None, None
+
+
+class _UnpermuteFn(torch.autograd.Function):
+    """y[t] = sum_j expert_out[where[t, j]] (two levels); adjoint: place where[t, j] receives dy[t]."""
+
+    @staticmethod
+    def forward(ctx, expert_out, red_table, tok_table, where, out_dtype):
+        ctx.save_for_backward(where)
+        ctx.n_places, ctx.dtype = expert_out.shape[0], expert_out.dtype
+        red = _ops.combine(expert_out, red_table, None, out_dtype=expert_out.dtype)
+        return _ops.combine(red, tok_table, None, out_dtype=out_dtype)
+
+    @staticmethod
+    def backward(ctx, gy):
+        (where,) = ctx.saved_tensors
+        return _ops.scatter_rows(gy.contiguous().to(ctx.dtype), where, ctx.n_places), None, None, None, None
 
 
 def _loopback_only(*groups):
@@ -75,8 +130,9 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         (payload, mask, gate_rows, u_src, node_counts), ex = _ops.k2_pack_raw(
             hidden_states, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
         _plan._guard(ex["status"], T, k, n_nodes, groups_m)
+        u_node = ex["u_node"]
     else:
-        payload, mask, gate_rows, u_src, node_counts, _inverse = general_hopa_planes(
+        payload, mask, gate_rows, u_src, node_counts, _inverse, u_node = general_hopa_planes(
             hidden_states, expert_idx, gates, world, n_experts, rpn)
 
     # Hop A (loop-back): what was packed for the wire is what arrives
@@ -123,6 +179,12 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
         st.red_table = _ops.index_chain(place, per_row)
         st.tok_table, _ = _ops.segment_table(u_src, T, min(k, n_nodes))
+    st.where, st.token_of_place = _ops.pair_places(order, r_idx, my_slot, u_src, u_node, expert_idx, slots)
+    if torch.is_grad_enabled():
+        if hidden_states.requires_grad:
+            permuted = _PermutedEdge.apply(hidden_states, st.where, permuted)
+        if probs.requires_grad:
+            pprobs = _ProbsEdge.apply(probs, st.where, expert_idx, pprobs)
     return permuted, tokens_per_expert, pprobs, st
 
 
@@ -134,5 +196,7 @@ def ta2a_unpermute(expert_out, st: TA2AState, out_like):
     its rows in ascending row order; each level accumulates in fp32 and rounds once to the
     tensor dtype."""
     _hip.need_device(expert_out)
+    if torch.is_grad_enabled() and expert_out.requires_grad:
+        return _UnpermuteFn.apply(expert_out, st.red_table, st.tok_table, st.where, out_like.dtype)
     red = _ops.combine(expert_out, st.red_table, None, out_dtype=expert_out.dtype)
     return _ops.combine(red, st.tok_table, None, out_dtype=out_like.dtype)

@@ -85,20 +85,20 @@ def build_expansion(expert_idx, inverse, n_rows: int, world: int, n_experts: int
 
 def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8):
     """Send side of the general (non-quota) branch: (payload, mask, gate_rows, u_src,
-    node_counts, inverse) with ``mask`` the [n_rows] int64 bitmask plane and ``gate_rows`` the
-    sparse [n_rows, slots] plane in the payload dtype."""
+    node_counts, inverse, u_node) with ``mask`` the [n_rows] int64 bitmask plane and ``gate_rows``
+    the sparse [n_rows, slots] plane in the payload dtype."""
     from .ta2a import plan_ta2a
     slots = (n_experts // world) * rpn
     if gates.dtype != x.dtype:
         raise RuntimeError(f"Index put requires the source and destination dtypes match, got {x.dtype} "
                            f"for the destination and {gates.dtype} for the source.")
-    u_src, _u_node, node_counts, inverse = plan_ta2a(expert_idx, world, n_experts, rpn, groups_m=None)
+    u_src, u_node, node_counts, inverse = plan_ta2a(expert_idx, world, n_experts, rpn, groups_m=None)
     n_rows = u_src.numel()
     payload = _ops.gather_rows(x, u_src)
     mask = build_expansion(expert_idx, inverse, n_rows, world, n_experts, rpn)
     gate_rows = torch.zeros((n_rows, slots), dtype=x.dtype, device=x.device)
     _ops.scatter_elems(gates, inverse, expert_idx, gate_rows, col_mod=slots)
-    return payload, mask, gate_rows, u_src, node_counts, inverse
+    return payload, mask, gate_rows, u_src, node_counts, inverse, u_node
 
 
 @dataclass

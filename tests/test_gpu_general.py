@@ -47,7 +47,7 @@ def test_general_send_side_planes(world, rpn, E, T, k, fmt):
     want = orc.plan_ta2a(e, world, E, rpn)
     for name, a, b in zip(("u_src", "u_node", "counts", "inverse"), got, want):
         same(a, b, name)
-    payload, mask, gate_rows, u_src, counts, inverse = general_hopa_planes(x.to(DEV), ed, gates.to(DEV), world, E, rpn)
+    payload, mask, gate_rows, u_src, counts, inverse, _u_node = general_hopa_planes(x.to(DEV), ed, gates.to(DEV), world, E, rpn)
     same(payload, to_np(x)[want[0]], "payload")
     same(mask, orc.build_expansion(e, want[3], want[0].size, world, E, rpn), "mask")
     same(gate_rows, orc.sparse_gate_plane(e, to_np(gates), want[3], want[0].size, slots), "gate_rows")
@@ -261,6 +261,67 @@ def test_seam_halves_loopback(world, rpn, E, T, k, M, H, fmt, branch, mode, monk
     for j in range(k):
         direct += x64 * ((e[:, j] % slots + 1) / slots)[:, None] * orc.decode_rows(gate_bits, fmt).astype(np.float64)[:, j:j + 1]
     assert np.abs(y64 - direct).max() <= (2e-6 if fmt == "f32" else 2e-2) * (np.abs(direct).max() + 1e-30)
+
+
+@pytest.mark.parametrize("world,rpn,E,T,k,M,H", [(4, 2, 8, 8, 4, 2, 6), (32, 8, 64, 48, 4, 2, 32),
+                                                   (64, 8, 256, 700, 8, 4, 64), (16, 4, 16, 12, 4, 1, 24)])
+@pytest.mark.parametrize("branch", ["quota", "general"])
+def test_seam_backward_is_the_adjoint(world, rpn, E, T, k, M, H, branch):
+    """Gradients of both halves against torch autograd (float64, CPU) over the same map written
+    with index ops: permuted = x[token_of_place], probs gathered at (token, expert) of each place,
+    y = index_add by token.  The tables themselves are checked bit-exact against the oracle."""
+    from terrace import ta2a
+    from terrace.ta2a_dispatch import ta2a_permute, ta2a_unpermute
+    if (E // world) * rpn > 63 and branch == "general":
+        pytest.skip("bitmask branch needs <= 63 slots per node")
+    announce("seam backward", (world, rpn, E, T, k, M, H), branch)
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    slots = (E // world) * rpn
+    e = equal_quota_routing(T, k, E, world // rpn, M, 77, sort_rows=True)
+    g = torch.Generator().manual_seed(T * H)
+    x = torch.randn(T, H, generator=g)
+    probs = torch.rand(T, E, generator=g)
+    G = torch.randn(T, H, generator=g)
+    rm = torch.zeros(T, E, dtype=torch.bool)
+    rm[torch.arange(T)[:, None], torch.from_numpy(e)] = True
+    xd, pd = x.to(DEV).requires_grad_(), probs.to(DEV).requires_grad_()
+    permuted, tpe, pprobs, st = ta2a_permute(xd, pd, rm.to(DEV), world=world, rank=0, rpn=rpn, n_experts=E,
+                                             groups_m=M if branch == "quota" else None)
+    o = _seam_oracle(x.numpy(), e, np.take_along_axis(probs.numpy(), e, 1), world, E, rpn,
+                     M if branch == "quota" else None, "f32")
+    _, u_node, _, _ = orc.plan_ta2a(e, world, E, rpn)
+    slot_sorted_np = np.repeat(np.arange(slots), o["tpe"])
+    # slot id of each arrival row, recovered from the expert-order histogram
+    slot_of_arrival = np.empty(o["order"].size, dtype=np.int64)
+    slot_of_arrival[o["order"]] = slot_sorted_np
+    where, tok = orc.pair_places(o["order"], o["r_idx"], slot_of_arrival, o["u_src"], u_node, e, slots)
+    same(st.where, where, "where"), same(st.token_of_place, tok, "token_of_place")
+    scale = ((torch.repeat_interleave(torch.arange(slots, device=DEV), tpe) + 1).float() / slots)[:, None]
+    expert_out = permuted * scale * pprobs[:, None]
+    assert expert_out.requires_grad
+    y = ta2a_unpermute(expert_out, st, xd)
+    (y * G.to(DEV)).sum().backward()
+    # reference: the same map with index ops, float64 autograd on the CPU
+    x64, p64 = x.double().requires_grad_(), probs.double().requires_grad_()
+    tok_t = torch.from_numpy(tok)
+    exp_of_place = torch.from_numpy(e)[tok_t][torch.from_numpy(where)[tok_t] == torch.arange(tok.size)[:, None]]
+    perm64 = x64[tok_t]
+    pp64 = p64[tok_t, exp_of_place]
+    eo64 = perm64 * scale.cpu().double() * pp64[:, None]
+    y64 = torch.zeros(T, H, dtype=torch.float64).index_add(0, tok_t, eo64)
+    (y64 * G.double()).sum().backward()
+    assert np.abs(y.detach().cpu().double().numpy() - y64.detach().numpy()).max() <= 1e-5 * float(y64.detach().abs().max())
+    for name, got, want in (("x.grad", xd.grad, x64.grad), ("probs.grad", pd.grad, p64.grad)):
+        assert got is not None, f"{name} is missing: the edge is not attached"
+        err = (got.cpu().double() - want).abs().max().item()
+        assert err <= 1e-5 * max(want.abs().max().item(), 1.0), f"{name} differs by {err}"
+    # probs.grad is zero exactly where the routing map is
+    assert torch.equal(pd.grad.cpu() != 0, rm) or (pd.grad.cpu()[~rm] == 0).all()
+    # without grad mode nothing is attached
+    with torch.no_grad():
+        p2, _, g2, st2 = ta2a_permute(xd, pd, rm.to(DEV), world=world, rank=0, rpn=rpn, n_experts=E,
+                                      groups_m=M if branch == "quota" else None)
+    assert not p2.requires_grad and not g2.requires_grad and torch.equal(p2, permuted.detach())
 
 
 def test_seam_refuses_process_groups_and_mismatched_probs():

@@ -153,3 +153,28 @@ def test_routing_map_to_topk_is_nonzero_plus_gather_and_fails_loud():
         orc.routing_map_to_topk(bad, probs)
     with pytest.raises(RuntimeError, match="all-empty"):
         orc.routing_map_to_topk(np.zeros((4, 8), bool), np.zeros((4, 8), np.float32))
+
+
+def test_pair_places_by_definition(literals):
+    """where[t, j] is the one place of the expert-order buffer holding token t's copy for expert
+    expert_idx[t, j]: checked by walking the chain backwards from every place."""
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"]:
+        slots, q, epr = (E // world) * rpn, k // M, E // world
+        e = equal_quota_routing(T, k, E, world // rpn, M, 9)
+        rng = np.random.default_rng(3)
+        hidden = rng.standard_normal((T, 4)).astype(np.float32)
+        gates = rng.standard_normal((T, k)).astype(np.float32)
+        payload, slot_tab, gate_tab, u_src, counts = orc.k2_pack(hidden, e, gates, world, E, rpn, M)
+        _, u_node, _, _ = orc.plan_ta2a(e, world, E, rpn)
+        send, gp, r_idx, slot_idx, _ = orc.k1_arrival(payload, slot_tab, gate_tab, q, epr, rpn)
+        permuted, order, tpe = orc.regroup(send, slot_idx, slots)
+        where, tok = orc.pair_places(order, r_idx, slot_idx, u_src, u_node, e, slots)
+        assert np.array_equal(np.sort(where.reshape(-1)), np.arange(T * k))          # a bijection onto the places
+        assert np.array_equal(permuted, hidden[tok])                                 # the place holds that token's row
+        for t in range(T):
+            for j in range(k):
+                i = where[t, j]
+                assert tok[i] == t
+                assert gp[order][i] == gates[t, j]                                   # and that expert's gate
+                # local expert of the place = node-local slot of expert (t, j)
+                assert np.searchsorted(np.cumsum(tpe), i, side="right") == e[t, j] % slots
