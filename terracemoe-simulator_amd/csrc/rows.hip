@@ -292,10 +292,95 @@ __device__ __forceinline__ void store_chunk(void *out_row, int64_t first_elem, c
     }
 }
 
-// Vector path: rows are 16-byte aligned multiples of 16 bytes.  One thread owns one 16-byte
-// chunk of one output row: blockIdx.x = row * slices + slice, chunk = slice*256 + threadIdx.x.
-template <int SRC, int OUT, int FANC, int BT>
-__global__ __launch_bounds__(BT) void combine_kernel(const uint8_t *__restrict__ src, int64_t src_row_bytes,
+// Vector path: rows are 16-byte aligned multiples of 16 bytes.  One thread owns one 16-byte chunk of
+// one output row: blockIdx.x = row * slices + slice, chunk = slice * blockDim.x + threadIdx.x.
+//
+// Everything a batch of source rows needs that is the same for the whole wave -- the row ids and
+// the weights -- is fetched first through addresses the compiler can prove uniform (scalar loads; 16-bit
+// weights are read as the aligned dword that holds them).  The batch's row loads are then issued back to
+// back with nothing between them that waits on memory, and only the accumulation that follows consumes
+// them in order.  Dead entries (idx < 0) load row 0 and are zeroed with selects: no branch splits the
+// batch.
+constexpr int kWNone = -1;
+
+template <int WD>
+__device__ __forceinline__ float uniform_weight(const void *w, int64_t i) {
+    if constexpr (WD == TERRACE_F32) {
+        return ((const float *)w)[i];
+    } else {
+        const uint32_t pair = ((const uint32_t *)w)[i >> 1];
+        const uint32_t bits = (i & 1) ? (pair >> 16) : (pair & 0xFFFFu);
+        if constexpr (WD == TERRACE_BF16) return __uint_as_float(bits << 16);
+        else return __half2float(__ushort_as_half((unsigned short)bits));
+    }
+}
+
+// One batch of exactly B source rows, no guards: B uniform index (and weight) fetches, B row loads
+// issued back to back, then the in-order accumulation.
+template <int SRC, int WD, int B>
+__device__ __forceinline__ void combine_batch(float *acc, const uint8_t *__restrict__ src, int64_t src_row_bytes,
+                                              const int64_t *__restrict__ idx_at, const void *__restrict__ w,
+                                              int64_t w_at, int64_t hidden, int64_t c) {
+    constexpr int N = Chunk<SRC>::N;
+    int64_t from[B];
+    float wj[B];
+#pragma unroll
+    for (int jj = 0; jj < B; ++jj) {
+        from[jj] = idx_at[jj];
+        if constexpr (WD != kWNone) wj[jj] = uniform_weight<WD>(w, w_at + jj);
+        else wj[jj] = 1.0f;
+    }
+    u32x4 raw[B];
+    float sc[B];
+#pragma unroll
+    for (int jj = 0; jj < B; ++jj) {
+        const uint8_t *s = src + (from[jj] < 0 ? 0 : from[jj]) * src_row_bytes;
+        raw[jj] = ld_stream((const u32x4 *)s + c);
+        if constexpr (SRC == TERRACE_FP8_E4M3_B128) sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
+        else sc[jj] = 1.0f;
+    }
+#pragma unroll
+    for (int jj = 0; jj < B; ++jj) {
+        const bool live = from[jj] >= 0;
+        const u32x4 r = live ? raw[jj] : zero_of<u32x4>();
+        const float scale = live ? sc[jj] : 0.0f, weight = live ? wj[jj] : 0.0f;
+        float f[N];
+        decode_chunk<SRC>(r, f);
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            float x = f[i];
+            if constexpr (SRC == TERRACE_FP8_E4M3_B128) x = __fmul_rn(x, scale);
+            if constexpr (WD != kWNone) x = __fmul_rn(x, weight);
+            acc[i] = __fadd_rn(acc[i], x);
+        }
+    }
+}
+
+template <int SRC, int OUT, int WD>
+__device__ __forceinline__ void combine_row_chunk(const uint8_t *__restrict__ src, int64_t src_row_bytes,
+                                                  const int64_t *__restrict__ idx_row, const void *__restrict__ w,
+                                                  int64_t w_base, int fan, int64_t hidden, int64_t c,
+                                                  uint8_t *__restrict__ out_row) {
+    constexpr int N = Chunk<SRC>::N;
+    float acc[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+    int j = 0;
+    for (; j + 8 <= fan; j += 8) combine_batch<SRC, WD, 8>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+    if (j + 4 <= fan) {
+        combine_batch<SRC, WD, 4>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+        j += 4;
+    }
+    if (j + 2 <= fan) {
+        combine_batch<SRC, WD, 2>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+        j += 2;
+    }
+    if (j < fan) combine_batch<SRC, WD, 1>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+    store_chunk<OUT, N>(out_row, c * N, acc);
+}
+
+template <int SRC, int OUT>
+__global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restrict__ src, int64_t src_row_bytes,
                                                          const int64_t *__restrict__ idx, const void *__restrict__ w,
                                                          int w_dtype, int64_t n_out, int fan, int64_t hidden,
                                                          uint8_t *__restrict__ out, int64_t out_row_bytes,
@@ -304,46 +389,15 @@ __global__ __launch_bounds__(BT) void combine_kernel(const uint8_t *__restrict__
     const int64_t row = blockIdx.x / slices;
     const int64_t c = (int64_t)(blockIdx.x - row * slices) * blockDim.x + threadIdx.x;
     if (c >= hidden / N) return;
-    float acc[N];
-#pragma unroll
-    for (int i = 0; i < N; ++i) acc[i] = 0.0f;
-    for (int j0 = 0; j0 < fan; j0 += FANC) {
-        u32x4 raw[FANC];
-        float wj[FANC], sc[FANC];
-        bool live[FANC];
-#pragma unroll
-        for (int jj = 0; jj < FANC; ++jj) {
-            const int j = j0 + jj;
-            live[jj] = false;
-            wj[jj] = 1.0f;
-            sc[jj] = 1.0f;
-            if (j < fan) {
-                const int64_t from = idx[row * fan + j];
-                if (from >= 0) {
-                    live[jj] = true;
-                    const uint8_t *s = src + from * src_row_bytes;
-                    raw[jj] = ld_stream((const u32x4 *)s + c);
-                    if constexpr (SRC == TERRACE_FP8_E4M3_B128)
-                        sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
-                    if (w) wj[jj] = load_weight(w, w_dtype, row * fan + j);
-                }
-            }
-        }
-#pragma unroll
-        for (int jj = 0; jj < FANC; ++jj) {
-            if (!live[jj]) continue;
-            float f[N];
-            decode_chunk<SRC>(raw[jj], f);
-#pragma unroll
-            for (int i = 0; i < N; ++i) {
-                float x = f[i];
-                if constexpr (SRC == TERRACE_FP8_E4M3_B128) x = __fmul_rn(x, sc[jj]);
-                if (w) x = __fmul_rn(x, wj[jj]);
-                acc[i] = __fadd_rn(acc[i], x);
-            }
-        }
-    }
-    store_chunk<OUT, N>(out + row * out_row_bytes, c * N, acc);
+    const int64_t *idx_row = idx + row * fan;
+    uint8_t *out_row = out + row * out_row_bytes;
+#define TERRACE_COMBINE_BODY(WD) \
+    combine_row_chunk<SRC, OUT, WD>(src, src_row_bytes, idx_row, w, row * fan, fan, hidden, c, out_row)
+    if (!w) TERRACE_COMBINE_BODY(kWNone);
+    else if (w_dtype == TERRACE_F32) TERRACE_COMBINE_BODY(TERRACE_F32);
+    else if (w_dtype == TERRACE_BF16) TERRACE_COMBINE_BODY(TERRACE_BF16);
+    else TERRACE_COMBINE_BODY(TERRACE_F16);
+#undef TERRACE_COMBINE_BODY
 }
 
 // Element path: any hidden, any alignment.
@@ -624,18 +678,8 @@ static void launch_combine_so(const void *src, const int64_t *idx, const void *w
     const int bt = one_wave ? kWave : kBlock;
     const int slices = (int)((chunks + bt - 1) / bt);
     const unsigned grid = (unsigned)(n_out * slices);
-#define TERRACE_COMBINE_LAUNCH(F)                                                                                 \
-    if (one_wave)                                                                                                 \
-        combine_kernel<SRC, OUT, F, kWave><<<grid, kWave, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype,     \
-                                                                  n_out, fan, hidden, (uint8_t *)out, orb, slices); \
-    else                                                                                                          \
-        combine_kernel<SRC, OUT, F, kBlock><<<grid, kBlock, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype,   \
-                                                                    n_out, fan, hidden, (uint8_t *)out, orb, slices)
-    if (fan >= 8) { TERRACE_COMBINE_LAUNCH(8); }
-    else if (fan >= 4) { TERRACE_COMBINE_LAUNCH(4); }
-    else if (fan >= 2) { TERRACE_COMBINE_LAUNCH(2); }
-    else { TERRACE_COMBINE_LAUNCH(1); }
-#undef TERRACE_COMBINE_LAUNCH
+    combine_kernel<SRC, OUT><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, fan, hidden,
+                                                 (uint8_t *)out, orb, slices);
 }
 
 template <int SRC>
@@ -653,7 +697,7 @@ int launch_combine(const void *src, int src_dtype, const int64_t *idx, const voi
     const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
     const int n = src_dtype == TERRACE_F32 ? 4 : (src_dtype == TERRACE_FP8_E4M3_B128 ? 16 : 8);
     const bool vec = hidden % n == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
-                     srb % 16 == 0 && orb % 16 == 0;
+                     srb % 16 == 0 && orb % 16 == 0 && ((uintptr_t)w & 3) == 0;   // weights are read as dwords
     if (!vec) {
         const int grid = (int)(n_out > 4096 ? 4096 : n_out);
         combine_elem_kernel<<<grid, kBlock, 0, s>>>((const uint8_t *)src, src_dtype, srb, idx, w, w_dtype, n_out, fan,
