@@ -213,6 +213,33 @@ TERRACE_API int terrace_unpack_planes(const void *packed, int64_t row_bytes, int
                                       int64_t a_bytes, void *b, int64_t b_bytes, void *c, int64_t c_bytes,
                                       terrace_stream_t stream);
 
+/* ---- zero-copy wire containers: the three stage kernels write / read the containers themselves ----
+ * (the follow-up terrace/ta2a_pack.py:462-466 asks for; layouts as terrace_pack_planes above)
+ *
+ * terrace_k2_pack_wire = terrace_k2_pack, but the slot-id and gate planes are written straight into the
+ * Hop-A small container wire [T*M, wire_words] i64: words [0,q) of a row are its ascending slot ids, the
+ * gates follow from word q, the rest of the row is zeroed (wire_words >= q + ceil(q*gate_bytes/8)).
+ * terrace_k1_arrival_wire = terrace_k1_arrival reading that container as it arrived (rwire) and writing the
+ * Hop-B container meta [P, 2] i64 (word 0 slot id, word 1 the gate then zeros); slot_idx / gate_pairs are
+ * optional extra outputs.  terrace_regroup_wire = terrace_regroup reading my_slot / my_gate out of an
+ * arrived Hop-B container my_meta [P, 2] (the gate plane is gathered only when permuted_gate != NULL). */
+TERRACE_API int terrace_k2_pack_wire(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T,
+                                     int64_t row_bytes, int gate_bytes, int k, int world, int n_experts, int rpn,
+                                     int groups_m, void *payload, int64_t *wire, int wire_words, int64_t *u_src,
+                                     int64_t *node_counts, int64_t *u_node, int64_t *inverse, int64_t *node_offsets,
+                                     int64_t *pair_table, int64_t *sort_order, int64_t *token_rows, void *gate_sorted,
+                                     int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+TERRACE_API int terrace_k1_arrival_wire(const void *rx, const int64_t *rwire, int wire_words, int64_t R,
+                                        int64_t row_bytes, int gate_bytes, int quota, int epr, int rpn, int my_local,
+                                        void *send_buf, int64_t *meta, int64_t *r_idx, int64_t *slot_idx,
+                                        void *gate_pairs, int64_t *i_send, int64_t *pair_pos, int32_t *status,
+                                        void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+TERRACE_API int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta, int64_t P, int64_t row_bytes,
+                                     int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted,
+                                     void *permuted_gate, int64_t *order, int64_t *dest, uint8_t *kept,
+                                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status,
+                                     void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+
 /* ---- the general (data-dependent fan-out) branch and the seam's entry helper ---- */
 
 /* plan_ta2a without groups_m (terrace/ta2a.py:70-275, general branch): one send row per occupied

@@ -111,10 +111,17 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
     G *__restrict__ gate_rows, int64_t *__restrict__ u_src, int64_t *__restrict__ u_node,
     int64_t *__restrict__ inverse, int64_t *__restrict__ pair_table, int64_t *__restrict__ sort_order,
     int64_t *__restrict__ token_rows, G *__restrict__ gate_sorted, int32_t *__restrict__ pos32,
-    int32_t *__restrict__ status) {
+    int32_t *__restrict__ status, int64_t mask_pitch, int64_t gate_pitch, int gate_pad) {
     const int lane = lane_id();
     const int unit = blockIdx.x * kWavesPerBlock + wave_in_block();
     if (unit >= n_units) return;
+    // mask / gate_rows may be [rows, quota] tables inside wider rows (a wire container): cell (r, i) of
+    // each is at r*pitch + i, and the gate_pad elements after a row's gates are zeroed
+    auto zero_row = [&](int64_t r) {
+        for (int i = 0; i < quota; ++i) mask[r * mask_pitch + i] = 0;
+        if (gates)
+            for (int i = 0; i < quota + gate_pad; ++i) gate_rows[r * gate_pitch + i] = G(0);
+    };
     int cur = lane < n_nodes ? table[(int64_t)lane * n_units + unit] : 0;      // lane n: cursor of node n
     int fault = 0, occupied = 0, off_quota = 0;
     for (int c = 0; c < kTokChunks; ++c) {
@@ -181,14 +188,8 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
                 if (gate_sorted) gate_sorted[t * k + j] = G(0);
             }
 #pragma unroll
-            for (int m = 0; m < KMAX; ++m) {
-                if (m < M && rows[m] >= 0) {
-                    for (int i = 0; i < quota; ++i) {
-                        mask[(int64_t)rows[m] * quota + i] = 0;
-                        if (gates) gate_rows[(int64_t)rows[m] * quota + i] = G(0);
-                    }
-                }
-            }
+            for (int m = 0; m < KMAX; ++m)
+                if (m < M && rows[m] >= 0) zero_row(rows[m]);
         }
         // ---- the token's experts ----
 #pragma unroll
@@ -209,8 +210,12 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
             for (int mm = 0; mm < KMAX; ++mm)
                 if (mm == m) r = rows[mm];
             const int64_t cell = (int64_t)r * quota + within;
-            mask[cell] = ej - nj * slots;
-            if (gates) gate_rows[cell] = gates[t * k + j];
+            mask[(int64_t)r * mask_pitch + within] = ej - nj * slots;
+            if (gates) {
+                gate_rows[(int64_t)r * gate_pitch + within] = gates[t * k + j];
+                if (within == 0)
+                    for (int z = 0; z < gate_pad; ++z) gate_rows[(int64_t)r * gate_pitch + quota + z] = G(0);
+            }
             if (inverse) inverse[t * k + j] = r;
             if (pair_table) pair_table[t * k + rank] = cell;
             if (sort_order) sort_order[t * k + rank] = j;
@@ -224,10 +229,7 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
         for (int64_t r = used + lane; r < S; r += kWave) {
             u_src[r] = 0;
             if (u_node) u_node[r] = 0;
-            for (int i = 0; i < quota; ++i) {
-                mask[r * quota + i] = 0;
-                if (gates) gate_rows[r * quota + i] = G(0);
-            }
+            zero_row(r);
         }
     }
     if (!status) return;
@@ -248,23 +250,26 @@ static void launch_place(const int64_t *expert_idx, const void *gates, int64_t T
                          int n_experts, int M, const Units &u, const int32_t *table, int64_t *mask, void *gate_rows,
                          int64_t *u_src, int64_t *u_node, int64_t *inverse, int64_t *pair_table,
                          int64_t *sort_order, int64_t *token_rows, void *gate_sorted, int32_t *pos32,
-                         int32_t *status, hipStream_t s) {
+                         int32_t *status, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
     const int blocks = (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock;
     if (u.chunks == 1)
         k2_place_kernel<KMAX, G, 1><<<blocks, kBlock, 0, s>>>(
             expert_idx, (const G *)gates, T, k, slots, n_nodes, n_experts, M, k / M, u.n_units, table, mask,
-            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status);
+            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status,
+            mask_pitch, gate_pitch, gate_pad);
     else
         k2_place_kernel<KMAX, G, 4><<<blocks, kBlock, 0, s>>>(
             expert_idx, (const G *)gates, T, k, slots, n_nodes, n_experts, M, k / M, u.n_units, table, mask,
-            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status);
+            (G *)gate_rows, u_src, u_node, inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, status,
+            mask_pitch, gate_pitch, gate_pad);
 }
 
 int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
                  int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                  int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                  int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, hipStream_t s) {
+                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, int64_t mask_pitch,
+                 int64_t gate_pitch, int gate_pad, hipStream_t s) {
     const Units u = token_units(T, n_nodes);
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + units_table_bytes(u));
@@ -282,7 +287,8 @@ int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gate
     launch_scan(u, table, node_counts, nullptr, node_offsets, status, s);
 #define TERRACE_PLACE(KM, G)                                                                                       \
     launch_place<KM, G>(expert_idx, gates, T, k, slots, n_nodes, n_experts, groups_m, u, table, mask, gate_rows,   \
-                        u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_sorted, pos32, status, s)
+                        u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_sorted, pos32, status,      \
+                        mask_pitch, gate_pitch, gate_pad, s)
     if (k <= 8) {
         if (gate_bytes == 4) TERRACE_PLACE(8, uint32_t);
         else TERRACE_PLACE(8, uint16_t);

@@ -45,8 +45,17 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
     int64_t sub;
     int div;
     int n_buckets;
+    // the plane may be a [rows, width] table sitting inside wider rows (a wire container): item
+    // r*width + i is then at plane[r*pitch + i]
+    int width = 1;
+    int64_t pitch = 1;
+    __device__ __forceinline__ int64_t at(int64_t item) const {
+        if (pitch == width) return plane[item];
+        const int64_t r = item / width;
+        return plane[r * pitch + (item - r * width)];
+    }
     __device__ __forceinline__ int operator()(int64_t item, bool *bad) const {
-        const int64_t v = plane[item] - sub;
+        const int64_t v = at(item) - sub;
         if (v < 0 || v >= (int64_t)n_buckets * div) {
             *bad = true;
             return 0;
@@ -344,19 +353,33 @@ struct EmitNothing {
 };
 
 struct EmitArrival {         // terrace/ops/__init__.py:287-299
-    const int64_t *rslot;
-    const void *rgate;
+    const int64_t *rslot;    // [R, quota] at row pitch slot_pitch (int64 elements)
+    const void *rgate;       // [R, quota] at row pitch gate_pitch (gate elements)
     int gate_bytes, quota;
+    int64_t slot_pitch, gate_pitch;
     void *gate_pairs;
     int64_t *r_idx, *slot_idx, *pair_pos;
     int32_t *pos32;
+    int64_t *meta;           // Hop-B container [P, 2]: word 0 the slot id, word 1 the gate then zeros; or NULL
     static constexpr bool kTallies = false;
     __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, const int32_t *, int *) const {
-        r_idx[dest] = p / quota;
-        slot_idx[dest] = rslot[p];
+        const int64_t r = p / quota;
+        const int i = (int)(p - r * quota);
+        const int64_t slot = rslot[r * slot_pitch + i];
+        r_idx[dest] = r;
+        if (slot_idx) slot_idx[dest] = slot;
+        uint32_t gbits = 0;
         if (rgate) {
-            if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = ((const uint32_t *)rgate)[p];
-            else ((uint16_t *)gate_pairs)[dest] = ((const uint16_t *)rgate)[p];
+            if (gate_bytes == 4) gbits = ((const uint32_t *)rgate)[r * gate_pitch + i];
+            else gbits = ((const uint16_t *)rgate)[r * gate_pitch + i];
+            if (gate_pairs) {
+                if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = gbits;
+                else ((uint16_t *)gate_pairs)[dest] = (uint16_t)gbits;
+            }
+        }
+        if (meta) {
+            meta[2 * (int64_t)dest] = slot;
+            meta[2 * (int64_t)dest + 1] = (int64_t)(uint64_t)gbits;
         }
         pos32[p] = dest;
         if (pair_pos) pair_pos[p] = dest;
@@ -420,6 +443,8 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
     int64_t *mask, *u_src, *u_node, *inverse, *pair_table, *sort_order, *token_rows;
     void *gate_rows, *gate_sorted;
     int32_t *pos32;
+    int64_t mask_pitch, gate_pitch;      // row pitches of the mask / gate_rows planes, in their own elements
+    int gate_pad;                        // gate elements to zero after a row's quota gates
     // status word 1 receives the number of occupied (token, node) pairs, word 2 the number of
     // those holding other than k/M experts: the two quantities terrace/ta2a.py:170-204 checks.
     static constexpr bool kTallies = true;
@@ -475,16 +500,21 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
             if (r / quota != m) return;
             const int i = r - m * quota;
             const int64_t cell = (int64_t)row * quota + i;
-            mask[cell] = e >= 0 ? e - ids.node(j) * slots : 0;
+            mask[(int64_t)row * mask_pitch + i] = e >= 0 ? e - ids.node(j) * slots : 0;
             if (gates) {
+                const int64_t gcell = (int64_t)row * gate_pitch + i;
                 if (gate_bytes == 4) {
                     const uint32_t gv = ((const uint32_t *)gates)[t * k + j];
-                    ((uint32_t *)gate_rows)[cell] = gv;
+                    ((uint32_t *)gate_rows)[gcell] = gv;
                     if (gate_sorted) ((uint32_t *)gate_sorted)[t * k + r] = gv;
+                    if (i == 0)
+                        for (int z = 0; z < gate_pad; ++z) ((uint32_t *)gate_rows)[gcell + quota + z] = 0u;
                 } else {
                     const uint16_t gv = ((const uint16_t *)gates)[t * k + j];
-                    ((uint16_t *)gate_rows)[cell] = gv;
+                    ((uint16_t *)gate_rows)[gcell] = gv;
                     if (gate_sorted) ((uint16_t *)gate_sorted)[t * k + r] = gv;
+                    if (i == 0)
+                        for (int z = 0; z < gate_pad; ++z) ((uint16_t *)gate_rows)[gcell + quota + z] = (uint16_t)0;
                 }
             }
             if (inverse) inverse[t * k + j] = row;
@@ -528,11 +558,11 @@ __global__ __launch_bounds__(kBlock) void fill_zero_kernel(uint8_t *__restrict__
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gather_elems_kernel(const T *__restrict__ src,
                                                               const int32_t *__restrict__ idx, int64_t n,
-                                                              T *__restrict__ out) {
+                                                              int64_t src_pitch, T *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     const int32_t a = idx[i];
-    out[i] = a < 0 ? T(0) : src[a];
+    out[i] = a < 0 ? T(0) : src[(int64_t)a * src_pitch];
 }
 
 __global__ void empty_outputs_kernel(int64_t *hist, float *hist_f, int64_t *offsets, int n, int32_t *status) {
@@ -664,21 +694,23 @@ size_t k1_workspace(int64_t R, int quota, int rpn) {
 int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                    int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
                    int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
-                   size_t ws_bytes, hipStream_t s) {
+                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, hipStream_t s) {
     if (R < 0 || quota <= 0 || epr <= 0 || rpn <= 0 || rpn > kMaxBuckets || my_local < 0 || my_local >= rpn ||
-        !i_send || (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0)
+        !i_send || (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0 || slot_pitch < quota || gate_pitch < quota)
         return TERRACE_EINVAL;
     const int64_t P = R * quota;
     if (P >= (int64_t)1 << 31) return TERRACE_EINVAL;
     if (P == 0) return empty_outputs(i_send, nullptr, nullptr, rpn, status, s);
-    if (!rslot || !r_idx || !slot_idx || !ws || (rx && !send_buf) || (rgate && !gate_pairs)) return TERRACE_EINVAL;
+    if (!rslot || !r_idx || (!slot_idx && !meta) || !ws || (rx && !send_buf) || (rgate && !gate_pairs && !meta))
+        return TERRACE_EINVAL;
     const Units u = make_units(P, rpn);
     const size_t table_bytes = units_table_bytes(u);
     if (ws_bytes < table_bytes + align_up((size_t)P * sizeof(int32_t), 256)) return TERRACE_ENOSPC;
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
-    KeyAffine key{rslot, 0, epr, rpn};
-    EmitArrival emit{rslot, rgate, gate_bytes, quota, gate_pairs, r_idx, slot_idx, pair_pos, pos32};
+    KeyAffine key{rslot, 0, epr, rpn, quota, slot_pitch};
+    EmitArrival emit{rslot, rgate, gate_bytes, quota, slot_pitch, gate_pitch, gate_pairs, r_idx, slot_idx, pair_pos,
+                     pos32, meta};
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
@@ -723,8 +755,9 @@ size_t regroup_workspace(int64_t P, int epr, int64_t capacity) {
 int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
                 int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
                 int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
-                int32_t *status, void *ws, size_t ws_bytes, hipStream_t s) {
+                int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, hipStream_t s) {
     if (P < 0 || epr <= 0 || epr > kMaxBuckets || my_local < 0 || !tokens_per_expert || row_bytes < 0 ||
+        slot_pitch < 1 || gate_pitch < 1 ||
         (gate_bytes != 2 && gate_bytes != 4) || P >= (int64_t)1 << 31 ||
         (capacity >= 0 && (int64_t)epr * capacity >= (int64_t)1 << 31))
         return TERRACE_EINVAL;
@@ -744,7 +777,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     int32_t *table = (int32_t *)ws;
     int32_t *order32 = (int32_t *)((char *)ws + table_bytes);
     int32_t *gidx = (int32_t *)((char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
-    KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr};
+    KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr, 1, slot_pitch};
     EmitRegroup emit{capacity, order, dest, kept, order32};
     int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK) return rc;
@@ -762,9 +795,9 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     if (my_gate && places > 0) {
         const int grid = (int)((places + kBlock - 1) / kBlock);
         if (gate_bytes == 4)
-            gather_elems_kernel<uint32_t><<<grid, kBlock, 0, s>>>((const uint32_t *)my_gate, src_of_place, places, (uint32_t *)permuted_gate);
+            gather_elems_kernel<uint32_t><<<grid, kBlock, 0, s>>>((const uint32_t *)my_gate, src_of_place, places, gate_pitch, (uint32_t *)permuted_gate);
         else
-            gather_elems_kernel<uint16_t><<<grid, kBlock, 0, s>>>((const uint16_t *)my_gate, src_of_place, places, (uint16_t *)permuted_gate);
+            gather_elems_kernel<uint16_t><<<grid, kBlock, 0, s>>>((const uint16_t *)my_gate, src_of_place, places, gate_pitch, (uint16_t *)permuted_gate);
     }
     rc = check_launch();
     if (rc != TERRACE_OK || !node_rx) return rc;
@@ -805,12 +838,12 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
                     int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                     int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
                     int64_t *token_rows, void *gate_sorted, int32_t *status, const Units &u, int32_t *table,
-                    int32_t *pos32, hipStream_t s) {
+                    int32_t *pos32, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
     const int quota = k / groups_m;
     KeyRun<KMAX> key{expert_idx, k, groups_m, quota, slots, n_nodes};
     EmitPack<KMAX> emit{expert_idx, gates, gate_bytes, k, groups_m, quota, slots, n_experts,
                         mask, u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_rows, gate_sorted,
-                        pos32};
+                        pos32, mask_pitch, gate_pitch, gate_pad};
     int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
@@ -820,7 +853,10 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
                 int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
                 void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node, int64_t *inverse,
                 int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order, int64_t *token_rows,
-                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, hipStream_t s) {
+                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, int64_t mask_pitch, int64_t gate_pitch,
+                int gate_pad, hipStream_t s) {
+    if (mask_pitch <= 0) mask_pitch = groups_m > 0 ? k / groups_m : 0;       // dense planes
+    if (gate_pitch <= 0) gate_pitch = groups_m > 0 ? k / groups_m : 0;
     if (T < 0 || k <= 0 || world <= 0 || rpn <= 0 || n_experts <= 0 || groups_m <= 0 || world % rpn ||
         n_experts % world || k % groups_m || row_bytes < 0 || (gate_bytes != 2 && gate_bytes != 4) || !node_counts)
         return TERRACE_EINVAL;
@@ -834,7 +870,8 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
     if (k2_token_path_applies(k, n_nodes))
         return run_k2_token(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts,
                             groups_m, payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets,
-                            pair_table, sort_order, token_rows, gate_sorted, status, ws, s);
+                            pair_table, sort_order, token_rows, gate_sorted, status, ws, mask_pitch, gate_pitch,
+                            gate_pad, s);
     const Units u = make_units(S, n_nodes);
     const size_t table_bytes = units_table_bytes(u);
     int32_t *table = (int32_t *)ws;
@@ -842,7 +879,7 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
 #define TERRACE_K2(KM)                                                                                        \
     run_k2_t<KM>(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts, groups_m, \
                  payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets, pair_table,     \
-                 sort_order, token_rows, gate_sorted, status, u, table, pos32, s)
+                 sort_order, token_rows, gate_sorted, status, u, table, pos32, mask_pitch, gate_pitch, gate_pad, s)
     if (k <= 8) return TERRACE_K2(8);
     if (k <= 16) return TERRACE_K2(16);
     return TERRACE_K2(0);

@@ -39,6 +39,7 @@ int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gate
                  int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                  int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                  int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, hipStream_t s);
+                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, int64_t mask_pitch,
+                 int64_t gate_pitch, int gate_pad, hipStream_t s);
 
 }  // namespace terrace

@@ -53,6 +53,12 @@ SIGNATURES = {
     "terrace_combine": (_I, [_P, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
     "terrace_pack_planes": (_I, [_P, _L, _P, _L, _P, _L, _L, _L, _P, _P]),
     "terrace_unpack_planes": (_I, [_P, _L, _L, _P, _L, _P, _L, _P, _L, _P]),
+    "terrace_k2_pack_wire": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I,
+                                  _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_k1_arrival_wire": (_I, [_P, _P, _I, _L, _L, _I, _I, _I, _I, _I,
+                                     _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_regroup_wire": (_I, [_P, _P, _L, _L, _I, _I, _I, _L,
+                                  _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_plan_general_workspace": (_Z, [_L, _I]),
     "terrace_plan_general": (_I, [_P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_build_mask": (_I, [_P, _P, _L, _I, _L, _P, _P, _P]),

@@ -210,6 +210,108 @@ def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extr
     return out
 
 
+def wire_words(quota: int, gate_bytes: int) -> int:
+    """int64 words of one Hop-A small container row: ``quota`` slot ids, then ``quota`` gates padded to a word."""
+    return quota + (quota * gate_bytes + 7) // 8
+
+
+def k2_pack_wire(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+    """``k2_pack_raw(..., extras=True)`` with the slot-id and gate planes written by the kernel straight
+    into the Hop-A small container: returns ((payload, mask, gate_rows, u_src, node_counts), extras) where
+    ``extras["wire"]`` is the [T*M, W] int64 container and ``mask`` / ``gate_rows`` are views into it."""
+    _require()
+    _hip.need_device(hidden, expert_idx, gates)
+    _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+    hidden, expert_idx, gates = hidden.contiguous(), expert_idx.contiguous(), gates.contiguous()
+    dev = expert_idx.device
+    T, k = expert_idx.shape
+    H = hidden.shape[1]
+    S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
+    gb = gates.element_size()
+    W = wire_words(q, gb)
+    payload = torch.empty((S, H), dtype=hidden.dtype, device=dev)
+    wire = torch.empty((S, W), dtype=torch.int64, device=dev)
+    u_src = torch.empty((S,), dtype=torch.int64, device=dev)
+    node_counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
+    ex = {"u_node": torch.empty((S,), dtype=torch.int64, device=dev),
+          "inverse": torch.empty((T * k,), dtype=torch.int64, device=dev),
+          "node_offsets": torch.empty((n_nodes,), dtype=torch.int64, device=dev),
+          "pair_table": torch.empty((T, k), dtype=torch.int64, device=dev),
+          "sort_order": torch.empty((T, k), dtype=torch.int64, device=dev),
+          "token_rows": torch.empty((T, groups_m), dtype=torch.int64, device=dev),
+          "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
+    _hip.call("terrace_k2_pack_wire", _hip.ptr(hidden), _hip.ptr(expert_idx), _hip.ptr(gates), T,
+              H * hidden.element_size(), gb, k, world, n_experts, rpn, groups_m, _hip.ptr(payload), _hip.ptr(wire), W,
+              _hip.ptr(u_src), _hip.ptr(node_counts), _hip.ptr(ex["u_node"]), _hip.ptr(ex["inverse"]),
+              _hip.ptr(ex["node_offsets"]), _hip.ptr(ex["pair_table"]), _hip.ptr(ex["sort_order"]),
+              _hip.ptr(ex["token_rows"]), _hip.ptr(ex["gate_sorted"]), _hip.ptr(st), _hip.ptr(ws), ws.numel(),
+              _hip.stream(dev))
+    per_word = 8 // gb
+    mask = wire[:, :q]
+    gate_rows = wire.view(gates.dtype)[:, q * per_word:q * per_word + q]
+    ex["status"], ex["wire"] = st, wire
+    return (payload, mask, gate_rows, u_src, node_counts), ex
+
+
+def k1_arrival_wire(rx, rwire, gate_dtype, quota, epr, rpn, my_local=0):
+    """The arrival chain reading an arrived Hop-A small container and writing the Hop-B container:
+    (send_buf, meta [P,2] int64, r_idx, i_send, pair_pos); ``meta[:, 0]`` is slot_idx and the first
+    element of word 1 (viewed in ``gate_dtype``) is gate_pairs."""
+    _require()
+    _hip.need_device(rx, rwire)
+    if rx.dim() != 2 or rwire.dim() != 2 or rwire.dtype != torch.int64 or rwire.shape[0] != rx.shape[0]:
+        raise RuntimeError("terrace::k1_arrival: rx must be [R, H] and the container [R, W] int64")
+    gb = torch.empty((), dtype=gate_dtype).element_size()
+    if gb not in (2, 4) or rwire.shape[1] < wire_words(quota, gb):
+        raise RuntimeError(f"terrace::k1_arrival: container rows of {rwire.shape[1]} words cannot hold quota {quota} "
+                           f"ids and {gate_dtype} gates")
+    if not (quota > 0 and epr > 0 and rpn > 0 and 0 <= my_local < rpn):
+        raise RuntimeError("terrace::k1_arrival: bad geometry scalars")
+    rx, rwire = rx.contiguous(), rwire.contiguous()
+    dev = rx.device
+    R, H = rx.shape
+    P = R * quota
+    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev)
+    meta = torch.empty((P, 2), dtype=torch.int64, device=dev)
+    r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
+    i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
+    pair_pos = torch.empty((P,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
+    _hip.call("terrace_k1_arrival_wire", _hip.ptr(rx), _hip.ptr(rwire), rwire.shape[1], R, H * rx.element_size(), gb,
+              quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(meta), _hip.ptr(r_idx), None, None,
+              _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return send_buf, meta, r_idx, i_send, pair_pos
+
+
+def regroup_wire(node_rx, my_meta, gate_dtype, epr, my_local=0):
+    """Drop-less expert-order regroup reading slot ids and gates out of an arrived Hop-B container:
+    (permuted, order, tokens_per_expert, place, permuted_gate)."""
+    _require()
+    _hip.need_device(node_rx, my_meta)
+    if my_meta.dim() != 2 or my_meta.shape[1] != 2 or my_meta.dtype != torch.int64:
+        raise RuntimeError("regroup: the Hop-B container must be [P, 2] int64")
+    node_rx, my_meta = node_rx.contiguous(), my_meta.contiguous()
+    dev = my_meta.device
+    P = my_meta.shape[0]
+    if node_rx.dim() != 2 or node_rx.shape[0] != P:
+        raise RuntimeError(f"regroup: node_rx {tuple(node_rx.shape)} does not have one row per pair ({P})")
+    gb = torch.empty((), dtype=gate_dtype).element_size()
+    permuted = torch.empty_like(node_rx)
+    pgate = torch.empty((P,), dtype=gate_dtype, device=dev)
+    order = torch.empty((P,), dtype=torch.int64, device=dev)
+    place = torch.empty((P,), dtype=torch.int64, device=dev)
+    tpe = torch.empty((epr,), dtype=torch.int64, device=dev)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, -1), dev)
+    _hip.call("terrace_regroup_wire", _hip.ptr(node_rx), _hip.ptr(my_meta), P, node_rx.shape[1] * node_rx.element_size(),
+              gb, epr, my_local, -1, _hip.ptr(permuted), _hip.ptr(pgate), _hip.ptr(order), _hip.ptr(place), None,
+              _hip.ptr(tpe), None, _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return permuted, order, tpe, place, pgate
+
+
 def plan_raw(expert_idx, world, n_experts, rpn, groups_m):
     """Index build only: (u_src, u_node, node_counts, inverse, extras incl. mask planes, status)."""
     _require()
@@ -774,4 +876,5 @@ __all__ = [
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
     "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
     "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table", "pair_places",
+    "wire_words", "k2_pack_wire", "k1_arrival_wire", "regroup_wire",
 ]

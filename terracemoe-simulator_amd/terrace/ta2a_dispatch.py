@@ -123,12 +123,16 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         assert k % groups_m == 0, f"k={k} not divisible by groups_m={groups_m}"
     quota = (k // groups_m) if groups_m else None
 
+    # Quota branch under the default "small" container mode: the three stage kernels write and read the
+    # wire containers themselves, so no pack / unpack pass runs at all.
+    fused_wire = quota is not None and pack_mode == "small"
     if quota is not None:
         if gates.dtype != hidden_states.dtype:
             raise RuntimeError(f"Index put requires the source and destination dtypes match, got "
                                f"{hidden_states.dtype} for the destination and {gates.dtype} for the source.")
-        (payload, mask, gate_rows, u_src, node_counts), ex = _ops.k2_pack_raw(
-            hidden_states, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+        packer = _ops.k2_pack_wire if fused_wire else (lambda *a: _ops.k2_pack_raw(*a, extras=True))
+        (payload, mask, gate_rows, u_src, node_counts), ex = packer(
+            hidden_states, expert_idx, gates, world, n_experts, rpn, groups_m)
         _plan._guard(ex["status"], T, k, n_nodes, groups_m)
         u_node = ex["u_node"]
     else:
@@ -136,7 +140,9 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
             hidden_states, expert_idx, gates, world, n_experts, rpn)
 
     # Hop A (loop-back): what was packed for the wire is what arrives
-    if pack_mode == "small":
+    if fused_wire:
+        rx, rwire = payload, ex["wire"]
+    elif pack_mode == "small":
         sbuf, lay = _pk.hopa_pack_small(gate_rows, mask)
         rgate, rmask = _pk.hopa_unpack_small(sbuf, lay)
         _pk.assert_not_aliased(sbuf, rgate, rmask)
@@ -149,23 +155,28 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         rx, rmask, rgate = payload, mask, gate_rows
     R = rx.shape[0]
 
-    if quota is not None:
-        exp_rx, gate_pairs, r_idx, slot_idx, _i_send, pair_pos = _ops.k1_arrival_raw(
-            rx, rmask, rgate, quota, epr, rpn, my_local, want_pair_pos=True)
+    if fused_wire:
+        # Hop B (loop-back): the container the arrival kernel wrote is what the expert card reads
+        node_rx, my_meta, r_idx, _i_send, pair_pos = _ops.k1_arrival_wire(rx, rwire, gates.dtype, quota, epr, rpn,
+                                                                          my_local)
+        my_slot = my_meta[:, 0]
+        permuted, order, tokens_per_expert, place, pprobs = _ops.regroup_wire(node_rx, my_meta, gates.dtype, slots, 0)
     else:
-        r_in, s_in = _expand_arrival(rmask, slots, None)
-        exp_rx, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx, r_in, s_in, rgate, epr, rpn)
-
-    # Hop B (loop-back)
-    node_rx = exp_rx
-    if pack_mode != "off":
-        bbuf = _pk.hopb_pack_meta(slot_idx, gate_pairs)
-        my_slot, my_gate = _pk.hopb_unpack_meta(bbuf, gate_pairs.dtype)
-    else:
-        my_slot, my_gate = slot_idx, gate_pairs
-
-    # every slot of the node is local under loop-back
-    permuted, order, tokens_per_expert, place, pprobs = _regroup_with_place(node_rx, my_slot, slots, 0, my_gate)
+        if quota is not None:
+            exp_rx, gate_pairs, r_idx, slot_idx, _i_send, pair_pos = _ops.k1_arrival_raw(
+                rx, rmask, rgate, quota, epr, rpn, my_local, want_pair_pos=True)
+        else:
+            r_in, s_in = _expand_arrival(rmask, slots, None)
+            exp_rx, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx, r_in, s_in, rgate, epr, rpn)
+        # Hop B (loop-back)
+        node_rx = exp_rx
+        if pack_mode != "off":
+            bbuf = _pk.hopb_pack_meta(slot_idx, gate_pairs)
+            my_slot, my_gate = _pk.hopb_unpack_meta(bbuf, gate_pairs.dtype)
+        else:
+            my_slot, my_gate = slot_idx, gate_pairs
+        # every slot of the node is local under loop-back
+        permuted, order, tokens_per_expert, place, pprobs = _regroup_with_place(node_rx, my_slot, slots, 0, my_gate)
 
     st = TA2AState()
     st.u_src, st.r_idx, st.order = u_src, r_idx, order

@@ -324,6 +324,51 @@ def test_seam_backward_is_the_adjoint(world, rpn, E, T, k, M, H, branch):
     assert not p2.requires_grad and not g2.requires_grad and torch.equal(p2, permuted.detach())
 
 
+@pytest.mark.parametrize("fmt", ["f32", "bf16", "f16"])
+def test_stage_kernels_write_and_read_the_wire_containers_themselves(literals, fmt):
+    """The zero-copy forms against the two-step forms (planes, then pack / unpack kernels): the same
+    container bits, padding included, and the same downstream planes."""
+    import terrace.ops as tops
+    from terrace import ta2a_pack
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"] + [[64, 8, 256, 3000, 8, 4], [64, 8, 256, 700, 24, 2], [1024, 8, 1024, 300, 4, 2]]:
+        announce("wire", (world, rpn, E, T, k, M), fmt)
+        q, epr, slots = k // M, E // world, (E // world) * rpn
+        e = equal_quota_routing(T, k, E, world // rpn, M, 13)
+        g = torch.Generator().manual_seed(T)
+        x = torch.randn(T, 32, generator=g).to(DT[fmt]).to(DEV)
+        gates = torch.rand(T, k, generator=g).to(DT[fmt]).to(DEV)
+        ed = torch.from_numpy(e).to(DEV)
+        plain, pex = tops.k2_pack_raw(x, ed, gates, world, E, rpn, M, extras=True)
+        fused, fex = tops.k2_pack_wire(x, ed, gates, world, E, rpn, M)
+        want_wire, lay = ta2a_pack.hopa_pack_small(plain[2], plain[1])
+        assert fex["wire"].shape == want_wire.shape == (T * M, lay.words)
+        assert torch.equal(fex["wire"], want_wire)
+        for a, b in zip(fused, plain):
+            assert torch.equal(a, b)
+        for name in ("u_node", "inverse", "node_offsets", "pair_table", "sort_order", "token_rows", "gate_sorted"):
+            assert torch.equal(fex[name], pex[name]), name
+        assert fex["status"].tolist() == pex["status"].tolist()
+        # arrival: reads the container, writes the Hop-B container
+        send, gp, r_idx, slot_idx, i_send, pair_pos = tops.k1_arrival_raw(plain[0], plain[1], plain[2], q, epr, rpn, 0,
+                                                                          want_pair_pos=True)
+        send2, meta, r_idx2, i_send2, pair_pos2 = tops.k1_arrival_wire(fused[0], fex["wire"], DT[fmt], q, epr, rpn, 0)
+        assert torch.equal(meta, ta2a_pack.hopb_pack_meta(slot_idx, gp))
+        for a, b in ((send2, send), (r_idx2, r_idx), (i_send2, i_send), (pair_pos2, pair_pos)):
+            assert torch.equal(a, b)
+        # expert card: reads the Hop-B container
+        perm, order, tpe, pgate = tops.regroup(send, slot_idx, slots, 0, None, my_gate=gp)
+        perm2, order2, tpe2, place2, pgate2 = tops.regroup_wire(send2, meta, DT[fmt], slots, 0)
+        for a, b in ((perm2, perm), (order2, order), (tpe2, tpe), (pgate2, pgate)):
+            assert torch.equal(a, b)
+        assert torch.equal(place2[order2], torch.arange(order2.numel(), device=DEV))
+    with pytest.raises(RuntimeError, match="cannot hold"):
+        tops.k1_arrival_wire(torch.zeros(4, 8, device=DEV), torch.zeros(4, 2, dtype=torch.int64, device=DEV),
+                             torch.float32, 2, 1, 4, 0)
+    empty = tops.k1_arrival_wire(torch.zeros(0, 8, device=DEV), torch.zeros(0, 3, dtype=torch.int64, device=DEV),
+                                 torch.float32, 2, 1, 4, 0)
+    assert empty[1].shape == (0, 2) and empty[3].tolist() == [0, 0, 0, 0]
+
+
 def test_seam_refuses_process_groups_and_mismatched_probs():
     from terrace.ta2a_dispatch import ta2a_permute
     announce("seam refusals")
