@@ -1,14 +1,16 @@
 // Row movers: the HBM-bound kernels of the dispatch/combine path.
 //
-//   copy_kernel          y = x                              (streaming-copy roofline probe)
-//   scatter_rows_kernel  dst[pos[r*fan+f]] = src[r]         (Hop-A pack, Hop-B arrival: a source
-//                                                            row is read once and written fan times)
-//   gather_rows_kernel   out[i] = src[idx[i]] or zeros      (expert-order regroup, capacity padding)
-//   combine_kernel       out[i] = sum_j w[i,j]*src[idx[i,j]] in fp32, one rounding at the end
+//   copy_kernel                   y = x                           (streaming-copy roofline probe)
+//   scatter_rows_{sliced,aligned} dst[pos[r*fan+f]] = src[r]      (Hop-A pack, Hop-B arrival: a source
+//                                                                  row is read once and written fan times)
+//   gather_rows_{sliced,flat}     out[i] = src[idx[i]] or zeros   (expert-order regroup, capacity padding)
+//   combine_kernel                out[i] = sum_j w[i,j]*src[idx[i,j]] in fp32, one rounding at the end
+//   planes_kernel                 wire containers: row = a | b | c | zero pad, and the inverse split
 //
-// A workgroup is 256 threads split into sub-groups of 64/128/256 lanes; a sub-group owns one
-// row at a time, so every index it needs is wave-uniform and each lane keeps several
-// independent 16-byte loads in flight.  Nothing here is a contraction: no MFMA, no LDS.
+// Rows that are multiples of 16 bytes move as one 16-byte vector per lane in one-wave workgroups whose
+// stores each cover one aligned kilobyte of the destination.  Other widths take scatter_rows_kernel /
+// gather_rows_kernel: 256-thread workgroups split into sub-groups of 64/128/256 lanes, a sub-group
+// owning one row at a time with 8/4/2/1-byte lanes.  Nothing here is a contraction: no MFMA, no LDS.
 #include "common.hpp"
 
 namespace terrace {
