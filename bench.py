@@ -1,6 +1,6 @@
 """Benchmark of one rank's dispatch/combine path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--graph]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM: T-Route -> dispatch index build + Hop-A deduplicated pack -> Hop-B arrival chain ->
@@ -45,6 +45,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture the step into a HIP graph and time its replays (reported beside the eager "
+                         "figure, which stays `value`)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1 << 20,
                     help="tokens of the workload the CPU baseline runs on (default: all of them)")
     return ap.parse_args()
@@ -202,6 +205,33 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # ---- optional: the same step as one HIP graph (launch overhead off the critical path) ----
+    graph_rec = None
+    if args.graph:
+        y_eager = step()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_graph = step()
+        same = True
+        for _ in range(3):                 # replays interleaved with eager work must all reproduce the eager result
+            graph.replay()
+            torch.cuda.synchronize()
+            same = same and bool(torch.equal(y_graph, y_eager))
+            step()
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_rec = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / args.steps, 4),
+                     "replays_match_eager": same}
+
     # ---- per-stage timings (each stage alone, HIP events on the launch stream) ----
     nbytes = configs.algorithmic_bytes(cfg)
     reps = max(args.steps, 5)
@@ -298,6 +328,8 @@ def main():
         "stages": stages, "kernels": kern, "roofline": roofline,
         "library": os.path.relpath(st.lib, ROOT),
     }
+    if graph_rec is not None:
+        out["hip_graph"] = graph_rec
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
         out["cpu_baseline"]["host_cores_available"] = os.cpu_count()
