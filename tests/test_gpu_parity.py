@@ -537,3 +537,48 @@ def test_hopb_meta_and_container_errors():
         pk.hopa_pack_small(torch.zeros(2, 2, device=DEV), ids[:2].int())
     with pytest.raises(RuntimeError, match="shape"):
         pk.hopb_pack_meta(ids[:2], torch.zeros(3, device=DEV))
+
+
+@pytest.mark.parametrize("row_bytes", [16, 48, 1024, 1040, 7392, 14336, 40, 6, 3])
+def test_row_movers_at_every_base_alignment(row_bytes):
+    """Straight through the C ABI with source and destination bases at 16-byte-granular (and, for
+    narrow rows, odd) offsets: the kilobyte-aligned chunking must neither skip nor overrun a byte."""
+    from ctypes import c_void_p
+    from terrace import _hip
+    announce("mover alignment", row_bytes)
+    lib = _hip.load()
+    g = torch.Generator().manual_seed(row_bytes)
+    n_src, n_out, fan = 37, 53, 3
+    step = 16 if row_bytes % 16 == 0 else (8 if row_bytes % 8 == 0 else 1)
+    stream = _hip.stream(torch.device(DEV))
+    for off_src, off_dst in [(0, 0), (step, 0), (0, step), (3 * step, 5 * step), (63 * step, 62 * step)]:
+        pad = 4096
+        src_buf = torch.randint(0, 256, (pad + n_src * row_bytes,), dtype=torch.uint8, generator=g).to(DEV)
+        src = src_buf[off_src:off_src + n_src * row_bytes].view(n_src, row_bytes)
+        idx = torch.randint(0, n_src, (n_out,), generator=g)
+        idx[7] = -1
+        out_buf = torch.full((pad + n_out * row_bytes + pad,), 0xAB, dtype=torch.uint8, device=DEV)
+        rc = lib.terrace_gather_rows(c_void_p(src.data_ptr()), _hip.ptr(idx.to(DEV)), n_out, row_bytes,
+                                     c_void_p(out_buf.data_ptr() + off_dst), stream)
+        assert rc == 0
+        got = out_buf[off_dst:off_dst + n_out * row_bytes].view(n_out, row_bytes).cpu()
+        want = src.cpu()[idx.clamp(min=0)]
+        want[idx < 0] = 0
+        assert torch.equal(got, want), (off_src, off_dst)
+        assert bool((out_buf[:off_dst] == 0xAB).all()) and bool((out_buf[off_dst + n_out * row_bytes:] == 0xAB).all())
+        # scatter: every destination row named at most once, a few left unnamed
+        n_dst = n_src * fan + 5
+        pos = torch.randperm(n_dst, generator=g)[:n_src * fan].view(n_src, fan).clone()
+        pos[3, 1] = -1
+        dst_buf = torch.full((pad + n_dst * row_bytes + pad,), 0xCD, dtype=torch.uint8, device=DEV)
+        rc = lib.terrace_scatter_rows(c_void_p(src.data_ptr()), _hip.ptr(pos.to(DEV)), n_src, fan, row_bytes,
+                                      c_void_p(dst_buf.data_ptr() + off_dst), stream)
+        assert rc == 0
+        got = dst_buf[off_dst:off_dst + n_dst * row_bytes].view(n_dst, row_bytes).cpu()
+        want = torch.full((n_dst, row_bytes), 0xCD, dtype=torch.uint8)
+        for r in range(n_src):
+            for f in range(fan):
+                if pos[r, f] >= 0:
+                    want[pos[r, f]] = src.cpu()[r]
+        assert torch.equal(got, want), (off_src, off_dst)
+        assert bool((dst_buf[:off_dst] == 0xCD).all()) and bool((dst_buf[off_dst + n_dst * row_bytes:] == 0xCD).all())
