@@ -61,25 +61,27 @@ __device__ __forceinline__ void best_step(float &v, int &i) {
     }
 }
 
-// Reduce over lane distances [from, to): from and to are powers of two (uniform).
-__device__ __forceinline__ void top2_range(float &a1, float &a2, int from, int to) {
-    if (from <= 1 && to > 1) top2_step<1>(a1, a2);
-    if (from <= 2 && to > 2) top2_step<2>(a1, a2);
-    if (from <= 4 && to > 4) top2_step<4>(a1, a2);
-    if (from <= 8 && to > 8) top2_step<8>(a1, a2);
-    if (from <= 16 && to > 16) top2_step<16>(a1, a2);
-    if (from <= 32 && to > 32) top2_step<32>(a1, a2);
+// Reduce over lane distances [FROM, TO): powers of two, known at compile time.
+template <int FROM, int TO>
+__device__ __forceinline__ void top2_range(float &a1, float &a2) {
+    if constexpr (FROM <= 1 && TO > 1) top2_step<1>(a1, a2);
+    if constexpr (FROM <= 2 && TO > 2) top2_step<2>(a1, a2);
+    if constexpr (FROM <= 4 && TO > 4) top2_step<4>(a1, a2);
+    if constexpr (FROM <= 8 && TO > 8) top2_step<8>(a1, a2);
+    if constexpr (FROM <= 16 && TO > 16) top2_step<16>(a1, a2);
+    if constexpr (FROM <= 32 && TO > 32) top2_step<32>(a1, a2);
 }
-__device__ __forceinline__ void best_range(float &v, int &i, int from, int to) {
-    if (from <= 1 && to > 1) best_step<1>(v, i);
-    if (from <= 2 && to > 2) best_step<2>(v, i);
-    if (from <= 4 && to > 4) best_step<4>(v, i);
-    if (from <= 8 && to > 8) best_step<8>(v, i);
-    if (from <= 16 && to > 16) best_step<16>(v, i);
-    if (from <= 32 && to > 32) best_step<32>(v, i);
+template <int FROM, int TO>
+__device__ __forceinline__ void best_range(float &v, int &i) {
+    if constexpr (FROM <= 1 && TO > 1) best_step<1>(v, i);
+    if constexpr (FROM <= 2 && TO > 2) best_step<2>(v, i);
+    if constexpr (FROM <= 4 && TO > 4) best_step<4>(v, i);
+    if constexpr (FROM <= 8 && TO > 8) best_step<8>(v, i);
+    if constexpr (FROM <= 16 && TO > 16) best_step<16>(v, i);
+    if constexpr (FROM <= 32 && TO > 32) best_step<32>(v, i);
 }
 
-// Shared epilogue: sel[0..k) holds the chosen expert ids (wave-private LDS).
+// Shared epilogue of the generic kernel: sel[0..k) holds the chosen expert ids (wave-private LDS).
 // An id outside [0, E) can only come from NaN scores (never ranked); it is clamped to 0.
 __device__ __forceinline__ void write_token(int *sel, float *raw, const float *gate_row, int k, int E, int64_t t,
                                             int64_t *expert_idx, float *gates) {
@@ -100,57 +102,70 @@ __device__ __forceinline__ void write_token(int *sel, float *raw, const float *g
 // ---------------------------------------------------------------------------------------------
 // register-resident kernel, mode "full"
 // ---------------------------------------------------------------------------------------------
-template <int VPL>
+// VPL consecutive scores per lane, LPG lanes per group (g = VPL*LPG), 64/LPG group positions per wave.
+// The token's row of gate values sits in registers beside its scores, so the lane that owns a chosen
+// expert hands over the raw gate itself and nothing is re-read from memory after the selection.
+template <int VPL, int LPG>
 __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restrict__ affinity,
                                                             const float *__restrict__ bias,
                                                             const float *__restrict__ gate_affinity, int64_t T, int E,
-                                                            int g, int k, int M, int pool, int lpg,
+                                                            int k, int M, int pool,
                                                             int64_t *__restrict__ expert_idx,
                                                             float *__restrict__ gates,
                                                             int64_t *__restrict__ group_idx) {
     extern __shared__ int32_t lds[];
+    constexpr int g = VPL * LPG;
+    constexpr int kGroupSlots = kWave / LPG;
     const int lane = lane_id();
     const int w = wave_in_block();
     int *sel = lds + w * 2 * k;
     float *raw = (float *)(sel + k);
     const int q = k / M;
-    const int my_group = lane / lpg;
-    const bool group_head = (lane & (lpg - 1)) == 0;
+    const int my_group = lane / LPG;
     float b[VPL];
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
         const int e = lane * VPL + i;
         b[i] = e < E ? bias[e] : 0.0f;
     }
-    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += (int64_t)gridDim.x * kWavesPerBlock) {
-        const float *row = affinity + t * E;
-        float s[VPL];
+    auto load_row = [&](const float *row, float *v, float fill) {
         if (E == kWave * VPL) {
-            typedef float fvec __attribute__((ext_vector_type(VPL)));
             if constexpr (VPL == 1) {
-                s[0] = row[lane];
+                v[0] = row[lane];
             } else if constexpr (VPL <= 4) {
-                const fvec v = *(const fvec *)(row + lane * VPL);
+                typedef float fvec __attribute__((ext_vector_type(VPL)));
+                const fvec x = *(const fvec *)(row + lane * VPL);
 #pragma unroll
-                for (int i = 0; i < VPL; ++i) s[i] = v[i];
+                for (int i = 0; i < VPL; ++i) v[i] = x[i];
             } else {
                 typedef float f4 __attribute__((ext_vector_type(4)));
 #pragma unroll
                 for (int c = 0; c < VPL / 4; ++c) {
-                    const f4 v = *(const f4 *)(row + lane * VPL + 4 * c);
+                    const f4 x = *(const f4 *)(row + lane * VPL + 4 * c);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) s[4 * c + i] = v[i];
+                    for (int i = 0; i < 4; ++i) v[4 * c + i] = x[i];
                 }
             }
-#pragma unroll
-            for (int i = 0; i < VPL; ++i) s[i] = __fadd_rn(s[i], b[i]);
         } else {
 #pragma unroll
             for (int i = 0; i < VPL; ++i) {
                 const int e = lane * VPL + i;
-                s[i] = e < E ? __fadd_rn(row[e], b[i]) : kNegInf;
+                v[i] = e < E ? row[e] : fill;
             }
         }
+    };
+    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += (int64_t)gridDim.x * kWavesPerBlock) {
+        float a[VPL], ga[VPL], s[VPL];
+        load_row(affinity + t * E, a, 0.0f);
+        if (gate_affinity) load_row(gate_affinity + t * E, ga, 0.0f);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int e = lane * VPL + i;
+            s[i] = e < E ? __fadd_rn(a[i], b[i]) : kNegInf;
+            if (!gate_affinity) ga[i] = a[i];
+        }
+        if (lane < k) sel[lane] = -1;
+        __builtin_amdgcn_wave_barrier();
         // group score: mean of the top two (or the top one) of the group's g values
         float a1 = kNegInf, a2 = kNegInf;
 #pragma unroll
@@ -159,29 +174,47 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             a2 = fmaxf(fminf(a1, v), a2);
             a1 = fmaxf(a1, v);
         }
-        top2_range(a1, a2, 1, lpg);
+        top2_range<1, LPG>(a1, a2);
         const bool real_group = my_group * g < E;
         float score = (pool >= 2 && g >= 2) ? __fmul_rn(__fadd_rn(a1, a2), 0.5f) : a1;
         if (!real_group) score = kNegInf;
         const int gid = real_group ? my_group : 0x7FFFFFFF;
         // top-M groups
         int my_rank = -1;
-        float pv = kPosInf;
-        int pi = -1;
-        for (int m = 0; m < M; ++m) {
-            float cv = kNegInf;
-            int ci = 0x7FFFFFFF;
-            if (real_group && after(score, gid, pv, pi)) {
-                cv = score;
-                ci = gid;
+        if constexpr (kGroupSlots <= 16) {
+            // few groups: every lane reads each group's score from that group's first lane and counts
+            // the groups ahead of its own; a NaN score is ahead of nothing and behind nothing
+            int ahead_of_me = 0;
+#pragma unroll
+            for (int G = 0; G < kGroupSlots; ++G) {
+                const float sg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(score), G * LPG));
+                const int ig = __builtin_amdgcn_readlane(gid, G * LPG);
+                ahead_of_me += ahead(sg, ig, score, gid) ? 1 : 0;
             }
-            best_range(cv, ci, lpg, kWave);
-            if (real_group && ci == gid) my_rank = m;
-            pv = cv;
-            pi = ci;
-            if (lane == 0) group_idx[t * M + m] = ci;
+            if (real_group && ahead_of_me < M && score == score) my_rank = ahead_of_me;
+            const bool files = (lane & (LPG - 1)) == 0 && my_rank >= 0;
+            if (files) group_idx[t * M + my_rank] = gid;
+            const int n_filed = __popcll(__ballot(files));
+            if (n_filed < M && lane >= n_filed && lane < M) group_idx[t * M + lane] = 0x7FFFFFFF;   // NaN scores only
+        } else {
+            float pv = kPosInf;
+            int pi = -1;
+            for (int m = 0; m < M; ++m) {
+                float cv = kNegInf;
+                int ci = 0x7FFFFFFF;
+                if (real_group && after(score, gid, pv, pi)) {
+                    cv = score;
+                    ci = gid;
+                }
+                best_range<LPG, kWave>(cv, ci);
+                if (real_group && ci == gid) my_rank = m;
+                pv = cv;
+                pi = ci;
+                if (lane == 0) group_idx[t * M + m] = ci;
+            }
         }
-        // every selected group picks its q experts, all groups at once
+        // every selected group picks its q experts, all groups at once; the owner lane of a pick
+        // files the id and its raw gate under the group's rank
         float ev = kPosInf;
         int ei = -1;
         for (int i = 0; i < q; ++i) {
@@ -195,13 +228,32 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
                     ci = e;
                 }
             }
-            best_range(cv, ci, 1, lpg);
+            best_range<1, LPG>(cv, ci);
             ev = cv;
             ei = ci;
-            if (group_head && my_rank >= 0) sel[my_rank * q + i] = ci;
+            if (my_rank >= 0 && (unsigned)(ci - lane * VPL) < (unsigned)VPL) {
+                float mine = ga[0];
+#pragma unroll
+                for (int x = 1; x < VPL; ++x)
+                    if (ci - lane * VPL == x) mine = ga[x];
+                sel[my_rank * q + i] = ci;
+                raw[my_rank * q + i] = mine;
+            }
         }
         __builtin_amdgcn_wave_barrier();
-        write_token(sel, raw, (gate_affinity ? gate_affinity : affinity) + t * E, k, E, t, expert_idx, gates);
+        // slots nobody filed (NaN scores are never picked): expert 0 and its gate
+        if (lane < k && ((volatile int *)sel)[lane] < 0) {
+            sel[lane] = 0;
+            raw[lane] = (gate_affinity ? gate_affinity : affinity)[t * E];
+        }
+        __builtin_amdgcn_wave_barrier();
+        float den = 0.0f;
+        for (int j = 0; j < k; ++j)
+            den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
+        if (lane < k) {
+            expert_idx[t * k + lane] = ((volatile int *)sel)[lane];
+            gates[t * k + lane] = __fdiv_rn(((volatile float *)raw)[lane], den);
+        }
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -371,19 +423,31 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
     while (vpl * kWave < E) vpl *= 2;
     const bool aligned = (((uintptr_t)affinity) & 15) == 0;
     if (!force_generic && mode == TERRACE_ROUTE_FULL && vpl <= 16 && g % vpl == 0 && is_pow2(g / vpl) &&
-        g / vpl <= kWave && (E != kWave * vpl || aligned)) {
+        g / vpl <= kWave && k <= kWave && (E != kWave * vpl || aligned) &&
+        (!gate_affinity || E != kWave * vpl || (((uintptr_t)gate_affinity) & 15) == 0)) {
         const int lpg = g / vpl;
         const size_t lds = (size_t)kWavesPerBlock * 2 * k * sizeof(int32_t);
-#define TERRACE_ROUTE(V)                                                                                      \
-    route_wave_kernel<V><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, g, k, M, pool, \
-                                                          lpg, expert_idx, gates, group_idx)
+#define TERRACE_ROUTE(V, L)                                                                                       \
+    route_wave_kernel<V, L><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, k, M, pool, \
+                                                             expert_idx, gates, group_idx)
+#define TERRACE_ROUTE_L(V)                          \
+    switch (lpg) {                                  \
+        case 1: TERRACE_ROUTE(V, 1); break;         \
+        case 2: TERRACE_ROUTE(V, 2); break;         \
+        case 4: TERRACE_ROUTE(V, 4); break;         \
+        case 8: TERRACE_ROUTE(V, 8); break;         \
+        case 16: TERRACE_ROUTE(V, 16); break;       \
+        case 32: TERRACE_ROUTE(V, 32); break;       \
+        default: TERRACE_ROUTE(V, 64); break;       \
+    }
         switch (vpl) {
-            case 1: TERRACE_ROUTE(1); break;
-            case 2: TERRACE_ROUTE(2); break;
-            case 4: TERRACE_ROUTE(4); break;
-            case 8: TERRACE_ROUTE(8); break;
-            default: TERRACE_ROUTE(16); break;
+            case 1: TERRACE_ROUTE_L(1); break;
+            case 2: TERRACE_ROUTE_L(2); break;
+            case 4: TERRACE_ROUTE_L(4); break;
+            case 8: TERRACE_ROUTE_L(8); break;
+            default: TERRACE_ROUTE_L(16); break;
         }
+#undef TERRACE_ROUTE_L
 #undef TERRACE_ROUTE
         return check_launch();
     }
