@@ -154,6 +154,20 @@ struct KeyRun {              // item = t*M + m  ->  node of the m-th run of toke
     }
 };
 
+// Lanes of the wave that hold the same key as this one (valid lanes only): one ballot per key bit
+// instead of one pass per distinct key.
+__device__ __forceinline__ uint64_t same_key_lanes(int key, bool valid, int key_bits) {
+    uint64_t peers = __ballot(valid);
+    for (int b = 0; b < key_bits; ++b) {
+        const bool bit = (key >> b) & 1;
+        const uint64_t set = __ballot(valid && bit);
+        peers &= bit ? set : ~set;
+    }
+    return peers;
+}
+
+__device__ __forceinline__ int bits_for(int n_buckets) { return n_buckets <= 1 ? 0 : 32 - __builtin_clz(n_buckets - 1); }
+
 // ---------------------------------------------------------------------------------------------
 // count: table is bucket-major, table[b * n_units + unit]
 // ---------------------------------------------------------------------------------------------
@@ -165,6 +179,7 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
     volatile int32_t *hist = lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
+    const int key_bits = bits_for(u.n_buckets);
     const int64_t first = (int64_t)unit * CH * kWave;
     int keys[CH];
 #pragma unroll
@@ -179,14 +194,9 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
     for (int c = 0; c < CH; ++c) {
         const int key = keys[c];
         const bool valid = key >= 0;
-        uint64_t todo = __ballot(valid);
-        while (todo) {
-            const int leader = __builtin_ctzll(todo);
-            const int kk = read_lane(key, leader);
-            const uint64_t peers = __ballot(key == kk);
-            if (lane == leader) hist[kk] = hist[kk] + __popcll(peers);
-            todo &= ~peers;
-        }
+        const uint64_t peers = same_key_lanes(key, valid, key_bits);
+        // the lowest lane of each key adds the key's count: distinct keys, distinct words
+        if (valid && lane == __builtin_ctzll(peers)) hist[key] = hist[key] + __popcll(peers);
         __builtin_amdgcn_wave_barrier();
     }
     for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)b * u.n_units + unit] = hist[b];
@@ -288,6 +298,7 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
     volatile int32_t *cursor = lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
+    const int key_bits = bits_for(u.n_buckets);
     const int64_t first = (int64_t)unit * CH * kWave;
     int fault = 0;
     int keys[CH];
@@ -308,17 +319,11 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
         const int key = keys[c];
         const bool valid = key >= 0;
         int32_t dest = 0;
-        uint64_t todo = __ballot(valid);
-        while (todo) {
-            const int leader = __builtin_ctzll(todo);
-            const int kk = read_lane(key, leader);
-            const uint64_t peers = __ballot(key == kk);
-            const int32_t base = cursor[kk];
-            if (key == kk) dest = base + __popcll(peers & lanes_below(lane));
-            __builtin_amdgcn_wave_barrier();
-            if (lane == leader) cursor[kk] = base + __popcll(peers);
-            todo &= ~peers;
-        }
+        const uint64_t peers = same_key_lanes(key, valid, key_bits);
+        const int32_t base = valid ? cursor[key] : 0;
+        if (valid) dest = base + __popcll(peers & lanes_below(lane));
+        __builtin_amdgcn_wave_barrier();
+        if (valid && lane == __builtin_ctzll(peers)) cursor[key] = base + __popcll(peers);
         __builtin_amdgcn_wave_barrier();
         if (valid) fault |= emit(item, key, dest, start, tally);
     }
