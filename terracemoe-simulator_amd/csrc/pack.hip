@@ -44,22 +44,19 @@ struct TokenRow {
     uint64_t occ;       // the lowest M of them: the ones that get a send row
     int fault;
     __device__ __forceinline__ void load(const int64_t *row, int k, int slots, int n_experts, int M) {
+        // the k ids first, as unconditional loads with nothing between them that waits on memory
+        int64_t v[KMAX];
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) v[j] = row[j < k ? j : 0];
         fault = 0;
         all = 0;
 #pragma unroll
         for (int j = 0; j < KMAX; ++j) {
-            e[j] = -1;
-            nd[j] = -1;
-            if (j < k) {
-                const int64_t v = row[j];
-                if (v >= 0 && v < n_experts) {
-                    e[j] = (int)v;
-                    nd[j] = (int)v / slots;
-                    all |= 1ull << nd[j];
-                } else {
-                    fault |= TERRACE_FAULT_ID_RANGE;
-                }
-            }
+            const bool ok = j < k && v[j] >= 0 && v[j] < n_experts;
+            e[j] = ok ? (int)v[j] : -1;
+            nd[j] = ok ? (int)v[j] / slots : -1;
+            if (ok) all |= 1ull << nd[j];
+            if (j < k && !ok) fault |= TERRACE_FAULT_ID_RANGE;
         }
         uint64_t rest = all;
         occ = 0;
@@ -130,6 +127,9 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
         TokenRow<KMAX> row;
         row.all = row.occ = 0;
         row.fault = 0;
+        G gate_of[KMAX];                  // the token's k gates: their loads go out ahead of the id loads
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) gate_of[j] = (live && gates) ? gates[t * k + (j < k ? j : 0)] : G(0);
         if (live) row.load(expert_idx + t * k, k, slots, n_experts, M);
         // ---- rank this chunk's (token, node) pairs, node by node ----
         int rows[KMAX];
@@ -212,14 +212,14 @@ __global__ __launch_bounds__(kBlock) void k2_place_kernel(
             const int64_t cell = (int64_t)r * quota + within;
             mask[(int64_t)r * mask_pitch + within] = ej - nj * slots;
             if (gates) {
-                gate_rows[(int64_t)r * gate_pitch + within] = gates[t * k + j];
+                gate_rows[(int64_t)r * gate_pitch + within] = gate_of[j];
                 if (within == 0)
                     for (int z = 0; z < gate_pad; ++z) gate_rows[(int64_t)r * gate_pitch + quota + z] = G(0);
             }
             if (inverse) inverse[t * k + j] = r;
             if (pair_table) pair_table[t * k + rank] = cell;
             if (sort_order) sort_order[t * k + rank] = j;
-            if (gates && gate_sorted) gate_sorted[t * k + rank] = gates[t * k + j];
+            if (gates && gate_sorted) gate_sorted[t * k + rank] = gate_of[j];
         }
     }
     // rows nobody claimed (possible only under a fan-out fault): zero them

@@ -49,18 +49,18 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
     // r*width + i is then at plane[r*pitch + i]
     int width = 1;
     int64_t pitch = 1;
-    __device__ __forceinline__ int64_t at(int64_t item) const {
-        if (pitch == width) return plane[item];
-        const int64_t r = item / width;
-        return plane[r * pitch + (item - r * width)];
+    // fetch() is one unconditional load (the kernels issue every chunk's fetch before any key is
+    // used, so the loads overlap); bucket() turns the fetched value into the key
+    __device__ __forceinline__ int64_t fetch(int64_t item) const {
+        const uint32_t r = (uint32_t)item / (uint32_t)width;            // items are below 2^31
+        const int64_t at = pitch == width ? item : (int64_t)r * pitch + (int64_t)((uint32_t)item - r * (uint32_t)width);
+        return plane[at];
     }
-    __device__ __forceinline__ int operator()(int64_t item, bool *bad) const {
-        const int64_t v = at(item) - sub;
-        if (v < 0 || v >= (int64_t)n_buckets * div) {
-            *bad = true;
-            return 0;
-        }
-        return (int)((uint32_t)v / (uint32_t)div);
+    __device__ __forceinline__ int bucket(int64_t, int64_t fetched, bool *bad) const {
+        const int64_t v = fetched - sub;
+        const bool out = v < 0 || v >= (int64_t)n_buckets * div;
+        if (out) *bad = true;
+        return out ? 0 : (int)((uint32_t)v / (uint32_t)div);
     }
 };
 
@@ -139,7 +139,8 @@ template <int KMAX>
 struct KeyRun {              // item = t*M + m  ->  node of the m-th run of token t's ascending row
     const int64_t *expert_idx;
     int k, groups_m, quota, slots, n_nodes;
-    __device__ __forceinline__ int operator()(int64_t item, bool *bad) const {
+    __device__ __forceinline__ int64_t fetch(int64_t) const { return 0; }
+    __device__ __forceinline__ int bucket(int64_t item, int64_t, bool *bad) const {
         const int64_t t = item / groups_m;
         const int m = (int)(item - t * groups_m);
         RowIds<KMAX> ids;
@@ -181,12 +182,19 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
     if (unit >= u.n_units) return;
     const int key_bits = bits_for(u.n_buckets);
     const int64_t first = (int64_t)unit * CH * kWave;
+    int64_t fetched[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {       // every chunk's load is issued before any key is computed
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        fetched[c] = key_of.fetch(item < u.n_items ? item : u.n_items - 1);
+    }
     int keys[CH];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {       // all chunks' keys are fetched before any is consumed
+    for (int c = 0; c < CH; ++c) {
         const int64_t item = first + (int64_t)c * kWave + lane;
         bool bad = false;
-        keys[c] = item < u.n_items ? key_of(item, &bad) : -1;
+        const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
+        keys[c] = item < u.n_items ? key : -1;
     }
     for (int b = lane; b < u.n_buckets; b += kWave) hist[b] = 0;
     __builtin_amdgcn_wave_barrier();
@@ -301,31 +309,47 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
     const int key_bits = bits_for(u.n_buckets);
     const int64_t first = (int64_t)unit * CH * kWave;
     int fault = 0;
+    // phase 1: every chunk's key load and the emitter's own input loads, all issued before any is used
+    int64_t fetched[CH];
+    typename EmitFn::Pre pre[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        const int64_t safe = item < u.n_items ? item : u.n_items - 1;
+        fetched[c] = key_of.fetch(safe);
+        pre[c] = emit.fetch(safe);
+    }
     int keys[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int64_t item = first + (int64_t)c * kWave + lane;
         bool bad = false;
-        keys[c] = item < u.n_items ? key_of(item, &bad) : -1;
-        if (bad) fault |= TERRACE_FAULT_ID_RANGE;
+        const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
+        keys[c] = item < u.n_items ? key : -1;
+        if (bad && item < u.n_items) fault |= TERRACE_FAULT_ID_RANGE;
     }
     for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)b * u.n_units + unit];
     __builtin_amdgcn_wave_barrier();
     const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
     int tally[2] = {0, 0};
+    // phase 2: places, in registers
+    int32_t dests[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const int64_t item = first + (int64_t)c * kWave + lane;
         const int key = keys[c];
         const bool valid = key >= 0;
-        int32_t dest = 0;
         const uint64_t peers = same_key_lanes(key, valid, key_bits);
         const int32_t base = valid ? cursor[key] : 0;
-        if (valid) dest = base + __popcll(peers & lanes_below(lane));
+        dests[c] = base + __popcll(peers & lanes_below(lane));
         __builtin_amdgcn_wave_barrier();
         if (valid && lane == __builtin_ctzll(peers)) cursor[key] = base + __popcll(peers);
         __builtin_amdgcn_wave_barrier();
-        if (valid) fault |= emit(item, key, dest, start, tally);
+    }
+    // phase 3: outputs
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int64_t item = first + (int64_t)c * kWave + lane;
+        if (keys[c] >= 0) fault |= emit(item, keys[c], dests[c], fetched[c], pre[c], start, tally);
     }
     if (!status) return;
     if (fault) atomicOr(&status[0], fault);
@@ -343,10 +367,17 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
 // ---------------------------------------------------------------------------------------------
 // emit functors
 // ---------------------------------------------------------------------------------------------
+// An emitter's fetch(item) loads what it needs beyond the key (issued with the key loads); its call
+// operator gets the key's fetched value and that Pre back and only computes and stores.
+struct NoPre {};
+
 struct EmitOrder {           // plain stable argsort: order[dest] = item
     int64_t *order;
     static constexpr bool kTallies = false;
-    __device__ __forceinline__ int operator()(int64_t item, int, int32_t dest, const int32_t *, int *) const {
+    typedef NoPre Pre;
+    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    __device__ __forceinline__ int operator()(int64_t item, int, int32_t dest, int64_t, Pre, const int32_t *,
+                                              int *) const {
         order[dest] = item;
         return 0;
     }
@@ -354,7 +385,11 @@ struct EmitOrder {           // plain stable argsort: order[dest] = item
 
 struct EmitNothing {
     static constexpr bool kTallies = false;
-    __device__ __forceinline__ int operator()(int64_t, int, int32_t, const int32_t *, int *) const { return 0; }
+    typedef NoPre Pre;
+    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    __device__ __forceinline__ int operator()(int64_t, int, int32_t, int64_t, Pre, const int32_t *, int *) const {
+        return 0;
+    }
 };
 
 struct EmitArrival {         // terrace/ops/__init__.py:287-299
@@ -367,24 +402,28 @@ struct EmitArrival {         // terrace/ops/__init__.py:287-299
     int32_t *pos32;
     int64_t *meta;           // Hop-B container [P, 2]: word 0 the slot id, word 1 the gate then zeros; or NULL
     static constexpr bool kTallies = false;
-    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, const int32_t *, int *) const {
-        const int64_t r = p / quota;
-        const int i = (int)(p - r * quota);
-        const int64_t slot = rslot[r * slot_pitch + i];
-        r_idx[dest] = r;
-        if (slot_idx) slot_idx[dest] = slot;
-        uint32_t gbits = 0;
+    struct Pre { uint32_t gbits; };
+    __device__ __forceinline__ Pre fetch(int64_t p) const {
+        Pre pre{0u};
         if (rgate) {
-            if (gate_bytes == 4) gbits = ((const uint32_t *)rgate)[r * gate_pitch + i];
-            else gbits = ((const uint16_t *)rgate)[r * gate_pitch + i];
-            if (gate_pairs) {
-                if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = gbits;
-                else ((uint16_t *)gate_pairs)[dest] = (uint16_t)gbits;
-            }
+            const uint32_t r = (uint32_t)p / (uint32_t)quota;
+            const int64_t at = (int64_t)r * gate_pitch + (int64_t)((uint32_t)p - r * (uint32_t)quota);
+            pre.gbits = gate_bytes == 4 ? ((const uint32_t *)rgate)[at] : (uint32_t)((const uint16_t *)rgate)[at];
+        }
+        return pre;
+    }
+    // `slot` is the value the key was computed from: rslot[r, i]
+    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, int64_t slot, Pre pre, const int32_t *,
+                                              int *) const {
+        r_idx[dest] = (int64_t)((uint32_t)p / (uint32_t)quota);
+        if (slot_idx) slot_idx[dest] = slot;
+        if (rgate && gate_pairs) {
+            if (gate_bytes == 4) ((uint32_t *)gate_pairs)[dest] = pre.gbits;
+            else ((uint16_t *)gate_pairs)[dest] = (uint16_t)pre.gbits;
         }
         if (meta) {
             meta[2 * (int64_t)dest] = slot;
-            meta[2 * (int64_t)dest + 1] = (int64_t)(uint64_t)gbits;
+            meta[2 * (int64_t)dest + 1] = (int64_t)(uint64_t)pre.gbits;
         }
         pos32[p] = dest;
         if (pair_pos) pair_pos[p] = dest;
@@ -401,8 +440,11 @@ struct EmitPairs {           // terrace/ta2a_fwd.py:605-628, general branch: pai
     int64_t *r_idx, *slot_idx, *ordo;
     int32_t *src32;          // source row of each output place (-1: row id out of range)
     static constexpr bool kTallies = false;
-    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, const int32_t *, int *) const {
-        const int64_t r = r_in[p], sl = slot_in[p];
+    struct Pre { int64_t r; };
+    __device__ __forceinline__ Pre fetch(int64_t p) const { return Pre{r_in[p]}; }
+    __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, int64_t sl, Pre pre, const int32_t *,
+                                              int *) const {
+        const int64_t r = pre.r;
         const bool ok = r >= 0 && r < R;
         r_idx[dest] = r;
         slot_idx[dest] = sl;
@@ -424,7 +466,10 @@ struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
     uint8_t *kept;
     int32_t *order32;
     static constexpr bool kTallies = false;
-    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, const int32_t *start, int *) const {
+    typedef NoPre Pre;
+    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre, const int32_t *start,
+                                              int *) const {
         order32[dest] = (int32_t)p;
         if (order) order[dest] = p;
         if (capacity >= 0) {
@@ -453,7 +498,9 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
     // status word 1 receives the number of occupied (token, node) pairs, word 2 the number of
     // those holding other than k/M experts: the two quantities terrace/ta2a.py:170-204 checks.
     static constexpr bool kTallies = true;
-    __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, const int32_t *,
+    typedef NoPre Pre;
+    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, int64_t, Pre, const int32_t *,
                                               int *tally) const {
         const int64_t t = item / groups_m;
         const int m = (int)(item - t * groups_m);
