@@ -1,14 +1,16 @@
-// T-Route: group-limited top-k with equal per-group quota, one wavefront per token.
+// T-Route: group-limited top-k with equal per-group quota, a token's scores spread over the lanes of
+// a wavefront.
 //
 // Selection order everywhere is the strict total order (value descending, index ascending):
 // "the next pick" is the largest candidate strictly after the previous pick in that order, so
 // no taken-flags are needed and ties always go to the lowest index.
 //
-//   route_wave_kernel     mode "full" when the E (padded) scores map onto the wave as VPL
-//                         consecutive values per lane and every group covers a power-of-two
-//                         number of whole lanes.  Scores never leave registers: group top-2 by a
-//                         DPP butterfly inside the group's lanes, top-M groups by a butterfly
-//                         across groups, then all M selected groups pick their q experts at once.
+//   route_wave_kernel     mode "full" when a token's E (padded) scores map onto 8..64 lanes as VPL
+//                         consecutive values per lane and every group covers a power-of-two number
+//                         of whole lanes; up to 8 tokens share a wave.  Scores never leave
+//                         registers: group top-2 by a DPP butterfly inside the group's lanes, top-M
+//                         groups by rank counting (or a butterfly across groups), then all M
+//                         selected groups pick their q experts at once.
 //   route_generic_kernel  every mode and every geometry; scores staged in wave-private LDS.
 //
 // Both write expert_idx / group_idx as int64 and gates = raw / (raw_0 + raw_1 + ... ) with the
@@ -102,10 +104,13 @@ __device__ __forceinline__ void write_token(int *sel, float *raw, const float *g
 // ---------------------------------------------------------------------------------------------
 // register-resident kernel, mode "full"
 // ---------------------------------------------------------------------------------------------
-// VPL consecutive scores per lane, LPG lanes per group (g = VPL*LPG), 64/LPG group positions per wave.
-// The token's row of gate values sits in registers beside its scores, so the lane that owns a chosen
-// expert hands over the raw gate itself and nothing is re-read from memory after the selection.
-template <int VPL, int LPG>
+// A wave holds TPW tokens side by side: LPT = 64/TPW lanes per token, VPL consecutive scores per lane,
+// LPG lanes per group (g = VPL*LPG), LPT/LPG group positions per token, so short rows (E = 64, 128)
+// fill the wave with 4 or 2 tokens instead of leaving lanes idle.  The kernel is bound by its vector
+// instruction count (about 330 per token at E = 256, k = 8), not by the row it reads.  The token's row of gate values sits in registers beside its scores, so
+// the lane that owns a chosen expert hands over the raw gate itself and nothing is re-read from memory
+// after the selection.
+template <int VPL, int LPG, int TPW>
 __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restrict__ affinity,
                                                             const float *__restrict__ bias,
                                                             const float *__restrict__ gate_affinity, int64_t T, int E,
@@ -114,34 +119,39 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
                                                             float *__restrict__ gates,
                                                             int64_t *__restrict__ group_idx) {
     extern __shared__ int32_t lds[];
+    constexpr int LPT = kWave / TPW;
     constexpr int g = VPL * LPG;
-    constexpr int kGroupSlots = kWave / LPG;
+    constexpr int kGroupSlots = LPT / LPG;
+    static_assert(LPG <= LPT, "a group cannot span more lanes than a token has");
     const int lane = lane_id();
     const int w = wave_in_block();
-    int *sel = lds + w * 2 * k;
+    const int tl = lane & (LPT - 1);             // lane within the token
+    const int slot = lane / LPT;                 // which of the wave's tokens
+    const int lane0 = lane - tl;                 // the token's first lane
+    int *sel = lds + (w * TPW + slot) * 2 * k;   // per token: k chosen ids, then their k raw gates
     float *raw = (float *)(sel + k);
     const int q = k / M;
-    const int my_group = lane / LPG;
+    const int my_group = tl / LPG;
     float b[VPL];
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
-        const int e = lane * VPL + i;
+        const int e = tl * VPL + i;
         b[i] = e < E ? bias[e] : 0.0f;
     }
-    auto load_row = [&](const float *row, float *v, float fill) {
-        if (E == kWave * VPL) {
+    auto load_row = [&](const float *row, float *v) {
+        if (E == LPT * VPL) {
             if constexpr (VPL == 1) {
-                v[0] = row[lane];
+                v[0] = row[tl];
             } else if constexpr (VPL <= 4) {
                 typedef float fvec __attribute__((ext_vector_type(VPL)));
-                const fvec x = *(const fvec *)(row + lane * VPL);
+                const fvec x = *(const fvec *)(row + tl * VPL);
 #pragma unroll
                 for (int i = 0; i < VPL; ++i) v[i] = x[i];
             } else {
                 typedef float f4 __attribute__((ext_vector_type(4)));
 #pragma unroll
                 for (int c = 0; c < VPL / 4; ++c) {
-                    const f4 x = *(const f4 *)(row + lane * VPL + 4 * c);
+                    const f4 x = *(const f4 *)(row + tl * VPL + 4 * c);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) v[4 * c + i] = x[i];
                 }
@@ -149,22 +159,35 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
         } else {
 #pragma unroll
             for (int i = 0; i < VPL; ++i) {
-                const int e = lane * VPL + i;
-                v[i] = e < E ? row[e] : fill;
+                const int e = tl * VPL + i;
+                v[i] = e < E ? row[e] : 0.0f;
             }
         }
     };
-    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += (int64_t)gridDim.x * kWavesPerBlock) {
+    // value held by lane `src` of this token's lanes
+    auto from_lane_f = [&](float v, int src) {
+        if constexpr (TPW == 1) return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src));
+        else return __shfl(v, lane0 + src, kWave);
+    };
+    auto from_lane_i = [&](int v, int src) {
+        if constexpr (TPW == 1) return __builtin_amdgcn_readlane(v, src);
+        else return __shfl(v, lane0 + src, kWave);
+    };
+    const int64_t stride = (int64_t)gridDim.x * kWavesPerBlock * TPW;
+    for (int64_t t0 = ((int64_t)blockIdx.x * kWavesPerBlock + w) * TPW; t0 < T; t0 += stride) {
+        const int64_t t = t0 + slot;
+        const bool live = t < T;
+        const int64_t tt = live ? t : T - 1;     // a dead slot recomputes the last token and stores nothing
         float a[VPL], ga[VPL], s[VPL];
-        load_row(affinity + t * E, a, 0.0f);
-        if (gate_affinity) load_row(gate_affinity + t * E, ga, 0.0f);
+        load_row(affinity + tt * E, a);
+        if (gate_affinity) load_row(gate_affinity + tt * E, ga);
 #pragma unroll
         for (int i = 0; i < VPL; ++i) {
-            const int e = lane * VPL + i;
+            const int e = tl * VPL + i;
             s[i] = e < E ? __fadd_rn(a[i], b[i]) : kNegInf;
             if (!gate_affinity) ga[i] = a[i];
         }
-        if (lane < k) sel[lane] = -1;
+        if (tl < k) sel[tl] = -1;
         __builtin_amdgcn_wave_barrier();
         // group score: mean of the top two (or the top one) of the group's g values
         float a1 = kNegInf, a2 = kNegInf;
@@ -187,15 +210,17 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             int ahead_of_me = 0;
 #pragma unroll
             for (int G = 0; G < kGroupSlots; ++G) {
-                const float sg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(score), G * LPG));
-                const int ig = __builtin_amdgcn_readlane(gid, G * LPG);
+                const float sg = from_lane_f(score, G * LPG);
+                const int ig = from_lane_i(gid, G * LPG);
                 ahead_of_me += ahead(sg, ig, score, gid) ? 1 : 0;
             }
             if (real_group && ahead_of_me < M && score == score) my_rank = ahead_of_me;
-            const bool files = (lane & (LPG - 1)) == 0 && my_rank >= 0;
-            if (files) group_idx[t * M + my_rank] = gid;
-            const int n_filed = __popcll(__ballot(files));
-            if (n_filed < M && lane >= n_filed && lane < M) group_idx[t * M + lane] = 0x7FFFFFFF;   // NaN scores only
+            const bool files = (tl & (LPG - 1)) == 0 && my_rank >= 0;
+            if (files && live) group_idx[t * M + my_rank] = gid;
+            uint64_t filed = __ballot(files) >> lane0;
+            if constexpr (LPT < kWave) filed &= (1ull << LPT) - 1ull;
+            const int n_filed = __popcll(filed);
+            if (n_filed < M && tl >= n_filed && tl < M && live) group_idx[t * M + tl] = 0x7FFFFFFF;   // NaN scores only
         } else {
             float pv = kPosInf;
             int pi = -1;
@@ -206,11 +231,11 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
                     cv = score;
                     ci = gid;
                 }
-                best_range<LPG, kWave>(cv, ci);
+                best_range<LPG, LPT>(cv, ci);
                 if (real_group && ci == gid) my_rank = m;
                 pv = cv;
                 pi = ci;
-                if (lane == 0) group_idx[t * M + m] = ci;
+                if (tl == 0 && live) group_idx[t * M + m] = ci;
             }
         }
         // every selected group picks its q experts, all groups at once; the owner lane of a pick
@@ -222,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             int ci = 0x7FFFFFFF;
 #pragma unroll
             for (int x = 0; x < VPL; ++x) {
-                const int e = lane * VPL + x;
+                const int e = tl * VPL + x;
                 if (e < E && after(s[x], e, ev, ei) && ahead(s[x], e, cv, ci)) {
                     cv = s[x];
                     ci = e;
@@ -231,28 +256,28 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             best_range<1, LPG>(cv, ci);
             ev = cv;
             ei = ci;
-            if (my_rank >= 0 && (unsigned)(ci - lane * VPL) < (unsigned)VPL) {
+            if (my_rank >= 0 && (unsigned)(ci - tl * VPL) < (unsigned)VPL) {
                 float mine = ga[0];
 #pragma unroll
                 for (int x = 1; x < VPL; ++x)
-                    if (ci - lane * VPL == x) mine = ga[x];
+                    if (ci - tl * VPL == x) mine = ga[x];
                 sel[my_rank * q + i] = ci;
                 raw[my_rank * q + i] = mine;
             }
         }
         __builtin_amdgcn_wave_barrier();
         // slots nobody filed (NaN scores are never picked): expert 0 and its gate
-        if (lane < k && ((volatile int *)sel)[lane] < 0) {
-            sel[lane] = 0;
-            raw[lane] = (gate_affinity ? gate_affinity : affinity)[t * E];
+        if (tl < k && ((volatile int *)sel)[tl] < 0) {
+            sel[tl] = 0;
+            raw[tl] = (gate_affinity ? gate_affinity : affinity)[tt * E];
         }
         __builtin_amdgcn_wave_barrier();
         float den = 0.0f;
         for (int j = 0; j < k; ++j)
             den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
-        if (lane < k) {
-            expert_idx[t * k + lane] = ((volatile int *)sel)[lane];
-            gates[t * k + lane] = __fdiv_rn(((volatile float *)raw)[lane], den);
+        if (tl < k && live) {
+            expert_idx[t * k + tl] = ((volatile int *)sel)[tl];
+            gates[t * k + tl] = __fdiv_rn(((volatile float *)raw)[tl], den);
         }
         __builtin_amdgcn_wave_barrier();
     }
@@ -417,40 +442,60 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
         return TERRACE_EINVAL;
     if (T == 0) return TERRACE_OK;
     if (!affinity || !bias || !expert_idx || !gates || !group_idx) return TERRACE_EINVAL;
-    int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;      // one token per wave
-    if (blocks > ((int64_t)1 << 24)) blocks = (int64_t)1 << 24;
-    int vpl = 1;
-    while (vpl * kWave < E) vpl *= 2;
-    const bool aligned = (((uintptr_t)affinity) & 15) == 0;
-    if (!force_generic && mode == TERRACE_ROUTE_FULL && vpl <= 16 && g % vpl == 0 && is_pow2(g / vpl) &&
-        g / vpl <= kWave && k <= kWave && (E != kWave * vpl || aligned) &&
-        (!gate_affinity || E != kWave * vpl || (((uintptr_t)gate_affinity) & 15) == 0)) {
-        const int lpg = g / vpl;
-        const size_t lds = (size_t)kWavesPerBlock * 2 * k * sizeof(int32_t);
-#define TERRACE_ROUTE(V, L)                                                                                       \
-    route_wave_kernel<V, L><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, k, M, pool, \
-                                                             expert_idx, gates, group_idx)
-#define TERRACE_ROUTE_L(V)                          \
-    switch (lpg) {                                  \
-        case 1: TERRACE_ROUTE(V, 1); break;         \
-        case 2: TERRACE_ROUTE(V, 2); break;         \
-        case 4: TERRACE_ROUTE(V, 4); break;         \
-        case 8: TERRACE_ROUTE(V, 8); break;         \
-        case 16: TERRACE_ROUTE(V, 16); break;       \
-        case 32: TERRACE_ROUTE(V, 32); break;       \
-        default: TERRACE_ROUTE(V, 64); break;       \
+    // Register-resident form.  VPL = 4 (one 16-byte load per lane) measured best wherever it fits
+    // (E = 256: 14.2 us for 16384 tokens against 16.0 at VPL 8 and 16.6 at VPL 16); smaller VPL serve
+    // groups of fewer than 4 experts, larger ones rows too long for 64 lanes of 4.  VPL must divide g
+    // into a power-of-two number of lanes and leave the token k lanes for its outputs.
+    const bool aligned = (((uintptr_t)affinity) & 15) == 0 && (!gate_affinity || (((uintptr_t)gate_affinity) & 15) == 0);
+    if (!force_generic && mode == TERRACE_ROUTE_FULL) {
+        static const int kVplOrder[] = {4, 2, 1, 8, 16};
+        for (int vpl : kVplOrder) {
+            if (g % vpl || !is_pow2(g / vpl)) continue;
+            const int lpg = g / vpl;
+            int lpt = 8;                                     // at most 8 tokens share a wave
+            while (lpt < lpg || lpt * vpl < E || lpt < k) lpt *= 2;
+            if (lpt > kWave) continue;
+            if (E == lpt * vpl && vpl > 1 && !aligned) continue;     // vector loads need 16-byte rows
+            const int tpw = kWave / lpt;
+            const int64_t waves = (T + tpw - 1) / tpw;
+            int64_t blocks = (waves + kWavesPerBlock - 1) / kWavesPerBlock;
+            if (blocks > ((int64_t)1 << 24)) blocks = (int64_t)1 << 24;
+            const size_t lds = (size_t)kWavesPerBlock * tpw * 2 * k * sizeof(int32_t);
+#define TERRACE_ROUTE(V, L, W)                                                                                  \
+    route_wave_kernel<V, L, W><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, k, M, pool, \
+                                                                expert_idx, gates, group_idx)
+#define TERRACE_ROUTE_W(V, L)                                \
+    switch (tpw) {                                           \
+        case 1: TERRACE_ROUTE(V, L, 1); break;               \
+        case 2: if constexpr (L <= 32) TERRACE_ROUTE(V, L, 2); break; \
+        case 4: if constexpr (L <= 16) TERRACE_ROUTE(V, L, 4); break; \
+        default: if constexpr (L <= 8) TERRACE_ROUTE(V, L, 8); break; \
     }
-        switch (vpl) {
-            case 1: TERRACE_ROUTE_L(1); break;
-            case 2: TERRACE_ROUTE_L(2); break;
-            case 4: TERRACE_ROUTE_L(4); break;
-            case 8: TERRACE_ROUTE_L(8); break;
-            default: TERRACE_ROUTE_L(16); break;
-        }
+#define TERRACE_ROUTE_L(V)                              \
+    switch (lpg) {                                      \
+        case 1: TERRACE_ROUTE_W(V, 1); break;           \
+        case 2: TERRACE_ROUTE_W(V, 2); break;           \
+        case 4: TERRACE_ROUTE_W(V, 4); break;           \
+        case 8: TERRACE_ROUTE_W(V, 8); break;           \
+        case 16: TERRACE_ROUTE_W(V, 16); break;         \
+        case 32: TERRACE_ROUTE_W(V, 32); break;         \
+        default: TERRACE_ROUTE_W(V, 64); break;         \
+    }
+            switch (vpl) {
+                case 16: TERRACE_ROUTE_L(16); break;
+                case 8: TERRACE_ROUTE_L(8); break;
+                case 4: TERRACE_ROUTE_L(4); break;
+                case 2: TERRACE_ROUTE_L(2); break;
+                default: TERRACE_ROUTE_L(1); break;
+            }
 #undef TERRACE_ROUTE_L
+#undef TERRACE_ROUTE_W
 #undef TERRACE_ROUTE
-        return check_launch();
+            return check_launch();
+        }
     }
+    int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;      // generic form: one token per wave
+    if (blocks > ((int64_t)1 << 24)) blocks = (int64_t)1 << 24;
     const int n_group_out = mode == TERRACE_ROUTE_QUOTA_ONLY ? n_groups : (mode == TERRACE_ROUTE_GLOBAL_TOPK ? k : M);
     const size_t lds = (size_t)kWavesPerBlock * (E + 2 * n_groups + 2 * k) * sizeof(int32_t);
     route_generic_kernel<<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, n_groups, k, M, pool,
