@@ -486,3 +486,30 @@ def test_hopa_send_splits_literal(literals):
     lit = literals["hopa_counts"]
     send = orc.hopa_send_splits(lit["node_counts"], lit["world"], lit["rpn"], lit["my_local"])
     assert send.tolist() == lit["send"] and send.dtype == np.int64
+
+
+@pytest.mark.parametrize("E,Ng,k,M", [(64, 8, 4, 2), (256, 8, 8, 4), (128, 16, 8, 2), (32, 4, 2, 1), (96, 8, 6, 3), (256, 8, 16, 4)])
+def test_route_gates_against_the_library_composition(E, Ng, k, M):
+    """gates = affinity.gather(1, expert_idx) / gates.sum(-1) as the reference writes it
+    (terrace/routing.py:94-95), evaluated by the installed torch on the CPU.  The library's reduction
+    order inside sum(-1) is its own affair: for k = 2, 4 and 8 (every benchmark geometry) it gives the
+    bits of the decreed left-to-right sum, for other k the two may differ in the last place."""
+    g = torch.Generator().manual_seed(E + k)
+    aff = torch.rand(4096, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.1
+    e, gates, _ = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M)
+    raw = aff.gather(1, torch.from_numpy(e))
+    lib = (raw / raw.sum(-1, keepdim=True)).numpy()
+    if k in (2, 4, 8):
+        assert np.array_equal(gates, lib)
+    else:
+        ulp = np.spacing(np.abs(lib).astype(np.float32))
+        assert np.all(np.abs(gates - lib) <= 4 * ulp)
+    # and the selection itself is the library's on untied inputs: top-M groups by mean of top-2, top-q inside
+    s = aff + bias
+    sg = s.view(-1, Ng, E // Ng)
+    score = sg.topk(min(2, E // Ng), dim=-1).values.mean(-1)
+    grp = score.topk(M, dim=-1).indices
+    local = sg.gather(1, grp[:, :, None].expand(-1, -1, E // Ng)).topk(k // M, dim=-1).indices
+    want = (grp[:, :, None] * (E // Ng) + local).reshape(-1, k)
+    assert np.array_equal(e, want.numpy())
