@@ -503,8 +503,7 @@ def test_route_gates_against_the_library_composition(E, Ng, k, M):
     if k in (2, 4, 8):
         assert np.array_equal(gates, lib)
     else:
-        ulp = np.spacing(np.abs(lib).astype(np.float32))
-        assert np.all(np.abs(gates - lib) <= 4 * ulp)
+        assert np.all(np.abs(gates - lib) <= 1e-6 * np.abs(lib))
     # and the selection itself is the library's on untied inputs: top-M groups by mean of top-2, top-q inside
     s = aff + bias
     sg = s.view(-1, Ng, E // Ng)
