@@ -16,7 +16,6 @@
 namespace terrace {
 
 // ---- general plan --------------------------------------------------------------------------------
-template <int KMAX>
 __global__ __launch_bounds__(kBlock) void plan_count_kernel(const int64_t *__restrict__ expert_idx, int64_t T, int k,
                                                             int slots, int n_nodes, int n_experts, int n_units,
                                                             int32_t *__restrict__ table) {
@@ -100,7 +99,7 @@ int run_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int
     int32_t *table = (int32_t *)ws;
     const int blocks = (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock;
     if (T > 0 && (!expert_idx || !u_src || !u_node || !inverse)) return TERRACE_EINVAL;
-    plan_count_kernel<0><<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, u.n_units, table);
+    plan_count_kernel<<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, u.n_units, table);
     launch_scan(u, table, counts, nullptr, nullptr, status, s);
     plan_place_kernel<<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, u.n_units, table, u_src,
                                                 u_node, inverse, status);
