@@ -117,6 +117,21 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict
     }
 }
 
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has an L2 of its own.
+// Where neighbouring chunks of a row share cache lines (rows that are not whole 128-byte lines, or fp8
+// rows whose block scales sit in one line), the `run` chunks of a row are therefore given ids that are
+// 8 apart, so one XCD fetches the shared lines once.  Ids are taken in blocks of 8*run: linear id
+// y*8 + x inside a block works on logical chunk x*run + y; a ragged last block keeps its order.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ uint32_t xcd_swizzle(uint32_t id, uint32_t run, uint32_t total) {
+    if (run == 0) return id;
+    const uint32_t block = kXcds * run;
+    const uint32_t base = id / block * block;
+    if (base + block > total) return id;
+    const uint32_t in = id - base;
+    return base + (in % kXcds) * run + in / kXcds;
+}
+
 // Sliced forms for 16-byte vectors: a workgroup is one wave, every lane moves exactly one vector, and
 // each wave's store covers one 1 KB-aligned kilobyte of the destination.  Many one-wave workgroups
 // keep loads and stores of different rows interleaved in the memory pipeline, which streams
@@ -130,8 +145,9 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict
 template <typename I>
 __global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ out,
                                                                  const I *__restrict__ idx, int64_t total_vecs,
-                                                                 int64_t row_vecs, int head) {
-    const int64_t first = (int64_t)blockIdx.x * kWave - head;            // wave-uniform, may be < 0 in block 0
+                                                                 int64_t row_vecs, int head, uint32_t run) {
+    const uint32_t chunk = xcd_swizzle(blockIdx.x, run, gridDim.x);
+    const int64_t first = (int64_t)chunk * kWave - head;                 // wave-uniform, may be < 0 in chunk 0
     const int64_t g = first + threadIdx.x;
     if (g < 0 || g >= total_vecs) return;
     int64_t row, i;
@@ -191,8 +207,9 @@ __global__ __launch_bounds__(kWave) void scatter_rows_aligned_kernel(const u32x4
                                                                      u32x4 *__restrict__ dst, const I *__restrict__ pos,
                                                                      int fan, int64_t row_vecs, uint32_t chunks,
                                                                      int head) {
-    const uint32_t row = blockIdx.x / chunks;
-    const int64_t c = blockIdx.x - row * chunks;
+    const uint32_t id = xcd_swizzle(blockIdx.x, chunks, gridDim.x);     // a row's chunks re-read each other's lines
+    const uint32_t row = id / chunks;
+    const int64_t c = id - row * chunks;
     const u32x4 *s = src + (int64_t)row * row_vecs;
     const I *p = pos + (int64_t)row * fan;
     for (int f = 0; f < fan; ++f) {
@@ -386,10 +403,11 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restri
                                                          const int64_t *__restrict__ idx, const void *__restrict__ w,
                                                          int w_dtype, int64_t n_out, int fan, int64_t hidden,
                                                          uint8_t *__restrict__ out, int64_t out_row_bytes,
-                                                         int slices) {
+                                                         int slices, uint32_t run) {
     constexpr int N = Chunk<SRC>::N;
-    const int64_t row = blockIdx.x / slices;
-    const int64_t c = (int64_t)(blockIdx.x - row * slices) * blockDim.x + threadIdx.x;
+    const uint32_t id = xcd_swizzle(blockIdx.x, run, gridDim.x);
+    const int64_t row = id / slices;
+    const int64_t c = (int64_t)(id - row * slices) * blockDim.x + threadIdx.x;
     if (c >= hidden / N) return;
     const int64_t *idx_row = idx + row * fan;
     uint8_t *out_row = out + row * out_row_bytes;
@@ -634,8 +652,10 @@ static bool launch_gather_sliced(const void *src, void *out, const I *idx, int64
                                                                        (uint32_t)(row_vecs / kWave));
         return true;
     }
+    // rows that are not whole lines: a row's chunks share lines on the source side
+    const uint32_t run = (row_vecs % 8) ? (uint32_t)((row_vecs + kWave - 1) / kWave) : 0u;
     gather_rows_flat_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, total, row_vecs,
-                                                                 head);
+                                                                 head, run);
     return true;
 }
 
@@ -680,8 +700,10 @@ static void launch_combine_so(const void *src, const int64_t *idx, const void *w
     const int bt = one_wave ? kWave : kBlock;
     const int slices = (int)((chunks + bt - 1) / bt);
     const unsigned grid = (unsigned)(n_out * slices);
+    // source rows that are not whole lines (and fp8 rows, whose scales share a line): one XCD per output row
+    const uint32_t run = (srb % 128 || SRC == TERRACE_FP8_E4M3_B128) && slices > 1 ? (uint32_t)slices : 0u;
     combine_kernel<SRC, OUT><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, fan, hidden,
-                                                 (uint8_t *)out, orb, slices);
+                                                 (uint8_t *)out, orb, slices, run);
 }
 
 template <int SRC>
