@@ -20,11 +20,16 @@ Units make_units(int64_t n_items, int n_buckets) {
     Units u;
     u.n_items = n_items;
     u.n_buckets = n_buckets;
-    // the smallest unit (most waves) whose count table stays within 16K entries
+    // Unit size: a chunk more per wave costs the count and rank passes about 1 us, a count table four
+    // times larger costs the one-workgroup scan about 6 us (16K entries 5.5 us, 64K entries 12 us).
+    // So one chunk per wave while the table stays within 16K entries, four while it stays within 64K,
+    // sixteen beyond.
     u.chunks = 16;
-    for (int ch : {1, 4}) {
-        if ((n_items + 64 * ch - 1) / (64 * ch) * n_buckets <= 16384) {
-            u.chunks = ch;
+    const int64_t limit[] = {16384, 65536};
+    const int choice[] = {1, 4};
+    for (int i = 0; i < 2; ++i) {
+        if ((n_items + 64 * choice[i] - 1) / (64 * choice[i]) * n_buckets <= limit[i]) {
+            u.chunks = choice[i];
             break;
         }
     }
@@ -288,9 +293,91 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__
     }
 }
 
+// Tables of up to 64K entries (every geometry make_units produces unless the bucket count itself is
+// huge): the same walk as scan_kernel -- each of the 16 waves owns a contiguous span and covers it 256
+// entries (one coalesced kilobyte) at a time -- but a wave first takes its whole span into registers,
+// all loads issued at once, and scans it there: one memory round trip in, one out.
+constexpr int kScanRegVecs = 16;                 // 16 x 256 entries per wave
+
+__global__ __launch_bounds__(kScanThreads) void scan_registers_kernel(Units u, int32_t *__restrict__ table,
+                                                                      int64_t *__restrict__ hist_i64,
+                                                                      float *__restrict__ hist_f32,
+                                                                      int64_t *__restrict__ offsets_i64,
+                                                                      int32_t *__restrict__ status) {
+    constexpr int kWaves = kScanThreads / kWave;
+    __shared__ int32_t wave_tot[kWaves];
+    __shared__ int32_t grand_total;
+    const int tid = threadIdx.x, lane = lane_id(), w = tid >> 6;
+    const int64_t n = (int64_t)u.n_units * u.n_buckets;
+    int32_t *start = table + n;
+    if (status && tid < TERRACE_STATUS_WORDS) status[tid] = 0;
+    const int64_t span = ((n + kWaves - 1) / kWaves + 255) / 256 * 256;            // <= kScanRegVecs * 256
+    const int64_t lo = w * span, hi = lo + span < n ? lo + span : n;
+    i32x4 v[kScanRegVecs];
+    int32_t s4[kScanRegVecs];
+#pragma unroll
+    for (int c = 0; c < kScanRegVecs; ++c) {
+        const int64_t i = lo + c * 256 + lane * 4;
+        v[c] = i32x4{0, 0, 0, 0};
+        if (lo + c * 256 < hi) v[c] = load4_guarded(table, i, hi);
+    }
+    int32_t sum = 0;
+#pragma unroll
+    for (int c = 0; c < kScanRegVecs; ++c) {
+        s4[c] = v[c][0] + v[c][1] + v[c][2] + v[c][3];
+        sum += s4[c];
+    }
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+    if (lane == 0) wave_tot[w] = sum;
+    __syncthreads();
+    if (tid < kWave) {
+        const int32_t t = tid < kWaves ? wave_tot[tid] : 0;
+        const int32_t ti = wave_inclusive_scan(t);
+        if (tid < kWaves) wave_tot[tid] = ti - t;
+        if (tid == kWaves - 1) grand_total = ti;
+    }
+    __syncthreads();
+    int32_t carry = wave_tot[w];
+#pragma unroll
+    for (int c = 0; c < kScanRegVecs; ++c) {
+        if (lo + c * 256 < hi) {                                                  // wave-uniform
+            const int64_t i = lo + c * 256 + lane * 4;
+            const int32_t incl = wave_inclusive_scan(s4[c]);
+            i32x4 o;
+            o[0] = carry + incl - s4[c];
+            o[1] = o[0] + v[c][0];
+            o[2] = o[1] + v[c][1];
+            o[3] = o[2] + v[c][2];
+            if (i + 3 < hi) {
+                *(i32x4 *)(table + i) = o;
+            } else {
+                if (i < hi) table[i] = o[0];
+                if (i + 1 < hi) table[i + 1] = o[1];
+                if (i + 2 < hi) table[i + 2] = o[2];
+            }
+            carry += __shfl(incl, kWave - 1, kWave);
+        }
+    }
+    __syncthreads();
+    for (int b = tid; b <= u.n_buckets; b += kScanThreads) {
+        const int32_t s0 = b < u.n_buckets ? table[(int64_t)b * u.n_units] : grand_total;
+        start[b] = s0;
+        if (b == u.n_buckets) break;
+        const int32_t s1 = b + 1 < u.n_buckets ? table[(int64_t)(b + 1) * u.n_units] : grand_total;
+        if (hist_i64) hist_i64[b] = s1 - s0;
+        if (hist_f32) hist_f32[b] = (float)(s1 - s0);
+        if (offsets_i64) offsets_i64[b] = s0;
+    }
+}
+
 void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
                  int32_t *status, hipStream_t s) {
-    scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
+    const int64_t n = (int64_t)u.n_units * u.n_buckets;
+    if (n <= (int64_t)kScanThreads * kScanRegVecs * 4)
+        scan_registers_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
+    else
+        scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
 }
 
 // ---------------------------------------------------------------------------------------------
