@@ -213,6 +213,25 @@ TERRACE_API int terrace_unpack_planes(const void *packed, int64_t row_bytes, int
                                       int64_t a_bytes, void *b, int64_t b_bytes, void *c, int64_t c_bytes,
                                       terrace_stream_t stream);
 
+/* ---- the stage operators in two phases: index planes first, rows later ----
+ * The reference ships counts and metadata ahead of the payload so that the receiving side's index work
+ * overlaps the row traffic (terrace/ta2a_dispatch.py:78-100 and :399-412, the "async counts" path).  Here:
+ * terrace_k2_pack with hidden == NULL and payload == NULL, terrace_k1_arrival[_wire] with rx == NULL and
+ * send_buf == NULL, and terrace_regroup[_wire] with node_rx == NULL and permuted == NULL write every index
+ * plane and leave the row mover's int32 position plane in the workspace.  The *_move call below then moves
+ * the rows -- on any stream that is ordered after the first phase -- reading that plane; its geometry
+ * arguments must repeat the first phase's and the workspace must be the same untouched buffer.
+ * n_nodes = world / rpn.  terrace_regroup_move also writes the zero padding rows of a capacity layout. */
+TERRACE_API int terrace_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, int n_nodes,
+                                     int groups_m, void *payload, const void *workspace, size_t workspace_bytes,
+                                     terrace_stream_t stream);
+TERRACE_API int terrace_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int rpn,
+                                        void *send_buf, const void *workspace, size_t workspace_bytes,
+                                        terrace_stream_t stream);
+TERRACE_API int terrace_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr, int64_t capacity,
+                                     void *permuted, const void *workspace, size_t workspace_bytes,
+                                     terrace_stream_t stream);
+
 /* ---- zero-copy wire containers: the three stage kernels write / read the containers themselves ----
  * (the follow-up terrace/ta2a_pack.py:462-466 asks for; layouts as terrace_pack_planes above)
  *

@@ -75,6 +75,12 @@ int run_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *s
 int run_map_count(const void *map, int64_t T, int E, int32_t *row_stats, hipStream_t s);
 int run_map_topk(const void *map, const void *probs, int elem_bytes, int64_t T, int E, int k, int64_t *expert_idx,
                  void *gates, hipStream_t s);
+int run_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, int n_nodes, int groups_m,
+                     void *payload, const void *ws, size_t ws_bytes, hipStream_t s);
+int run_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int rpn, void *send_buf,
+                        const void *ws, size_t ws_bytes, hipStream_t s);
+int run_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr, int64_t capacity, void *permuted,
+                     const void *ws, size_t ws_bytes, hipStream_t s);
 }  // namespace terrace
 
 using namespace terrace;
@@ -212,6 +218,24 @@ int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta, int64_t P,
     return run_regroup(node_rx, my_meta, gate_plane, P, row_bytes, gate_bytes, epr, my_local, capacity, permuted,
                        permuted_gate, order, dest, kept, tokens_per_expert, kept_per_expert, status, workspace,
                        workspace_bytes, 2, 2 * (8 / gate_bytes), (hipStream_t)stream);
+}
+
+int terrace_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, int n_nodes, int groups_m,
+                         void *payload, const void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_k2_pack_move(hidden, T, row_bytes, k, n_nodes, groups_m, payload, workspace, workspace_bytes,
+                            (hipStream_t)stream);
+}
+
+int terrace_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int rpn, void *send_buf,
+                            const void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_k1_arrival_move(rx, R, row_bytes, quota, rpn, send_buf, workspace, workspace_bytes,
+                               (hipStream_t)stream);
+}
+
+int terrace_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr, int64_t capacity,
+                         void *permuted, const void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_regroup_move(node_rx, P, row_bytes, epr, capacity, permuted, workspace, workspace_bytes,
+                            (hipStream_t)stream);
 }
 
 int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes, void *out,

@@ -32,6 +32,10 @@ static Units token_units(int64_t T, int n_nodes) {
     return u;
 }
 
+const int32_t *k2_token_positions(const void *ws, int64_t T, int n_nodes) {
+    return (const int32_t *)((const char *)ws + units_table_bytes(token_units(T, n_nodes)));
+}
+
 size_t k2_token_workspace(int64_t T, int n_nodes, int groups_m) {
     return units_table_bytes(token_units(T, n_nodes)) + align_up((size_t)T * groups_m * sizeof(int32_t), 256);
 }

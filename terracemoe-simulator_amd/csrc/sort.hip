@@ -1025,4 +1025,55 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
 #undef TERRACE_K2
 }
 
+// ---- second phase of the three stage operators ---------------------------------------------------
+// A stage call with its row pointers NULL builds the index planes only and leaves the int32 position plane
+// of its row mover in the workspace; these launch that mover later, possibly on another stream, so the
+// index chain of the next stage can run beside the row traffic of this one.  The geometry arguments must
+// repeat the first phase's: they locate the plane.
+int run_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, int n_nodes, int groups_m,
+                     void *payload, const void *ws, size_t ws_bytes, hipStream_t s) {
+    if (T < 0 || k <= 0 || groups_m <= 0 || k % groups_m || n_nodes <= 0 || n_nodes > kMaxBuckets ||
+        row_bytes < 0 || T * groups_m >= (int64_t)1 << 31)
+        return TERRACE_EINVAL;
+    const int64_t S = T * groups_m;
+    if (S == 0 || row_bytes == 0) return TERRACE_OK;
+    if (!hidden || !payload || !ws) return TERRACE_EINVAL;
+    if (ws_bytes < k2_workspace(T, k, n_nodes, groups_m)) return TERRACE_ENOSPC;
+    const int32_t *pos32 = k2_token_path_applies(k, n_nodes)
+                               ? k2_token_positions(ws, T, n_nodes)
+                               : (const int32_t *)((const char *)ws + units_table_bytes(make_units(S, n_nodes)));
+    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
+}
+
+int run_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int rpn, void *send_buf,
+                        const void *ws, size_t ws_bytes, hipStream_t s) {
+    if (R < 0 || quota <= 0 || rpn <= 0 || rpn > kMaxBuckets || row_bytes < 0 || R * quota >= (int64_t)1 << 31)
+        return TERRACE_EINVAL;
+    const int64_t P = R * quota;
+    if (P == 0 || row_bytes == 0) return TERRACE_OK;
+    if (!rx || !send_buf || !ws) return TERRACE_EINVAL;
+    if (ws_bytes < k1_workspace(R, quota, rpn)) return TERRACE_ENOSPC;
+    const int32_t *pos32 = (const int32_t *)((const char *)ws + units_table_bytes(make_units(P, rpn)));
+    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
+}
+
+int run_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr, int64_t capacity, void *permuted,
+                     const void *ws, size_t ws_bytes, hipStream_t s) {
+    if (P < 0 || epr <= 0 || epr > kMaxBuckets || row_bytes < 0 || P >= (int64_t)1 << 31 ||
+        (capacity >= 0 && (int64_t)epr * capacity >= (int64_t)1 << 31))
+        return TERRACE_EINVAL;
+    const int64_t places = capacity >= 0 ? (int64_t)epr * capacity : P;
+    if (places == 0 || row_bytes == 0) return TERRACE_OK;
+    if (!permuted) return TERRACE_EINVAL;
+    if (P == 0) {       // all padding
+        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        return check_launch();
+    }
+    if (!node_rx || !ws) return TERRACE_EINVAL;
+    if (ws_bytes < regroup_workspace(P, epr, capacity)) return TERRACE_ENOSPC;
+    const int32_t *order32 = (const int32_t *)((const char *)ws + units_table_bytes(make_units(P, epr)));
+    const int32_t *gidx = (const int32_t *)((const char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
+    return launch_gather_rows<int32_t>(node_rx, permuted, capacity >= 0 ? gidx : order32, places, row_bytes, s);
+}
+
 }  // namespace terrace

@@ -35,6 +35,8 @@ int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, 
 // is outside that and the caller must take the (token, run)-item path.
 bool k2_token_path_applies(int k, int n_nodes);
 size_t k2_token_workspace(int64_t T, int n_nodes, int groups_m);
+// Where run_k2_token leaves the [T, groups_m] int32 send-row positions inside its workspace.
+const int32_t *k2_token_positions(const void *ws, int64_t T, int n_nodes);
 int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
                  int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                  int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,

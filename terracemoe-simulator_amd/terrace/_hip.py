@@ -17,7 +17,7 @@ ENV_LIB = "TERRACE_OPS_LIB"
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(os.path.dirname(PKG_DIR), "lib")
 
-OK = 0
+OK, EINVAL, ENOSPC, ELAUNCH = 0, -22, -28, -5
 F32, BF16, F16, FP8_B128 = 0, 1, 2, 3
 MODE_CODES = {"full": 0, "group_limited": 1, "quota_only": 2, "global_topk": 3}
 FORCE_GENERIC = 0x100
@@ -59,6 +59,9 @@ SIGNATURES = {
                                      _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_regroup_wire": (_I, [_P, _P, _L, _L, _I, _I, _I, _L,
                                   _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "terrace_k2_pack_move": (_I, [_P, _L, _L, _I, _I, _I, _P, _P, _Z, _P]),
+    "terrace_k1_arrival_move": (_I, [_P, _L, _L, _I, _I, _P, _P, _Z, _P]),
+    "terrace_regroup_move": (_I, [_P, _L, _L, _I, _L, _P, _P, _Z, _P]),
     "terrace_plan_general_workspace": (_Z, [_L, _I]),
     "terrace_plan_general": (_I, [_P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_build_mask": (_I, [_P, _P, _L, _I, _L, _P, _P, _P]),

@@ -380,6 +380,144 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
     return out + (pgate,) if my_gate is not None else out
 
 
+# ---- the stage operators in two phases (index planes first, rows later) -----------------------------
+def k2_pack_index(expert_idx, gates, world, n_experts, rpn, groups_m):
+    """First phase of :func:`k2_pack_raw`: every index plane, no rows.  Returns
+    ((mask, gate_rows, u_src, node_counts), extras) with ``extras["workspace"]`` holding what
+    :func:`k2_pack_move` needs to move the rows later."""
+    _require()
+    _hip.need_device(expert_idx, gates)
+    if expert_idx.dim() != 2 or gates.shape != expert_idx.shape:
+        raise ValueError("k2_pack: expert_idx/gates must be 2-D and of one shape")
+    if expert_idx.dtype != torch.int64:
+        raise RuntimeError("k2_pack: expert_idx must be int64")
+    if gates.element_size() not in (2, 4):
+        raise RuntimeError(f"k2_pack: unsupported gate dtype {gates.dtype}")
+    if world <= 0 or rpn <= 0 or groups_m <= 0 or n_experts <= 0:
+        raise ValueError("k2_pack: bad geometry scalars")
+    T, k = expert_idx.shape
+    if world % rpn or n_experts % world or k % groups_m:
+        raise ValueError(f"k2_pack: world={world} rpn={rpn} n_experts={n_experts} k={k} "
+                         f"groups_m={groups_m} not divisible")
+    expert_idx, gates = expert_idx.contiguous(), gates.contiguous()
+    dev = expert_idx.device
+    S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
+    i64 = dict(dtype=torch.int64, device=dev)
+    mask = torch.empty((S, q), **i64)
+    gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
+    u_src = torch.empty((S,), **i64)
+    node_counts = torch.empty((n_nodes,), **i64)
+    ex = {"u_node": torch.empty((S,), **i64), "inverse": torch.empty((T * k,), **i64),
+          "node_offsets": torch.empty((n_nodes,), **i64), "pair_table": torch.empty((T, k), **i64),
+          "sort_order": torch.empty((T, k), **i64), "token_rows": torch.empty((T, groups_m), **i64),
+          "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
+    _hip.call("terrace_k2_pack", None, _hip.ptr(expert_idx), _hip.ptr(gates), T, 0, gates.element_size(), k,
+              world, n_experts, rpn, groups_m, None, _hip.ptr(mask), _hip.ptr(gate_rows), _hip.ptr(u_src),
+              _hip.ptr(node_counts), _hip.ptr(ex["u_node"]), _hip.ptr(ex["inverse"]), _hip.ptr(ex["node_offsets"]),
+              _hip.ptr(ex["pair_table"]), _hip.ptr(ex["sort_order"]), _hip.ptr(ex["token_rows"]),
+              _hip.ptr(ex["gate_sorted"]), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    ex["status"], ex["workspace"] = st, ws
+    return (mask, gate_rows, u_src, node_counts), ex
+
+
+def k2_pack_move(hidden, workspace, k, world, rpn, groups_m):
+    """Second phase: the Hop-A payload [T*groups_m, H] of ``hidden`` from the first phase's workspace."""
+    _require()
+    _hip.need_device(hidden, workspace)
+    if hidden.dim() != 2:
+        raise ValueError("k2_pack: hidden must be 2-D")
+    hidden = hidden.contiguous()
+    T, H = hidden.shape
+    payload = torch.empty((T * groups_m, H), dtype=hidden.dtype, device=hidden.device)
+    _hip.call("terrace_k2_pack_move", _hip.ptr(hidden), T, H * hidden.element_size(), k, world // rpn, groups_m,
+              _hip.ptr(payload), _hip.ptr(workspace), workspace.numel(), _hip.stream(hidden.device))
+    return payload
+
+
+def k1_arrival_index(rslot, rgate, quota, epr, rpn, my_local=0):
+    """First phase of :func:`k1_arrival_raw`: (gate_pairs, r_idx, slot_idx, i_send, pair_pos, workspace)."""
+    _require()
+    _hip.need_device(rslot, rgate)
+    if rslot.dim() != 2 or rgate.dim() != 2 or rslot.shape != rgate.shape or rslot.shape[1] != quota:
+        raise RuntimeError(f"k1_arrival: rslot {tuple(rslot.shape)} / rgate {tuple(rgate.shape)} must be [R, {quota}]")
+    if rslot.dtype != torch.int64:
+        raise RuntimeError("k1_arrival: rslot must be int64")
+    if rgate.element_size() not in (2, 4):
+        raise RuntimeError(f"k1_arrival: unsupported gate dtype {rgate.dtype}")
+    if quota <= 0 or epr <= 0 or rpn <= 0 or not 0 <= my_local < rpn:
+        raise RuntimeError("k1_arrival: bad geometry scalars")
+    rslot, rgate = rslot.contiguous(), rgate.contiguous()
+    dev = rslot.device
+    R = rslot.shape[0]
+    P = R * quota
+    i64 = dict(dtype=torch.int64, device=dev)
+    gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
+    r_idx, slot_idx, pair_pos = torch.empty((P,), **i64), torch.empty((P,), **i64), torch.empty((P,), **i64)
+    i_send = torch.empty((rpn,), **i64)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
+    _hip.call("terrace_k1_arrival", None, _hip.ptr(rslot), _hip.ptr(rgate), R, 0, rgate.element_size(), quota, epr,
+              rpn, my_local, None, _hip.ptr(gate_pairs), _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send),
+              _hip.ptr(pair_pos), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return gate_pairs, r_idx, slot_idx, i_send, pair_pos, ws
+
+
+def k1_arrival_move(rx, workspace, quota, rpn):
+    """Second phase: ``send_buf`` [R*quota, H] of the arrived rows ``rx`` from the first phase's workspace."""
+    _require()
+    _hip.need_device(rx, workspace)
+    if rx.dim() != 2:
+        raise RuntimeError("k1_arrival: rx must be 2-D")
+    rx = rx.contiguous()
+    R, H = rx.shape
+    send_buf = torch.empty((R * quota, H), dtype=rx.dtype, device=rx.device)
+    _hip.call("terrace_k1_arrival_move", _hip.ptr(rx), R, H * rx.element_size(), quota, rpn, _hip.ptr(send_buf),
+              _hip.ptr(workspace), workspace.numel(), _hip.stream(rx.device))
+    return send_buf
+
+
+def regroup_index(my_slot, epr, my_local=0, capacity=None):
+    """First phase of :func:`regroup`: a dict with tokens_per_expert, kept_per_expert, the row -> place plane
+    ``dest`` (-1 = dropped), ``order`` (drop-less) or ``kept`` (capacity), and the workspace."""
+    _require()
+    _hip.need_device(my_slot)
+    if my_slot.dtype != torch.int64:
+        raise RuntimeError("regroup: my_slot must be int64")
+    my_slot = my_slot.contiguous().reshape(-1)
+    dev = my_slot.device
+    P = my_slot.numel()
+    cap = -1 if capacity is None else int(capacity)
+    i64 = dict(dtype=torch.int64, device=dev)
+    tpe, kpe, dest = torch.empty((epr,), **i64), torch.empty((epr,), **i64), torch.empty((P,), **i64)
+    order = torch.empty((P,), **i64) if capacity is None else None
+    kept = torch.empty((P,), dtype=torch.uint8, device=dev) if capacity is not None else None
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, cap), dev)
+    _hip.call("terrace_regroup", None, _hip.ptr(my_slot), None, P, 0, 4, epr, my_local, cap, None, None,
+              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    return {"tokens_per_expert": tpe, "kept_per_expert": kpe, "dest": dest, "order": order,
+            "kept": None if kept is None else kept.bool(), "workspace": ws}
+
+
+def regroup_move(node_rx, workspace, epr, capacity=None):
+    """Second phase: the expert-order buffer ([P, H], or [epr*capacity, H] with zero padding rows)."""
+    _require()
+    _hip.need_device(node_rx, workspace)
+    if node_rx.dim() != 2:
+        raise RuntimeError("regroup: node_rx must be 2-D")
+    node_rx = node_rx.contiguous()
+    P, H = node_rx.shape
+    cap = -1 if capacity is None else int(capacity)
+    places = P if capacity is None else epr * cap
+    permuted = torch.empty((places, H), dtype=node_rx.dtype, device=node_rx.device)
+    _hip.call("terrace_regroup_move", _hip.ptr(node_rx), P, H * node_rx.element_size(), epr, cap,
+              _hip.ptr(permuted), _hip.ptr(workspace), workspace.numel(), _hip.stream(node_rx.device))
+    return permuted
+
+
 def gather_rows(src, idx):
     """``src[idx]`` for a 2-D ``src``; negative indices give zero rows."""
     _require()

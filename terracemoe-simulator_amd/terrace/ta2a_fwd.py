@@ -10,6 +10,7 @@ the balanced size) and every expert slot of the node treated as local.
 """
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass
 
 import torch
@@ -123,24 +124,91 @@ class LoopbackState:
     capacity: int | None
 
 
+_INDEX_STREAMS: dict = {}
+
+
+def _index_stream(device) -> "torch.cuda.Stream":
+    """The per-device stream (default priority) the index chain runs on beside the row movers."""
+    key = torch.device(device).index
+    if key is None:
+        key = torch.cuda.current_device()
+    s = _INDEX_STREAMS.get(key)
+    if s is None:
+        s = _INDEX_STREAMS[key] = torch.cuda.Stream(device=key)
+    return s
+
+
+def _adopt(stream, *items):
+    """Tensors allocated under another stream that ``stream`` will also use: tell the allocator."""
+    for t in items:
+        if isinstance(t, dict):
+            _adopt(stream, *t.values())
+        elif isinstance(t, torch.Tensor) and t.is_cuda:
+            t.record_stream(stream)
+
+
 def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8, groups_m: int = 1,
-                      capacity: int | None = None) -> LoopbackState:
-    """Stages 2-4 on one GPU: index build + Hop-A pack, arrival chain, expert-order regroup."""
+                      capacity: int | None = None, overlap: bool | None = None) -> LoopbackState:
+    """Stages 2-4 on one GPU: index build + Hop-A pack, arrival chain, expert-order regroup.
+
+    ``overlap`` (default: the ``TERRACE_OVERLAP`` environment switch, off unless "1"): every index plane
+    of the three stages depends only on index planes of the stage before, never on moved rows -- the
+    property the reference uses when it ships counts and metadata ahead of the payload
+    (terrace/ta2a_dispatch.py:78-100, 399-412).  With ``overlap`` the whole index chain, the combine's
+    place table included, runs ahead on a second stream while the current stream moves rows back to back,
+    each mover waiting only for the event of its own stage's planes.  The results are the same tensors
+    either way.  It is off by default because on one GPU it measured slower: the movers do run back to
+    back, but each of the five cross-stream waits costs about 11 us where the index kernel it hides costs
+    5 us (T=16384, H=7168 bf16: 1.81 ms a step against 1.69 ms).  The two-phase operators underneath are
+    what a multi-GPU caller needs regardless, with the payload exchange between the phases."""
     epr = n_experts // world
     slots = epr * rpn
     k = expert_idx.shape[1]
     quota = k // groups_m
-    (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
-        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
-    send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = _ops.k1_arrival_raw(
-        payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True)
-    if capacity is None:
-        permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots)
-        kept = None
-    else:
-        permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity)
+    if overlap is None:
+        overlap = os.environ.get("TERRACE_OVERLAP", "0") == "1"
+    if not overlap or x.shape[0] == 0:
+        (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
+            x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+        send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = _ops.k1_arrival_raw(
+            payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True)
+        if capacity is None:
+            permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots)
+            kept = None
+        else:
+            permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity)
+        return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
+                             slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
+
+    _ops._check_k2(x, expert_idx, gates, world, n_experts, rpn, groups_m)
+    dev = x.device
+    rows = torch.cuda.current_stream(dev)
+    index = _index_stream(dev)
+    index.wait_stream(rows)
+    with torch.cuda.stream(index):
+        (mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_index(
+            expert_idx, gates, world, n_experts, rpn, groups_m)
+        packed = index.record_event()
+        gate_pairs, r_idx, slot_idx, i_send, pair_pos, ws_arrival = _ops.k1_arrival_index(
+            mask, gate_rows, quota, epr, rpn, 0)
+        arrived = index.record_event()
+        rg = _ops.regroup_index(slot_idx, slots, 0, capacity)
+        regrouped = index.record_event()
+        place = rg["dest"]
+        where = _ops.index_chain2(place, pair_pos, extras["pair_table"])
+        chained = index.record_event()
+    _adopt(rows, mask, gate_rows, u_src, node_counts, extras, gate_pairs, r_idx, slot_idx, i_send, pair_pos,
+           ws_arrival, rg, where)
+    rows.wait_event(packed)
+    payload = _ops.k2_pack_move(x, extras["workspace"], k, world, rpn, groups_m)
+    rows.wait_event(arrived)
+    send_buf = _ops.k1_arrival_move(payload, ws_arrival, quota, rpn)
+    rows.wait_event(regrouped)
+    permuted = _ops.regroup_move(send_buf, rg["workspace"], slots, capacity)
+    rows.wait_event(chained)            # joins the index stream: nothing of it is in flight on return
+    extras["where"] = where
     return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
-                         slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
+                         slot_idx, i_send, pair_pos, permuted, rg["tokens_per_expert"], place, rg["kept"], capacity)
 
 
 def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
@@ -176,7 +244,9 @@ def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, wei
     node ascending across the token's rows -- which is the order the reference's two
     ``index_add`` levels add in (terrace/ta2a_fwd.py:661-670 there), accumulated in fp32.
     """
-    where = _ops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
+    where = st.extras.get("where")
+    if where is None:
+        where = _ops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
     w = st.extras["gate_sorted"] if weights is None else weights
     return _ops.combine(ye, where, w, out_dtype=out_dtype, fp8_hidden=fp8_hidden)
 

@@ -226,3 +226,70 @@ def test_full_size_index_planes_and_round_trip(name):
         xf = x.float()
     err = ((got - xf * gsum).abs().max() / xf.abs().max()).item()
     assert err <= 2 * TOL[cfg.fmt], err
+
+
+def _state_planes(st):
+    planes = {k: getattr(st, k) for k in ("payload", "mask", "gate_rows", "u_src", "node_counts", "send_buf",
+                                           "gate_pairs", "r_idx", "slot_idx", "i_send", "pair_pos", "permuted",
+                                           "tokens_per_expert", "place", "kept")}
+    for k in ("u_node", "inverse", "node_offsets", "pair_table", "sort_order", "token_rows", "gate_sorted"):
+        planes["extras." + k] = st.extras[k]
+    return planes
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c4", "c5"])
+def test_two_phase_operators_and_overlapped_dispatch_equal_the_single_calls(name):
+    """Index-only first phases + the *_move second phases, run by loopback_dispatch(overlap=True) with the
+    index chain on a second stream, must give bit for bit what the one-call operators give -- twice in a
+    row, so that memory handed back by the first pass is reused while both streams are busy."""
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    cfg = configs.CONFIGS[name].scaled(3000)
+    announce("two-phase", cfg.name, cfg.T)
+    inp = configs.make_inputs(cfg)
+    e, g, _, _ = _route(cfg, inp)
+    x = inp["x"].to(DEV)
+    gates = g.to(cfg.gate_dtype)
+    cap = cfg.capacity(cfg.slots)
+    args = (x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    plain = loopback_dispatch(*args, overlap=False)
+    ye = plain.permuted.clone() if cfg.fmt != "fp8" else configs.quantise_fp8_rows(
+        torch.randn(plain.permuted.shape[0], cfg.hidden, device=DEV))
+    fp8_hidden = cfg.hidden if cfg.fmt == "fp8" else None
+    y_plain = loopback_combine(ye, plain, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+    for _ in range(2):
+        both = loopback_dispatch(*args, overlap=True)
+        y_both = loopback_combine(ye, both, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+        torch.cuda.synchronize()
+        want, got = _state_planes(plain), _state_planes(both)
+        for k, w in want.items():
+            if w is None:
+                assert got[k] is None, k
+            else:
+                assert torch.equal(got[k], w), f"{k} differs between the one-call and the two-phase dispatch"
+        assert torch.equal(y_both, y_plain)
+
+
+def test_move_phases_refuse_bad_arguments():
+    from terrace import _hip
+    import terrace.ops as tops
+    tops.status()
+    ws = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    x = torch.zeros((64, 64), dtype=torch.float32, device=DEV)
+    out = torch.zeros((128, 64), dtype=torch.float32, device=DEV)
+    s = _hip.stream(DEV)
+    lib = _hip.load()
+    # a workspace smaller than the first phase's is refused, not read out of bounds
+    assert lib.terrace_k2_pack_move(_hip.ptr(x), 1 << 20, 256, 8, 8, 4, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.ENOSPC
+    assert lib.terrace_k1_arrival_move(_hip.ptr(x), 1 << 20, 256, 2, 8, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.ENOSPC
+    assert lib.terrace_regroup_move(_hip.ptr(x), 1 << 20, 256, 32, -1, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.ENOSPC
+    # geometry and null pointers
+    assert lib.terrace_k2_pack_move(_hip.ptr(x), 64, 256, 8, 8, 3, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.EINVAL
+    assert lib.terrace_k2_pack_move(None, 64, 256, 8, 8, 4, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.EINVAL
+    assert lib.terrace_k1_arrival_move(_hip.ptr(x), 64, 256, 0, 8, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.EINVAL
+    assert lib.terrace_regroup_move(_hip.ptr(x), 64, 256, 0, -1, _hip.ptr(out), _hip.ptr(ws), 4096, s) == _hip.EINVAL
+    # nothing to move is fine without any pointer
+    assert lib.terrace_k2_pack_move(None, 0, 256, 8, 8, 4, None, None, 0, s) == _hip.OK
+    assert lib.terrace_k1_arrival_move(None, 0, 256, 2, 8, None, None, 0, s) == _hip.OK
+    assert lib.terrace_regroup_move(None, 0, 256, 32, -1, None, None, 0, s) == _hip.OK
+    torch.cuda.synchronize()
