@@ -61,7 +61,12 @@ enum terrace_route_mode { /* terrace/routing.py:66 _MODES, same order */
     TERRACE_ROUTE_GLOBAL_TOPK = 3,
     /* or-ed into `mode`: use the LDS-staged kernel even where the register-resident one
      * applies (both give identical results; this exists so tests can compare them) */
-    TERRACE_ROUTE_FORCE_GENERIC = 0x100
+    TERRACE_ROUTE_FORCE_GENERIC = 0x100,
+    /* or-ed into `mode`: `gates` is a bf16 / f16 plane and each gate is rounded to nearest-even on the way
+     * out -- the cast to the payload dtype that the gate plane needs anyway (terrace/ta2a_dispatch.py:550-564),
+     * without a launch of its own */
+    TERRACE_ROUTE_GATES_BF16 = 0x200,
+    TERRACE_ROUTE_GATES_F16 = 0x400
 };
 
 enum terrace_fault {
@@ -81,13 +86,13 @@ TERRACE_API const char *terrace_strerror(int status);
 TERRACE_API int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t stream);
 
 /* T-Route (terrace/routing.py:45-96).  affinity [T,E] f32, bias [E] f32, gate_affinity
- * [T,E] f32 or NULL (= affinity).  Writes expert_idx [T,k] i64, gates [T,k] f32,
+ * [T,E] f32 or NULL (= affinity).  Writes expert_idx [T,k] i64, gates [T,k] f32 (bf16 / f16 with the mode flags),
  * group_idx [T,G] i64 with G = top_groups (full, group_limited), n_groups (quota_only) or
  * top_k (global_topk).  Ties go to the lowest index; gates are raw/sum(raw) with the sum
  * taken left to right in fp32.  pool = TRouteConfig.group_score_pool (1 or 2). */
 TERRACE_API int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T,
                     int n_experts, int n_groups, int top_k, int top_groups, int pool, int mode,
-                    int64_t *expert_idx, float *gates, int64_t *group_idx, terrace_stream_t stream);
+                    int64_t *expert_idx, void *gates, int64_t *group_idx, terrace_stream_t stream);
 
 /* expert_load (terrace/routing.py:112-113) and fixed_hist (terrace/ta2a_fwd.py:299-321):
  * out[b] = #{i : idx[i] == b}; out is int64 [n_buckets] or, with as_float != 0, float32. */

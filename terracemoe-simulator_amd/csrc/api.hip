@@ -19,8 +19,8 @@ int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src,
 template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
 int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
-                int k, int M, int pool, int mode, int64_t *expert_idx, float *gates, int64_t *group_idx,
-                int force_generic, hipStream_t s);
+                int k, int M, int pool, int mode, int64_t *expert_idx, void *gates, int gate_dtype,
+                int64_t *group_idx, int force_generic, hipStream_t s);
 size_t hist_workspace(int64_t n, int n_buckets);
 int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status, void *ws,
              size_t ws_bytes, hipStream_t s);
@@ -107,11 +107,15 @@ int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t 
 }
 
 int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int n_experts,
-                    int n_groups, int top_k, int top_groups, int pool, int mode, int64_t *expert_idx, float *gates,
+                    int n_groups, int top_k, int top_groups, int pool, int mode, int64_t *expert_idx, void *gates,
                     int64_t *group_idx, terrace_stream_t stream) {
     const int force = (mode & TERRACE_ROUTE_FORCE_GENERIC) ? 1 : 0;
-    return run_t_route(affinity, bias, gate_affinity, T, n_experts, n_groups, top_k, top_groups, pool,
-                       mode & ~TERRACE_ROUTE_FORCE_GENERIC, expert_idx, gates, group_idx, force, (hipStream_t)stream);
+    const int flags = TERRACE_ROUTE_FORCE_GENERIC | TERRACE_ROUTE_GATES_BF16 | TERRACE_ROUTE_GATES_F16;
+    if ((mode & TERRACE_ROUTE_GATES_BF16) && (mode & TERRACE_ROUTE_GATES_F16)) return TERRACE_EINVAL;
+    const int gate_dtype = (mode & TERRACE_ROUTE_GATES_BF16) ? TERRACE_BF16
+                                                             : ((mode & TERRACE_ROUTE_GATES_F16) ? TERRACE_F16 : TERRACE_F32);
+    return run_t_route(affinity, bias, gate_affinity, T, n_experts, n_groups, top_k, top_groups, pool, mode & ~flags,
+                       expert_idx, gates, gate_dtype, group_idx, force, (hipStream_t)stream);
 }
 
 size_t terrace_hist_workspace(int64_t n, int n_buckets) { return hist_workspace(n, n_buckets); }

@@ -85,8 +85,16 @@ __device__ __forceinline__ void best_range(float &v, int &i) {
 
 // Shared epilogue of the generic kernel: sel[0..k) holds the chosen expert ids (wave-private LDS).
 // An id outside [0, E) can only come from NaN scores (never ranked); it is clamped to 0.
+// A gate goes out as fp32, or rounded to nearest-even to the 16-bit type the payload is in (what the caller's
+// `gates.to(payload dtype)` would do in a launch of its own).
+__device__ __forceinline__ void store_gate(void *gates, int gate_dtype, int64_t at, float v) {
+    if (gate_dtype == TERRACE_F32) ((float *)gates)[at] = v;
+    else if (gate_dtype == TERRACE_BF16) ((uint16_t *)gates)[at] = (uint16_t)f32_to_bf16_bits(v);
+    else ((uint16_t *)gates)[at] = __half_as_ushort(__float2half_rn(v));
+}
+
 __device__ __forceinline__ void write_token(int *sel, float *raw, const float *gate_row, int k, int E, int64_t t,
-                                            int64_t *expert_idx, float *gates) {
+                                            int64_t *expert_idx, void *gates, int gate_dtype) {
     const int lane = lane_id();
     for (int j = lane; j < k; j += kWave) {
         if ((unsigned)sel[j] >= (unsigned)E) sel[j] = 0;
@@ -97,7 +105,7 @@ __device__ __forceinline__ void write_token(int *sel, float *raw, const float *g
     for (int j = 0; j < k; ++j) den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
     for (int j = lane; j < k; j += kWave) {
         expert_idx[t * k + j] = sel[j];
-        gates[t * k + j] = __fdiv_rn(((volatile float *)raw)[j], den);
+        store_gate(gates, gate_dtype, t * k + j, __fdiv_rn(((volatile float *)raw)[j], den));
     }
 }
 
@@ -116,7 +124,7 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
                                                             const float *__restrict__ gate_affinity, int64_t T, int E,
                                                             int k, int M, int pool,
                                                             int64_t *__restrict__ expert_idx,
-                                                            float *__restrict__ gates,
+                                                            void *__restrict__ gates, int gate_dtype,
                                                             int64_t *__restrict__ group_idx) {
     extern __shared__ int32_t lds[];
     constexpr int LPT = kWave / TPW;
@@ -277,7 +285,7 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
         if (tl < k && live) {
             expert_idx[t * k + tl] = ((volatile int *)sel)[tl];
-            gates[t * k + tl] = __fdiv_rn(((volatile float *)raw)[tl], den);
+            store_gate(gates, gate_dtype, t * k + tl, __fdiv_rn(((volatile float *)raw)[tl], den));
         }
         __builtin_amdgcn_wave_barrier();
     }
@@ -304,7 +312,7 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
                                                                const float *__restrict__ gate_affinity, int64_t T,
                                                                int E, int n_groups, int k, int M, int pool, int mode,
                                                                int n_group_out, int64_t *__restrict__ expert_idx,
-                                                               float *__restrict__ gates,
+                                                               void *__restrict__ gates, int gate_dtype,
                                                                int64_t *__restrict__ group_idx) {
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
@@ -422,7 +430,7 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
             }
         }
         __builtin_amdgcn_wave_barrier();
-        write_token(sel, raw, (gate_affinity ? gate_affinity : affinity) + t * E, k, E, t, expert_idx, gates);
+        write_token(sel, raw, (gate_affinity ? gate_affinity : affinity) + t * E, k, E, t, expert_idx, gates, gate_dtype);
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -431,9 +439,10 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
 static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 
 int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
-                int k, int M, int pool, int mode, int64_t *expert_idx, float *gates, int64_t *group_idx,
-                int force_generic, hipStream_t s) {
-    if (T < 0 || E <= 0 || n_groups <= 0 || k <= 0 || M <= 0 || pool < 1 || pool > 2 || mode < 0 || mode > 3)
+                int k, int M, int pool, int mode, int64_t *expert_idx, void *gates, int gate_dtype,
+                int64_t *group_idx, int force_generic, hipStream_t s) {
+    if (T < 0 || E <= 0 || n_groups <= 0 || k <= 0 || M <= 0 || pool < 1 || pool > 2 || mode < 0 || mode > 3 ||
+        (gate_dtype != TERRACE_F32 && gate_dtype != TERRACE_BF16 && gate_dtype != TERRACE_F16))
         return TERRACE_EINVAL;
     if (E % n_groups || k % M || k > E || E > 2048 || M > n_groups) return TERRACE_EINVAL;
     const int g = E / n_groups;
@@ -463,7 +472,7 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
             const size_t lds = (size_t)kWavesPerBlock * tpw * 2 * k * sizeof(int32_t);
 #define TERRACE_ROUTE(V, L, W)                                                                                  \
     route_wave_kernel<V, L, W><<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, k, M, pool, \
-                                                                expert_idx, gates, group_idx)
+                                                                expert_idx, gates, gate_dtype, group_idx)
 #define TERRACE_ROUTE_W(V, L)                                \
     switch (tpw) {                                           \
         case 1: TERRACE_ROUTE(V, L, 1); break;               \
@@ -499,7 +508,7 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
     const int n_group_out = mode == TERRACE_ROUTE_QUOTA_ONLY ? n_groups : (mode == TERRACE_ROUTE_GLOBAL_TOPK ? k : M);
     const size_t lds = (size_t)kWavesPerBlock * (E + 2 * n_groups + 2 * k) * sizeof(int32_t);
     route_generic_kernel<<<(int)blocks, kBlock, lds, s>>>(affinity, bias, gate_affinity, T, E, n_groups, k, M, pool,
-                                                          mode, n_group_out, expert_idx, gates, group_idx);
+                                                          mode, n_group_out, expert_idx, gates, gate_dtype, group_idx);
     return check_launch();
 }
 

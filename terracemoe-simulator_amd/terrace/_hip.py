@@ -21,6 +21,7 @@ OK, EINVAL, ENOSPC, ELAUNCH = 0, -22, -28, -5
 F32, BF16, F16, FP8_B128 = 0, 1, 2, 3
 MODE_CODES = {"full": 0, "group_limited": 1, "quota_only": 2, "global_topk": 3}
 FORCE_GENERIC = 0x100
+GATES_FLAG = {torch.float32: 0, torch.bfloat16: 0x200, torch.float16: 0x400}
 FAULT_ID_RANGE, FAULT_QUOTA, FAULT_FANOUT = 1, 2, 4
 STATUS_WORDS = 4
 

@@ -376,7 +376,7 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
     if capacity is None:
         out = (permuted, order, tpe)
     else:
-        out = (permuted, dest, kept.bool(), tpe, kpe)
+        out = (permuted, dest, kept.view(torch.bool), tpe, kpe)
     return out + (pgate,) if my_gate is not None else out
 
 
@@ -499,7 +499,7 @@ def regroup_index(my_slot, epr, my_local=0, capacity=None):
               _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st),
               _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     return {"tokens_per_expert": tpe, "kept_per_expert": kpe, "dest": dest, "order": order,
-            "kept": None if kept is None else kept.bool(), "workspace": ws}
+            "kept": None if kept is None else kept.view(torch.bool), "workspace": ws}
 
 
 def regroup_move(node_rx, workspace, epr, capacity=None):

@@ -46,12 +46,17 @@ class TRouteConfig:
 
 
 def t_route(affinity: torch.Tensor, bias: torch.Tensor, cfg: TRouteConfig, mode: str = "full", *,
-            gate_affinity: torch.Tensor | None = None, _force_generic: bool = False):
+            gate_affinity: torch.Tensor | None = None, gates_dtype: torch.dtype = torch.float32,
+            _force_generic: bool = False):
     """Returns (expert_idx [T, k] int64, gates [T, k] float32, group_idx [T, M] int64).
 
-    ``gate_affinity`` (an addition to the reference signature) is the [T, E] table the gate
-    values are read from; it defaults to ``affinity``.  Selection never looks at it.
+    Two additions to the reference signature: ``gate_affinity`` is the [T, E] table the gate values
+    are read from (default ``affinity``; selection never looks at it), and ``gates_dtype``
+    (float32, bfloat16 or float16) has the kernel write ``gates.to(gates_dtype)`` directly -- the
+    payload-dtype gate plane the dispatch needs, without the extra cast launch.
     """
+    if gates_dtype not in _hip.GATES_FLAG:
+        raise ValueError(f"gates_dtype must be float32, bfloat16 or float16, got {gates_dtype}")
     if mode not in _MODES:
         raise ValueError(f"unknown routing mode {mode!r}; expected one of {_MODES}")
     if mode == "quota_only" and cfg.top_k // cfg.n_groups < 1:
@@ -78,9 +83,9 @@ def t_route(affinity: torch.Tensor, bias: torch.Tensor, cfg: TRouteConfig, mode:
     n_g_out = {"full": cfg.top_groups, "group_limited": cfg.top_groups, "quota_only": cfg.n_groups,
                "global_topk": cfg.top_k}[mode]
     expert_idx = torch.empty((T, cfg.top_k), dtype=torch.int64, device=dev)
-    gates = torch.empty((T, cfg.top_k), dtype=torch.float32, device=dev)
+    gates = torch.empty((T, cfg.top_k), dtype=gates_dtype, device=dev)
     group_idx = torch.empty((T, n_g_out), dtype=torch.int64, device=dev)
-    code = _hip.MODE_CODES[mode] | (_hip.FORCE_GENERIC if _force_generic else 0)
+    code = _hip.MODE_CODES[mode] | (_hip.FORCE_GENERIC if _force_generic else 0) | _hip.GATES_FLAG[gates_dtype]
     _hip.call("terrace_t_route", _hip.ptr(aff), _hip.ptr(b), _hip.ptr(ga), T, cfg.n_experts, cfg.n_groups,
               cfg.top_k, cfg.top_groups, cfg.group_score_pool, code, _hip.ptr(expert_idx), _hip.ptr(gates),
               _hip.ptr(group_idx), _hip.stream(dev))

@@ -132,6 +132,38 @@ def test_route_other_modes(mode):
         same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
 
 
+@pytest.mark.parametrize("generic", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_route_gates_in_the_payload_dtype(generic, dtype):
+    """gates_dtype: the kernel's 16-bit gates are the fp32 gates rounded to nearest-even -- the bits of torch's
+    own cast (and of the oracle's) -- and nothing else of the result moves."""
+    import terrace
+    announce("route gates dtype", generic, dtype)
+    g = torch.Generator().manual_seed(3)
+    for (T, E, Ng, k, M) in [(2048, 256, 8, 8, 4), (700, 64, 8, 4, 2), (65, 96, 4, 8, 4), (300, 128, 16, 8, 2)]:
+        logits = torch.randn(T, E, generator=g)
+        bias = torch.randn(E, generator=g) * 0.1
+        gate_tab = torch.exp(logits - logits.max(-1, keepdim=True).values)
+        cfg = terrace.TRouteConfig(E, Ng, k, M)
+        args = (logits.to(DEV), bias.to(DEV), cfg)
+        e32, g32, grp32 = terrace.t_route(*args, gate_affinity=gate_tab.to(DEV), _force_generic=generic)
+        e16, g16, grp16 = terrace.t_route(*args, gate_affinity=gate_tab.to(DEV), gates_dtype=dtype,
+                                          _force_generic=generic)
+        assert g16.dtype == dtype and torch.equal(e16, e32) and torch.equal(grp16, grp32)
+        assert torch.equal(g16, g32.to(dtype))
+        _, og, _ = orc.t_route(logits.numpy(), bias.numpy(), E, Ng, k, M, gate_affinity=gate_tab.numpy())
+        assert torch.equal(g16.cpu(), torch.from_numpy(og).to(dtype))
+    for mode in ("group_limited", "quota_only", "global_topk"):
+        cfg = terrace.TRouteConfig(64, 8, 8, 4)
+        aff = torch.rand(200, 64, generator=g).to(DEV)
+        zero = torch.zeros(64, device=DEV)
+        _, g32, _ = terrace.t_route(aff, zero, cfg, mode=mode)
+        _, g16, _ = terrace.t_route(aff, zero, cfg, mode=mode, gates_dtype=dtype)
+        assert torch.equal(g16, g32.to(dtype))
+    with pytest.raises(ValueError):
+        terrace.t_route(aff, zero, cfg, gates_dtype=torch.float64)
+
+
 def test_expert_load_and_hist_and_argsort():
     import terrace
     from terrace.ta2a_fwd import _stable_argsort_small, fixed_hist
