@@ -571,6 +571,52 @@ def test_hopb_meta_and_container_errors():
         pk.hopb_pack_meta(ids[:2], torch.zeros(3, device=DEV))
 
 
+@pytest.mark.parametrize("rows", [0, 1, 2, 3, 17])
+def test_unpacked_planes_own_their_memory(rows):
+    """What the reference guards with ``_own`` (terrace/ta2a_pack.py:182-205 there, exercised by its
+    tests/test_ta2a_pack_alias.py): no unpacked plane may live in the container's storage, at one row
+    least of all, so the planes must read back right after the container's memory is handed back."""
+    from terrace import ta2a_pack as pk
+    announce("container ownership", rows)
+    H, q, slots = 2048, 3, 24
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        payload = (torch.arange(rows * H, dtype=torch.float32).reshape(rows, H) % 251).to(dtype).to(DEV)
+        gate = torch.full((rows, q), 0.5, dtype=dtype, device=DEV)
+        ids = torch.arange(rows * q, dtype=torch.int64, device=DEV).reshape(rows, q)
+        buf, lay = pk.hopa_pack(payload, gate, ids)
+        rx, rgate, rmask = pk.hopa_unpack(buf, lay)
+        pk.assert_not_aliased(buf, rx, rgate, rmask)
+        for plane in (rx, rgate, rmask):
+            assert plane.numel() == 0 or plane.untyped_storage().data_ptr() != buf.untyped_storage().data_ptr()
+        torch.cuda.synchronize()
+        buf.untyped_storage().resize_(0)
+        assert torch.equal(rx, payload) and torch.equal(rgate, gate) and torch.equal(rmask, ids)
+        assert torch.equal(rmask // 3, ids // 3)
+    # the bitmask format (1-D id plane) and the Hop-B container
+    payload = torch.zeros(rows, H, dtype=torch.bfloat16, device=DEV)
+    buf, lay = pk.hopa_pack(payload, torch.zeros(rows, slots, dtype=torch.bfloat16, device=DEV),
+                            torch.arange(rows, dtype=torch.int64, device=DEV))
+    assert lay.id_1d
+    pk.assert_not_aliased(buf, *pk.hopa_unpack(buf, lay))
+    slot = torch.arange(rows, dtype=torch.int64, device=DEV)
+    meta = pk.hopb_pack_meta(slot, torch.ones(rows, dtype=torch.bfloat16, device=DEV))
+    s2, g2 = pk.hopb_unpack_meta(meta, torch.bfloat16)
+    pk.assert_not_aliased(meta, s2, g2)
+    torch.cuda.synchronize()
+    meta.untyped_storage().resize_(0)
+    assert torch.equal(s2, slot) and bool((g2 == 1).all())
+
+
+def test_alias_tripwire_fires_on_a_view():
+    from terrace import ta2a_pack as pk
+    buf = torch.zeros(4, 8, dtype=torch.int64, device=DEV)
+    view = buf[:, :2]
+    with pytest.raises(RuntimeError, match="shared storage"):
+        pk.assert_not_aliased(buf, view)
+    pk.assert_not_aliased(buf, view.clone())
+    pk.assert_not_aliased(buf, torch.zeros(0, dtype=torch.int64, device=DEV), None)
+
+
 @pytest.mark.parametrize("row_bytes", [16, 48, 1024, 1040, 7392, 14336, 40, 6, 3])
 def test_row_movers_at_every_base_alignment(row_bytes):
     """Straight through the C ABI with source and destination bases at 16-byte-granular (and, for
