@@ -69,7 +69,8 @@ def event_ms(fn, reps, torch):
 def cpu_baseline(cfg, sample_tokens):
     """The CPU oracle timed on the host cores over `sample_tokens` tokens of the same geometry:
     the OpenMP C restatement (oracle/terrace_oracle.c) when its library is built, else the numpy
-    one.  Best of three passes; algorithmic GB/s over the same stage set as the GPU figure."""
+    one.  Passes are repeated for about eight seconds (3 to 40 of them: the hosts are shared and noisy) and
+    each stage's best time counts; algorithmic GB/s over the same stage set as the GPU figure."""
     import numpy as np
     import torch
     from oracle import c_oracle as corc
@@ -87,9 +88,10 @@ def cpu_baseline(cfg, sample_tokens):
     else:
         x, gcast, fmt = inp["x"].numpy(), orc.f32_to_bf16, "fp8"
     impl = corc if use_c else orc
-    best = None
-    for _attempt in range(3):          # later passes run on warm pages
+    best, totals, began = None, [], time.perf_counter()
+    while len(totals) < 3 or (len(totals) < 40 and time.perf_counter() - began < 8.0):
         t = _oracle_pass(impl, orc, np, small, logits, bias, ga, x, gcast, fmt, use_c)
+        totals.append(sum(t.values()))
         best = t if best is None else {k: min(best[k], t[k]) for k in t}
     t = best
     nbytes = sum(configs.algorithmic_bytes(small).values())
@@ -97,8 +99,10 @@ def cpu_baseline(cfg, sample_tokens):
     cores = corc.threads() if use_c else 1
     what = f"OpenMP C oracle ({cores} threads)" if use_c else "numpy oracle (1 thread)"
     return {"value": round(nbytes / total / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{what}, whole path on {small.T} of {cfg.T} tokens of {cfg.name}, best of 3 passes "
-                      f"({total:.3f} s: " + ", ".join(f"{k} {v:.3f}" for k, v in t.items()) + ")",
+            "sample": f"{what}, whole path on {small.T} of {cfg.T} tokens of {cfg.name}, each stage's best of "
+                      f"{len(totals)} passes ({total:.3f} s: " + ", ".join(f"{k} {v:.3f}" for k, v in t.items()) +
+                      f"; whole passes took {min(totals):.3f} to {max(totals):.3f} s, median "
+                      f"{sorted(totals)[len(totals) // 2]:.3f})",
             "arrival_us_per_row": round(t["arrival"] * 1e6 / small.pairs, 4)}
 
 
