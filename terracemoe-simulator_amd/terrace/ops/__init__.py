@@ -104,16 +104,18 @@ def _require():
 def _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local):
     """Same refusals as the reference binding (terrace/ops/csrc/terrace_ops.cpp:123-144),
     minus its NPU-only limits (63 slots, 32-byte rows)."""
-    if rx.dim() != 2 or rslot.dim() != 2 or rgate.dim() != 2:
+    if (rx is not None and rx.dim() != 2) or rslot.dim() != 2 or rgate.dim() != 2:
         raise RuntimeError("terrace::k1_arrival: rx/rslot/rgate must be 2-D")
     if rslot.dtype != torch.int64:
         raise RuntimeError("terrace::k1_arrival: rslot must be int64 (quota wire format)")
-    if rgate.dtype != rx.dtype and rx.dtype != torch.uint8:
+    if rx is not None and rgate.dtype != rx.dtype and rx.dtype != torch.uint8:
         raise RuntimeError("terrace::k1_arrival: rgate dtype must equal rx dtype (the gate plane is "
                            "allocated from the payload)")
-    if not (rslot.shape[1] == quota and rgate.shape[1] == quota and rslot.shape[0] == rx.shape[0]
-            and rgate.shape[0] == rx.shape[0]):
-        raise RuntimeError(f"terrace::k1_arrival: geometry mismatch (rx {tuple(rx.shape)}, rslot "
+    n_rows = rslot.shape[0] if rx is None else rx.shape[0]
+    if not (rslot.shape[1] == quota and rgate.shape[1] == quota and rslot.shape[0] == n_rows
+            and rgate.shape[0] == n_rows):
+        raise RuntimeError(f"terrace::k1_arrival: geometry mismatch (rx "
+                           f"{None if rx is None else tuple(rx.shape)}, rslot "
                            f"{tuple(rslot.shape)}, rgate {tuple(rgate.shape)}, quota {quota})")
     if not (quota > 0 and epr > 0 and rpn > 0 and 0 <= my_local < rpn):
         raise RuntimeError("terrace::k1_arrival: bad geometry scalars")
@@ -121,16 +123,24 @@ def _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local):
         raise RuntimeError(f"terrace::k1_arrival: unsupported gate dtype {rgate.dtype}")
 
 
-def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=False, status_out=None):
-    """(send_buf, gate_pairs, r_idx, slot_idx, i_send[, pair_pos]) -- one library call."""
+def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=False, status_out=None,
+                   workspace_out=None):
+    """(send_buf, gate_pairs, r_idx, slot_idx, i_send[, pair_pos]) -- one library call.
+
+    ``rx`` None: the index planes only (``send_buf`` is None); the workspace, which then holds what
+    :func:`k1_arrival_move` needs, is appended to the list ``workspace_out``."""
     _require()
     _hip.need_device(rx, rslot, rgate)
     _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local)
-    rx, rslot, rgate = rx.contiguous(), rslot.contiguous(), rgate.contiguous()
-    dev = rx.device
-    R, H = rx.shape
+    rslot, rgate = rslot.contiguous(), rgate.contiguous()
+    dev = rslot.device
+    R = rslot.shape[0]
     P = R * quota
-    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev)
+    send_buf, row_bytes = None, 0
+    if rx is not None:
+        rx = rx.contiguous()
+        row_bytes = rx.shape[1] * rx.element_size()
+        send_buf = torch.empty((P, rx.shape[1]), dtype=rx.dtype, device=dev)
     gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
     r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
@@ -138,10 +148,12 @@ def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=
     pair_pos = torch.empty((P,), dtype=torch.int64, device=dev) if want_pair_pos else None
     st = status_out if status_out is not None else _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
-    _hip.call("terrace_k1_arrival", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, H * rx.element_size(),
+    _hip.call("terrace_k1_arrival", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, row_bytes,
               rgate.element_size(), quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(gate_pairs),
               _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(st),
               _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    if workspace_out is not None:
+        workspace_out.append(ws)
     out = (send_buf, gate_pairs, r_idx, slot_idx, i_send)
     return out + (pair_pos,) if want_pair_pos else out
 
@@ -149,13 +161,13 @@ def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=
 def _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
     """Refusals of terrace/ops/k2_ref.py:87-108 (same exception classes), minus the id-range
     read-back (reported through the status words instead) and the 63-slot mask bound."""
-    if expert_idx.dim() != 2 or hidden.dim() != 2 or gates.dim() != 2:
+    if expert_idx.dim() != 2 or (hidden is not None and hidden.dim() != 2) or gates.dim() != 2:
         raise ValueError("k2_pack: hidden/expert_idx/gates must be 2-D")
     T, k = expert_idx.shape
-    if hidden.shape[0] != T or gates.shape != expert_idx.shape:
-        raise ValueError(f"k2_pack: geometry mismatch (hidden {tuple(hidden.shape)}, expert_idx "
-                         f"{tuple(expert_idx.shape)}, gates {tuple(gates.shape)})")
-    if gates.dtype != hidden.dtype and hidden.dtype != torch.uint8:
+    if (hidden is not None and hidden.shape[0] != T) or gates.shape != expert_idx.shape:
+        raise ValueError(f"k2_pack: geometry mismatch (hidden {None if hidden is None else tuple(hidden.shape)}, "
+                         f"expert_idx {tuple(expert_idx.shape)}, gates {tuple(gates.shape)})")
+    if hidden is not None and gates.dtype != hidden.dtype and hidden.dtype != torch.uint8:
         raise RuntimeError(f"k2_pack: gates dtype {gates.dtype} != hidden dtype {hidden.dtype} -- the gate "
                            f"plane derives from the payload; cast at the caller")
     if gates.element_size() not in (2, 4):
@@ -169,36 +181,43 @@ def _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
                          f"groups_m={groups_m} not divisible")
 
 
+def _k2_extras(T, k, n_nodes, groups_m, gate_dtype, dev):
+    """The send side's optional planes: what plan_ta2a returns beside u_src, and the combine's per-token tables."""
+    i64 = dict(dtype=torch.int64, device=dev)
+    return {"u_node": torch.empty((T * groups_m,), **i64), "inverse": torch.empty((T * k,), **i64),
+            "node_offsets": torch.empty((n_nodes,), **i64), "pair_table": torch.empty((T, k), **i64),
+            "sort_order": torch.empty((T, k), **i64), "token_rows": torch.empty((T, groups_m), **i64),
+            "gate_sorted": torch.empty((T, k), dtype=gate_dtype, device=dev)}
+
+
 def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=False, status_out=None):
     """(payload, mask, gate_rows, u_src, node_counts) and, with ``extras``, a dict holding
     u_node, inverse, node_offsets, pair_table, sort_order, token_rows, gate_sorted and the
-    status words."""
+    status words.
+
+    ``hidden`` None: the index planes only (``payload`` is None); ``extras["workspace"]`` then
+    holds what :func:`k2_pack_move` needs."""
     _require()
     _hip.need_device(hidden, expert_idx, gates)
     _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
-    hidden, expert_idx, gates = hidden.contiguous(), expert_idx.contiguous(), gates.contiguous()
+    expert_idx, gates = expert_idx.contiguous(), gates.contiguous()
     dev = expert_idx.device
     T, k = expert_idx.shape
-    H = hidden.shape[1]
     S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
-    payload = torch.empty((S, H), dtype=hidden.dtype, device=dev)
+    payload, row_bytes = None, 0
+    if hidden is not None:
+        hidden = hidden.contiguous()
+        row_bytes = hidden.shape[1] * hidden.element_size()
+        payload = torch.empty((S, hidden.shape[1]), dtype=hidden.dtype, device=dev)
     mask = torch.empty((S, q), dtype=torch.int64, device=dev)
     gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
     u_src = torch.empty((S,), dtype=torch.int64, device=dev)
     node_counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
-    ex = {}
-    if extras:
-        ex = {"u_node": torch.empty((S,), dtype=torch.int64, device=dev),
-              "inverse": torch.empty((T * k,), dtype=torch.int64, device=dev),
-              "node_offsets": torch.empty((n_nodes,), dtype=torch.int64, device=dev),
-              "pair_table": torch.empty((T, k), dtype=torch.int64, device=dev),
-              "sort_order": torch.empty((T, k), dtype=torch.int64, device=dev),
-              "token_rows": torch.empty((T, groups_m), dtype=torch.int64, device=dev),
-              "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
+    ex = _k2_extras(T, k, n_nodes, groups_m, gates.dtype, dev) if extras else {}
     st = status_out if status_out is not None else _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
     _hip.call("terrace_k2_pack", _hip.ptr(hidden), _hip.ptr(expert_idx), _hip.ptr(gates), T,
-              H * hidden.element_size(), gates.element_size(), k, world, n_experts, rpn, groups_m,
+              row_bytes, gates.element_size(), k, world, n_experts, rpn, groups_m,
               _hip.ptr(payload), _hip.ptr(mask), _hip.ptr(gate_rows), _hip.ptr(u_src), _hip.ptr(node_counts),
               _hip.ptr(ex.get("u_node")), _hip.ptr(ex.get("inverse")), _hip.ptr(ex.get("node_offsets")),
               _hip.ptr(ex.get("pair_table")), _hip.ptr(ex.get("sort_order")), _hip.ptr(ex.get("token_rows")),
@@ -206,6 +225,8 @@ def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extr
     out = (payload, mask, gate_rows, u_src, node_counts)
     if extras:
         ex["status"] = st
+        if hidden is None:
+            ex["workspace"] = ws
         return out, ex
     return out
 
@@ -233,13 +254,7 @@ def k2_pack_wire(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
     wire = torch.empty((S, W), dtype=torch.int64, device=dev)
     u_src = torch.empty((S,), dtype=torch.int64, device=dev)
     node_counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
-    ex = {"u_node": torch.empty((S,), dtype=torch.int64, device=dev),
-          "inverse": torch.empty((T * k,), dtype=torch.int64, device=dev),
-          "node_offsets": torch.empty((n_nodes,), dtype=torch.int64, device=dev),
-          "pair_table": torch.empty((T, k), dtype=torch.int64, device=dev),
-          "sort_order": torch.empty((T, k), dtype=torch.int64, device=dev),
-          "token_rows": torch.empty((T, groups_m), dtype=torch.int64, device=dev),
-          "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
+    ex = _k2_extras(T, k, n_nodes, groups_m, gates.dtype, dev)
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
     _hip.call("terrace_k2_pack_wire", _hip.ptr(hidden), _hip.ptr(expert_idx), _hip.ptr(gates), T,
@@ -385,41 +400,8 @@ def k2_pack_index(expert_idx, gates, world, n_experts, rpn, groups_m):
     """First phase of :func:`k2_pack_raw`: every index plane, no rows.  Returns
     ((mask, gate_rows, u_src, node_counts), extras) with ``extras["workspace"]`` holding what
     :func:`k2_pack_move` needs to move the rows later."""
-    _require()
-    _hip.need_device(expert_idx, gates)
-    if expert_idx.dim() != 2 or gates.shape != expert_idx.shape:
-        raise ValueError("k2_pack: expert_idx/gates must be 2-D and of one shape")
-    if expert_idx.dtype != torch.int64:
-        raise RuntimeError("k2_pack: expert_idx must be int64")
-    if gates.element_size() not in (2, 4):
-        raise RuntimeError(f"k2_pack: unsupported gate dtype {gates.dtype}")
-    if world <= 0 or rpn <= 0 or groups_m <= 0 or n_experts <= 0:
-        raise ValueError("k2_pack: bad geometry scalars")
-    T, k = expert_idx.shape
-    if world % rpn or n_experts % world or k % groups_m:
-        raise ValueError(f"k2_pack: world={world} rpn={rpn} n_experts={n_experts} k={k} "
-                         f"groups_m={groups_m} not divisible")
-    expert_idx, gates = expert_idx.contiguous(), gates.contiguous()
-    dev = expert_idx.device
-    S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
-    i64 = dict(dtype=torch.int64, device=dev)
-    mask = torch.empty((S, q), **i64)
-    gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
-    u_src = torch.empty((S,), **i64)
-    node_counts = torch.empty((n_nodes,), **i64)
-    ex = {"u_node": torch.empty((S,), **i64), "inverse": torch.empty((T * k,), **i64),
-          "node_offsets": torch.empty((n_nodes,), **i64), "pair_table": torch.empty((T, k), **i64),
-          "sort_order": torch.empty((T, k), **i64), "token_rows": torch.empty((T, groups_m), **i64),
-          "gate_sorted": torch.empty((T, k), dtype=gates.dtype, device=dev)}
-    st = _hip.new_status(dev)
-    ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
-    _hip.call("terrace_k2_pack", None, _hip.ptr(expert_idx), _hip.ptr(gates), T, 0, gates.element_size(), k,
-              world, n_experts, rpn, groups_m, None, _hip.ptr(mask), _hip.ptr(gate_rows), _hip.ptr(u_src),
-              _hip.ptr(node_counts), _hip.ptr(ex["u_node"]), _hip.ptr(ex["inverse"]), _hip.ptr(ex["node_offsets"]),
-              _hip.ptr(ex["pair_table"]), _hip.ptr(ex["sort_order"]), _hip.ptr(ex["token_rows"]),
-              _hip.ptr(ex["gate_sorted"]), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
-    ex["status"], ex["workspace"] = st, ws
-    return (mask, gate_rows, u_src, node_counts), ex
+    out, ex = k2_pack_raw(None, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+    return out[1:], ex
 
 
 def k2_pack_move(hidden, workspace, k, world, rpn, groups_m):
@@ -438,30 +420,9 @@ def k2_pack_move(hidden, workspace, k, world, rpn, groups_m):
 
 def k1_arrival_index(rslot, rgate, quota, epr, rpn, my_local=0):
     """First phase of :func:`k1_arrival_raw`: (gate_pairs, r_idx, slot_idx, i_send, pair_pos, workspace)."""
-    _require()
-    _hip.need_device(rslot, rgate)
-    if rslot.dim() != 2 or rgate.dim() != 2 or rslot.shape != rgate.shape or rslot.shape[1] != quota:
-        raise RuntimeError(f"k1_arrival: rslot {tuple(rslot.shape)} / rgate {tuple(rgate.shape)} must be [R, {quota}]")
-    if rslot.dtype != torch.int64:
-        raise RuntimeError("k1_arrival: rslot must be int64")
-    if rgate.element_size() not in (2, 4):
-        raise RuntimeError(f"k1_arrival: unsupported gate dtype {rgate.dtype}")
-    if quota <= 0 or epr <= 0 or rpn <= 0 or not 0 <= my_local < rpn:
-        raise RuntimeError("k1_arrival: bad geometry scalars")
-    rslot, rgate = rslot.contiguous(), rgate.contiguous()
-    dev = rslot.device
-    R = rslot.shape[0]
-    P = R * quota
-    i64 = dict(dtype=torch.int64, device=dev)
-    gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
-    r_idx, slot_idx, pair_pos = torch.empty((P,), **i64), torch.empty((P,), **i64), torch.empty((P,), **i64)
-    i_send = torch.empty((rpn,), **i64)
-    st = _hip.new_status(dev)
-    ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
-    _hip.call("terrace_k1_arrival", None, _hip.ptr(rslot), _hip.ptr(rgate), R, 0, rgate.element_size(), quota, epr,
-              rpn, my_local, None, _hip.ptr(gate_pairs), _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send),
-              _hip.ptr(pair_pos), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
-    return gate_pairs, r_idx, slot_idx, i_send, pair_pos, ws
+    ws = []
+    out = k1_arrival_raw(None, rslot, rgate, quota, epr, rpn, my_local, want_pair_pos=True, workspace_out=ws)
+    return out[1:] + (ws[0],)
 
 
 def k1_arrival_move(rx, workspace, quota, rpn):
