@@ -293,3 +293,97 @@ def test_move_phases_refuse_bad_arguments():
     assert lib.terrace_k1_arrival_move(None, 0, 256, 2, 8, None, None, 0, s) == _hip.OK
     assert lib.terrace_regroup_move(None, 0, 256, 32, -1, None, None, 0, s) == _hip.OK
     torch.cuda.synchronize()
+
+
+def test_two_host_threads_on_two_streams_do_not_disturb_each_other():
+    """The library keeps no state between calls: two host threads, each on a stream of its own, running the
+    whole path on different inputs at the same time get bit for bit what they get one after the other."""
+    import threading
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    announce("two threads, two streams")
+    jobs = []
+    for name, T in (("c1", 3000), ("c4", 2500)):
+        cfg = configs.CONFIGS[name].scaled(T)
+        inp = configs.make_inputs(cfg)
+        e, g, _, _ = _route(cfg, inp)
+        jobs.append((cfg, inp["x"].to(DEV), e, g.to(cfg.gate_dtype)))
+
+    def run(job):
+        cfg, x, e, gates = job
+        st = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cfg.capacity(cfg.slots))
+        y = loopback_combine(st.permuted, st, out_dtype=cfg.out_dtype)
+        return st.permuted, st.place, st.tokens_per_expert, y
+
+    serial = [run(j) for j in jobs]
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                for _ in range(5):
+                    out = run(jobs[i])
+                torch.cuda.current_stream().synchronize()
+                results[i] = out
+        except Exception as exc:               # surfaced below: an exception in a thread is otherwise lost
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for want, got in zip(serial, results):
+        assert got is not None
+        for w, g_ in zip(want, got):
+            assert torch.equal(w, g_)
+
+
+@pytest.mark.parametrize("name", ["c2", "c4", "c5"])
+def test_the_whole_step_replays_as_one_hip_graph(name):
+    """Route, dispatch and combine launch kernels only (no allocation of their own, no memset, no host
+    synchronisation), so a step records into a HIP graph; every replay, with eager work and synchronisations
+    in between, must reproduce the eager result bit for bit."""
+    import terrace
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    cfg = configs.CONFIGS[name].scaled(2048)
+    announce("graph replay", cfg.name)
+    inp = configs.make_inputs(cfg)
+    logits, bias, x = inp["logits"].to(DEV), inp["bias"].to(DEV), inp["x"].to(DEV)
+    ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(DEV)
+    rcfg = terrace.TRouteConfig(cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups)
+    cap = cfg.capacity(cfg.slots)
+    fp8_hidden = cfg.hidden if cfg.fmt == "fp8" else None
+    first = loopback_dispatch(x, *terrace.t_route(logits, bias, rcfg, gate_affinity=ga, gates_dtype=cfg.gate_dtype)[:2],
+                              cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    ye = first.permuted.clone() if cfg.fmt != "fp8" else configs.quantise_fp8_rows(
+        torch.randn(first.permuted.shape[0], cfg.hidden, device=DEV))
+
+    def step():
+        e, g, _ = terrace.t_route(logits, bias, rcfg, gate_affinity=ga, gates_dtype=cfg.gate_dtype)
+        st = loopback_dispatch(x, e, g, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+        return loopback_combine(ye, st, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden), st.permuted
+
+    y_eager, p_eager = step()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_graph, p_graph = step()
+    for _ in range(3):
+        y_graph.zero_(), p_graph.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y_eager) and torch.equal(p_graph, p_eager)
+        y_again, _ = step()
+        torch.cuda.synchronize()
+        assert torch.equal(y_again, y_eager)
