@@ -222,6 +222,42 @@ def test_k2_pack_reference_geometries(literals, fmt, sort_rows):
                 assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("geom", [(8, 8, 64, 500, 4, 1), (16, 8, 192, 333, 8, 2), (16, 8, 1024, 700, 8, 2),
+                                  (64, 8, 1024, 2100, 8, 4)], ids=lambda g: "w%dr%dE%dT%dk%dM%d" % g)
+def test_nodes_wider_than_the_reference_mask_bound(geom):
+    """The reference stops at 63 expert slots per node because its general branch ships them as one int64 bitmask
+    (terrace/ops/k2_ref.py:95-108, csrc/terrace_ops.cpp:123-144).  The quota wire format has no such limit and
+    this build lifts it there: the send side, the arrival chain and the regroup on nodes of 64 to 512 slots,
+    against the oracle's pieces (plan + row gather + quota wire planes), which carry no bound of their own."""
+    import terrace.ops as tops
+    world, rpn, E, T, k, M = geom
+    epr, n_nodes, q = E // world, world // rpn, k // M
+    slots = epr * rpn
+    assert slots > 63
+    announce("wide nodes", geom, slots)
+    e = equal_quota_routing(T, k, E, n_nodes, M, 77, False)
+    g = torch.Generator().manual_seed(78)
+    hidden = rows_of(torch.randn(T, 96, generator=g), "bf16")
+    gates = rows_of(torch.rand(T, k, generator=g), "bf16")
+    with pytest.raises(ValueError, match="slots"):
+        orc.k2_pack(to_np(hidden), e, to_np(gates), world, E, rpn, M)        # the oracle keeps the reference's refusal
+    u_src, u_node, counts, inverse = orc.plan_ta2a(e, world, E, rpn, M)
+    payload = to_np(hidden)[u_src]
+    mask, gate_rows = orc.pack_quota_wire(e, to_np(gates), inverse, T * M, slots, q)
+    got, ex = tops.k2_pack_raw(hidden.to(DEV), torch.from_numpy(e).to(DEV), gates.to(DEV), world, E, rpn, M, extras=True)
+    for name, a, b in zip(("payload", "mask", "gate_rows", "u_src", "node_counts"), got, (payload, mask, gate_rows, u_src, counts)):
+        same(a, b, name)
+    same(ex["u_node"], u_node, "u_node"), same(ex["inverse"], inverse, "inverse")
+    assert ex["status"].tolist() == [0, T * M, 0, 0] and int(to_np(got[1]).max()) >= 63
+    send, gp, r_idx, s_idx, i_send = orc.k1_arrival(payload, mask, gate_rows, q, epr, rpn)
+    arr = tops.k1_arrival_raw(got[0], got[1], got[2], q, epr, rpn, 0)
+    for name, a, b in zip(("send_buf", "gate_pairs", "r_idx", "slot_idx", "i_send"), arr, (send, gp, r_idx, s_idx, i_send)):
+        same(a, b, name)
+    perm, order, tpe = orc.regroup(send, s_idx, slots)
+    rg = tops.regroup(arr[0], arr[3], slots)
+    same(rg[0], perm, "permuted"), same(rg[1], order, "order"), same(rg[2], tpe, "tokens_per_expert")
+
+
 def test_plan_and_wire_functions_match_oracle(literals):
     from terrace import ta2a
     from terrace.ta2a_fwd import _pack_quota_wire
