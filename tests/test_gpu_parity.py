@@ -164,6 +164,57 @@ def test_route_gates_in_the_payload_dtype(generic, dtype):
         terrace.t_route(aff, zero, cfg, gates_dtype=torch.float64)
 
 
+@pytest.mark.parametrize("generic", [False, True])
+def test_route_with_masked_experts(generic):
+    """A bias of -inf is how a caller switches an expert off.  With at least two live experts left in every
+    group nothing but the order (value descending, index ascending, -inf last) is involved: bit-exact against
+    the oracle, and no masked expert is ever picked while its group has q live ones."""
+    import terrace
+    announce("route masked", generic)
+    g = torch.Generator().manual_seed(21)
+    for (T, E, Ng, k, M) in [(1500, 256, 8, 8, 4), (700, 64, 8, 4, 2), (300, 128, 16, 8, 2)]:
+        gs, q = E // Ng, k // M
+        logits = torch.randn(T, E, generator=g)
+        bias = torch.randn(E, generator=g) * 0.1
+        dead = torch.zeros(E, dtype=torch.bool)
+        for grp in range(Ng):                                      # switch off all but q+1 .. gs experts of each group
+            n_dead = int(torch.randint(0, gs - q, (1,), generator=g))
+            dead[grp * gs + torch.randperm(gs, generator=g)[:n_dead]] = True
+        bias[dead] = -float("inf")
+        cfg = terrace.TRouteConfig(E, Ng, k, M)
+        e, gt, grp_idx = terrace.t_route(logits.to(DEV), bias.to(DEV), cfg, _force_generic=generic)
+        oe, og, ogrp = orc.t_route(logits.numpy(), bias.numpy(), E, Ng, k, M)
+        same(e, oe, "expert_idx"), same(grp_idx, ogrp, "group_idx"), same(gt, og, "gates")
+        assert not bool(dead.to(DEV)[e].any())
+
+
+@pytest.mark.parametrize("generic", [False, True])
+def test_route_contains_nan_scores(generic):
+    """NaN affinities mean a broken model, not a defined routing; what is promised is containment: every id
+    written is a valid expert (or, for group_idx, the no-group sentinel), clean tokens of the same batch are
+    routed as if the bad ones were not there, and nothing hangs."""
+    import terrace
+    announce("route nan", generic)
+    T, E, Ng, k, M = 512, 256, 8, 8, 4
+    g = torch.Generator().manual_seed(22)
+    logits = torch.randn(T, E, generator=g)
+    bad = torch.zeros(T, dtype=torch.bool)
+    bad[::7] = True
+    poisoned = logits.clone()
+    poisoned[bad, ::3] = float("nan")
+    poisoned[5 * 7] = float("nan")                                   # one token with nothing but NaN
+    zero = torch.zeros(E)
+    cfg = terrace.TRouteConfig(E, Ng, k, M)
+    e, gt, grp = terrace.t_route(poisoned.to(DEV), zero.to(DEV), cfg, _force_generic=generic)
+    torch.cuda.synchronize()
+    assert bool(((e >= 0) & (e < E)).all())
+    assert bool(((grp >= 0) & (grp < Ng) | (grp == 0x7FFFFFFF)).all())
+    oe, og, ogrp = orc.t_route(logits.numpy(), zero.numpy(), E, Ng, k, M)
+    ok = ~bad
+    assert np.array_equal(to_np(e)[ok.numpy()], oe[ok.numpy()]) and np.array_equal(to_np(gt)[ok.numpy()], og[ok.numpy()])
+    assert np.array_equal(to_np(grp)[ok.numpy()], ogrp[ok.numpy()])
+
+
 def test_expert_load_and_hist_and_argsort():
     import terrace
     from terrace.ta2a_fwd import _stable_argsort_small, fixed_hist
