@@ -173,32 +173,36 @@ TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, con
                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status,
                     void *workspace, size_t workspace_bytes, terrace_stream_t stream);
 
-/* out[i] = src[idx[i]] for i < n_out (row gather; idx < 0 writes a zero row). */
-TERRACE_API int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes,
-                        void *out, terrace_stream_t stream);
+/* Row ids a caller passes to the four entry points below are never turned into an address unchecked: an id
+ * outside [0, n_src) (resp. [0, n_dst), the table length) is a dead entry -- a zero row, a copy not made,
+ * no contribution, -1 -- exactly like a negative one.  (The reference's x[u_src] / index_add would raise.) */
 
-/* dst[pos[r*fan + f]] = src[r] for r < n_src, f < fan (pos < 0 skips that copy): a source row
- * is read once and written fan times.  The mover behind terrace_k2_pack (pos = token_rows)
+/* out[i] = src[idx[i]] for i < n_out (row gather over the n_src rows of src; a dead idx writes a zero row). */
+TERRACE_API int terrace_gather_rows(const void *src, int64_t n_src, const int64_t *idx, int64_t n_out,
+                                    int64_t row_bytes, void *out, terrace_stream_t stream);
+
+/* dst[pos[r*fan + f]] = src[r] for r < n_src, f < fan (a dead pos skips that copy; dst has n_dst rows): a
+ * source row is read once and written fan times.  The mover behind terrace_k2_pack (pos = token_rows)
  * and terrace_k1_arrival (pos = pair_pos); exposed so it can be driven and timed on its own. */
 TERRACE_API int terrace_scatter_rows(const void *src, const int64_t *pos, int64_t n_src, int fan,
-                                     int64_t row_bytes, void *dst, terrace_stream_t stream);
+                                     int64_t row_bytes, void *dst, int64_t n_dst, terrace_stream_t stream);
 
-/* out[i] = table[idx[i]] over int64 planes; idx < 0 or table value < 0 gives -1. */
-TERRACE_API int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out,
-                        terrace_stream_t stream);
+/* out[i] = table[idx[i]] over int64 planes (table has n_table entries); a dead idx gives -1. */
+TERRACE_API int terrace_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n,
+                                    int64_t *out, terrace_stream_t stream);
 
 /* out[i] = outer[inner[idx[i]]], -1 propagating at either level (one launch for the two
  * look-ups that turn a token's Hop-A pair ids into places of the expert-order buffer). */
-TERRACE_API int terrace_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n,
-                                     int64_t *out, terrace_stream_t stream);
+TERRACE_API int terrace_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *inner, int64_t n_inner,
+                                     const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream);
 
 /* Gate-weighted combine (terrace/ta2a_fwd.py:658-670; one level: terrace/ep_dist.py:121-122):
- *   out[i,:] = sum_{j<fan} w[i,j] * decode(src[idx[i,j],:])      (idx < 0 contributes nothing)
+ *   out[i,:] = sum_{j<fan} w[i,j] * decode(src[idx[i,j],:])      (idx outside [0, n_src) contributes nothing)
  * accumulated in fp32 as acc = fl(acc + fl(w*x)) for j = 0..fan-1, rounded once to out_dtype.
  * src rows are src_dtype (F32, BF16, F16 or FP8_E4M3_B128 with `hidden` elements per row),
  * weights [n_out,fan] are w_dtype (F32, BF16, F16) or NULL (all ones), idx is [n_out,fan] i64,
  * out is [n_out,hidden] of out_dtype (F32, BF16 or F16). */
-TERRACE_API int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const void *weights,
+TERRACE_API int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
                     int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
                     terrace_stream_t stream);
 

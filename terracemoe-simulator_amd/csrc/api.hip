@@ -3,11 +3,12 @@
 
 namespace terrace {
 int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
-int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
-                   int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
-int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
-int launch_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
-                        hipStream_t s);
+int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
+                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
+int launch_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n, int64_t *out,
+                       hipStream_t s);
+int launch_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *inner, int64_t n_inner,
+                        const int64_t *idx, int64_t n, int64_t *out, hipStream_t s);
 int launch_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,
                        int64_t n_rows, int64_t row_bytes, void *out, hipStream_t s);
 int launch_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, void *a, int64_t a_bytes, void *b,
@@ -15,9 +16,10 @@ int launch_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, 
 int launch_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send, hipStream_t s);
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
-                        hipStream_t s);
+                        int64_t n_dst, hipStream_t s);
 template <typename I>
-int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, int64_t n_src,
+                       hipStream_t s);
 int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
                 int k, int M, int pool, int mode, int64_t *expert_idx, void *gates, int gate_dtype,
                 int64_t *group_idx, int force_generic, hipStream_t s);
@@ -242,39 +244,42 @@ int terrace_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int 
                             (hipStream_t)stream);
 }
 
-int terrace_gather_rows(const void *src, const int64_t *idx, int64_t n_out, int64_t row_bytes, void *out,
-                        terrace_stream_t stream) {
-    if (n_out < 0 || row_bytes < 0) return TERRACE_EINVAL;
-    if (n_out && row_bytes && (!src || !idx || !out)) return TERRACE_EINVAL;
-    return launch_gather_rows<int64_t>(src, out, idx, n_out, row_bytes, (hipStream_t)stream);
+int terrace_gather_rows(const void *src, int64_t n_src, const int64_t *idx, int64_t n_out, int64_t row_bytes,
+                        void *out, terrace_stream_t stream) {
+    if (n_out < 0 || row_bytes < 0 || n_src < 0) return TERRACE_EINVAL;
+    if (n_out && row_bytes && ((!src && n_src) || !idx || !out)) return TERRACE_EINVAL;
+    return launch_gather_rows<int64_t>(src, out, idx, n_out, row_bytes, n_src, (hipStream_t)stream);
 }
 
 int terrace_scatter_rows(const void *src, const int64_t *pos, int64_t n_src, int fan, int64_t row_bytes, void *dst,
-                         terrace_stream_t stream) {
-    if (n_src < 0 || fan <= 0 || row_bytes < 0) return TERRACE_EINVAL;
-    if (n_src && row_bytes && (!src || !pos || !dst)) return TERRACE_EINVAL;
-    return launch_scatter_rows<int64_t>(src, dst, pos, n_src, fan, row_bytes, (hipStream_t)stream);
+                         int64_t n_dst, terrace_stream_t stream) {
+    if (n_src < 0 || fan <= 0 || row_bytes < 0 || n_dst < 0) return TERRACE_EINVAL;
+    if (n_src && row_bytes && (!src || !pos || (!dst && n_dst))) return TERRACE_EINVAL;
+    return launch_scatter_rows<int64_t>(src, dst, pos, n_src, fan, row_bytes, n_dst, (hipStream_t)stream);
 }
 
-int terrace_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream) {
-    if (n < 0 || (n && (!table || !idx || !out))) return TERRACE_EINVAL;
-    return launch_index_chain(table, idx, n, out, (hipStream_t)stream);
+int terrace_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n, int64_t *out,
+                        terrace_stream_t stream) {
+    if (n < 0 || n_table < 0 || (n && ((!table && n_table) || !idx || !out))) return TERRACE_EINVAL;
+    return launch_index_chain(table, n_table, idx, n, out, (hipStream_t)stream);
 }
 
-int terrace_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
-                         terrace_stream_t stream) {
-    if (n < 0 || (n && (!outer || !inner || !idx || !out))) return TERRACE_EINVAL;
-    return launch_index_chain2(outer, inner, idx, n, out, (hipStream_t)stream);
+int terrace_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *inner, int64_t n_inner,
+                         const int64_t *idx, int64_t n, int64_t *out, terrace_stream_t stream) {
+    if (n < 0 || n_outer < 0 || n_inner < 0) return TERRACE_EINVAL;
+    if (n && ((!outer && n_outer) || (!inner && n_inner) || !idx || !out)) return TERRACE_EINVAL;
+    return launch_index_chain2(outer, n_outer, inner, n_inner, idx, n, out, (hipStream_t)stream);
 }
 
-int terrace_combine(const void *src, int src_dtype, const int64_t *idx, const void *weights, int w_dtype,
-                    int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, terrace_stream_t stream) {
-    if (n_out < 0 || fan <= 0 || hidden < 0) return TERRACE_EINVAL;
+int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
+                    int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
+                    terrace_stream_t stream) {
+    if (n_out < 0 || fan <= 0 || hidden < 0 || n_src < 0) return TERRACE_EINVAL;
     if (src_dtype < TERRACE_F32 || src_dtype > TERRACE_FP8_E4M3_B128 || !float_dtype(out_dtype)) return TERRACE_EINVAL;
     if (weights && !float_dtype(w_dtype)) return TERRACE_EINVAL;
     if (src_dtype == TERRACE_FP8_E4M3_B128 && hidden % 128) return TERRACE_EINVAL;
-    if (n_out && hidden && (!src || !idx || !out)) return TERRACE_EINVAL;
-    return launch_combine(src, src_dtype, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
+    if (n_out && hidden && ((!src && n_src) || !idx || !out)) return TERRACE_EINVAL;
+    return launch_combine(src, n_src, src_dtype, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
                           (hipStream_t)stream);
 }
 

@@ -318,7 +318,7 @@ int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gate
 #undef TERRACE_PLACE
     int rc = check_launch();
     if (rc != TERRACE_OK || !hidden) return rc;
-    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
+    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
 }
 
 }  // namespace terrace

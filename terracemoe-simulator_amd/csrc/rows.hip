@@ -49,13 +49,20 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V
     }
 }
 
+// Row ids a caller hands in are never trusted with an address: an id is used only if it lies in [0, bound),
+// which one unsigned compare decides ((uint64_t)id < (uint64_t)bound is false for negative ids too).  An id
+// outside is a dead entry -- a zero row for a gather, no contribution for the combine, a copy not made for a
+// scatter.  The stage operators bound the planes their own index kernels wrote all the same.
+__device__ __forceinline__ bool row_in(int64_t id, int64_t bound) { return (uint64_t)id < (uint64_t)bound; }
+
 // ---------------------------------------------------------------------------------------------
 // scatter: one read, fan writes
 // ---------------------------------------------------------------------------------------------
 template <typename V, int VPT, typename I>
 __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restrict__ src, V *__restrict__ dst,
                                                               const I *__restrict__ pos, int64_t n_src,
-                                                              int fan, int64_t row_vecs, int tpr_log2) {
+                                                              int fan, int64_t row_vecs, int tpr_log2,
+                                                              int64_t n_dst) {
     const int tpr = 1 << tpr_log2;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
     const int lane = threadIdx.x & (tpr - 1);
@@ -72,7 +79,7 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restric
         }
         for (int f = 0; f < fan; ++f) {
             const int64_t d = p[f];
-            if (d < 0) continue;
+            if (!row_in(d, n_dst)) continue;
             V *o = dst + d * row_vecs;
 #pragma unroll
             for (int u = 0; u < VPT; ++u) {
@@ -89,7 +96,7 @@ __global__ __launch_bounds__(kBlock) void scatter_rows_kernel(const V *__restric
 template <typename V, int VPT, typename I>
 __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict__ src, V *__restrict__ out,
                                                              const I *__restrict__ idx, int64_t n_out,
-                                                             int64_t row_vecs, int tpr_log2) {
+                                                             int64_t row_vecs, int tpr_log2, int64_t n_src) {
     const int tpr = 1 << tpr_log2;
     const int sub = __builtin_amdgcn_readfirstlane(threadIdx.x >> tpr_log2);
     const int lane = threadIdx.x & (tpr - 1);
@@ -97,7 +104,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const V *__restrict
     if (row >= n_out) return;
     const int64_t from = (int64_t)idx[row];
     V *o = out + row * row_vecs;
-    if (from < 0) {
+    if (!row_in(from, n_src)) {
         for (int64_t i = lane; i < row_vecs; i += tpr) st_stream(o + i, zero_of<V>());
         return;
     }
@@ -145,7 +152,8 @@ __device__ __forceinline__ uint32_t xcd_swizzle(uint32_t id, uint32_t run, uint3
 template <typename I>
 __global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__restrict__ src, u32x4 *__restrict__ out,
                                                                  const I *__restrict__ idx, int64_t total_vecs,
-                                                                 int64_t row_vecs, int head, uint32_t run) {
+                                                                 int64_t row_vecs, int head, uint32_t run,
+                                                                 int64_t n_src) {
     const uint32_t chunk = xcd_swizzle(blockIdx.x, run, gridDim.x);
     const int64_t first = (int64_t)chunk * kWave - head;                 // wave-uniform, may be < 0 in chunk 0
     const int64_t g = first + threadIdx.x;
@@ -165,7 +173,7 @@ __global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__
     }
     const int64_t from = (int64_t)idx[row];
     u32x4 v = zero_of<u32x4>();
-    if (from >= 0) v = ld_stream(src + from * row_vecs + i);
+    if (row_in(from, n_src)) v = ld_stream(src + from * row_vecs + i);
     st_stream(out + g, v);
 }
 
@@ -173,13 +181,13 @@ __global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__
 template <typename I>
 __global__ __launch_bounds__(kWave) void gather_rows_sliced_kernel(const u32x4 *__restrict__ src,
                                                                    u32x4 *__restrict__ out, const I *__restrict__ idx,
-                                                                   int64_t row_vecs, uint32_t slices) {
+                                                                   int64_t row_vecs, uint32_t slices, int64_t n_src) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
     const int64_t i = (int64_t)slice * kWave + threadIdx.x;
     const int64_t from = (int64_t)idx[row];
     u32x4 v = zero_of<u32x4>();
-    if (from >= 0) v = ld_stream(src + from * row_vecs + i);
+    if (row_in(from, n_src)) v = ld_stream(src + from * row_vecs + i);
     st_stream(out + (int64_t)row * row_vecs + i, v);
 }
 
@@ -187,7 +195,8 @@ __global__ __launch_bounds__(kWave) void gather_rows_sliced_kernel(const u32x4 *
 template <typename I>
 __global__ __launch_bounds__(kWave) void scatter_rows_sliced_kernel(const u32x4 *__restrict__ src,
                                                                     u32x4 *__restrict__ dst, const I *__restrict__ pos,
-                                                                    int fan, int64_t row_vecs, uint32_t slices) {
+                                                                    int fan, int64_t row_vecs, uint32_t slices,
+                                                                    int64_t n_dst) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
     const int64_t i = (int64_t)slice * kWave + threadIdx.x;
@@ -195,7 +204,7 @@ __global__ __launch_bounds__(kWave) void scatter_rows_sliced_kernel(const u32x4 
     const I *p = pos + (int64_t)row * fan;
     for (int f = 0; f < fan; ++f) {
         const int64_t d = p[f];
-        if (d >= 0) st_stream(dst + d * row_vecs + i, v);
+        if (row_in(d, n_dst)) st_stream(dst + d * row_vecs + i, v);
     }
 }
 
@@ -206,7 +215,7 @@ template <typename I>
 __global__ __launch_bounds__(kWave) void scatter_rows_aligned_kernel(const u32x4 *__restrict__ src,
                                                                      u32x4 *__restrict__ dst, const I *__restrict__ pos,
                                                                      int fan, int64_t row_vecs, uint32_t chunks,
-                                                                     int head) {
+                                                                     int head, int64_t n_dst) {
     const uint32_t id = xcd_swizzle(blockIdx.x, chunks, gridDim.x);     // a row's chunks re-read each other's lines
     const uint32_t row = id / chunks;
     const int64_t c = id - row * chunks;
@@ -214,7 +223,7 @@ __global__ __launch_bounds__(kWave) void scatter_rows_aligned_kernel(const u32x4
     const I *p = pos + (int64_t)row * fan;
     for (int f = 0; f < fan; ++f) {
         const int64_t d = p[f];
-        if (d < 0) continue;
+        if (!row_in(d, n_dst)) continue;
         const int64_t base = d * row_vecs;
         const int64_t i = c * kWave - ((base + head) & (kWave - 1)) + threadIdx.x;
         if (i >= 0 && i < row_vecs) st_stream(dst + base + i, s[i]);
@@ -339,7 +348,7 @@ __device__ __forceinline__ float uniform_weight(const void *w, int64_t i) {
 template <int SRC, int WD, int B>
 __device__ __forceinline__ void combine_batch(float *acc, const uint8_t *__restrict__ src, int64_t src_row_bytes,
                                               const int64_t *__restrict__ idx_at, const void *__restrict__ w,
-                                              int64_t w_at, int64_t hidden, int64_t c) {
+                                              int64_t w_at, int64_t hidden, int64_t c, int64_t n_src) {
     constexpr int N = Chunk<SRC>::N;
     int64_t from[B];
     float wj[B];
@@ -353,14 +362,14 @@ __device__ __forceinline__ void combine_batch(float *acc, const uint8_t *__restr
     float sc[B];
 #pragma unroll
     for (int jj = 0; jj < B; ++jj) {
-        const uint8_t *s = src + (from[jj] < 0 ? 0 : from[jj]) * src_row_bytes;
+        const uint8_t *s = src + (row_in(from[jj], n_src) ? from[jj] : 0) * src_row_bytes;
         raw[jj] = ld_stream((const u32x4 *)s + c);
         if constexpr (SRC == TERRACE_FP8_E4M3_B128) sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
         else sc[jj] = 1.0f;
     }
 #pragma unroll
     for (int jj = 0; jj < B; ++jj) {
-        const bool live = from[jj] >= 0;
+        const bool live = row_in(from[jj], n_src);
         const u32x4 r = live ? raw[jj] : zero_of<u32x4>();
         const float scale = live ? sc[jj] : 0.0f, weight = live ? wj[jj] : 0.0f;
         float f[N];
@@ -379,22 +388,22 @@ template <int SRC, int OUT, int WD>
 __device__ __forceinline__ void combine_row_chunk(const uint8_t *__restrict__ src, int64_t src_row_bytes,
                                                   const int64_t *__restrict__ idx_row, const void *__restrict__ w,
                                                   int64_t w_base, int fan, int64_t hidden, int64_t c,
-                                                  uint8_t *__restrict__ out_row) {
+                                                  uint8_t *__restrict__ out_row, int64_t n_src) {
     constexpr int N = Chunk<SRC>::N;
     float acc[N];
 #pragma unroll
     for (int i = 0; i < N; ++i) acc[i] = 0.0f;
     int j = 0;
-    for (; j + 8 <= fan; j += 8) combine_batch<SRC, WD, 8>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+    for (; j + 8 <= fan; j += 8) combine_batch<SRC, WD, 8>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c, n_src);
     if (j + 4 <= fan) {
-        combine_batch<SRC, WD, 4>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+        combine_batch<SRC, WD, 4>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c, n_src);
         j += 4;
     }
     if (j + 2 <= fan) {
-        combine_batch<SRC, WD, 2>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+        combine_batch<SRC, WD, 2>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c, n_src);
         j += 2;
     }
-    if (j < fan) combine_batch<SRC, WD, 1>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c);
+    if (j < fan) combine_batch<SRC, WD, 1>(acc, src, src_row_bytes, idx_row + j, w, w_base + j, hidden, c, n_src);
     store_chunk<OUT, N>(out_row, c * N, acc);
 }
 
@@ -403,7 +412,7 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restri
                                                          const int64_t *__restrict__ idx, const void *__restrict__ w,
                                                          int w_dtype, int64_t n_out, int fan, int64_t hidden,
                                                          uint8_t *__restrict__ out, int64_t out_row_bytes,
-                                                         int slices, uint32_t run) {
+                                                         int slices, uint32_t run, int64_t n_src) {
     constexpr int N = Chunk<SRC>::N;
     const uint32_t id = xcd_swizzle(blockIdx.x, run, gridDim.x);
     const int64_t row = id / slices;
@@ -412,7 +421,7 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restri
     const int64_t *idx_row = idx + row * fan;
     uint8_t *out_row = out + row * out_row_bytes;
 #define TERRACE_COMBINE_BODY(WD) \
-    combine_row_chunk<SRC, OUT, WD>(src, src_row_bytes, idx_row, w, row * fan, fan, hidden, c, out_row)
+    combine_row_chunk<SRC, OUT, WD>(src, src_row_bytes, idx_row, w, row * fan, fan, hidden, c, out_row, n_src)
     if (!w) TERRACE_COMBINE_BODY(kWNone);
     else if (w_dtype == TERRACE_F32) TERRACE_COMBINE_BODY(TERRACE_F32);
     else if (w_dtype == TERRACE_BF16) TERRACE_COMBINE_BODY(TERRACE_BF16);
@@ -440,13 +449,13 @@ __global__ __launch_bounds__(kBlock) void combine_elem_kernel(const uint8_t *__r
                                                               int64_t src_row_bytes, const int64_t *__restrict__ idx,
                                                               const void *__restrict__ w, int w_dtype, int64_t n_out,
                                                               int fan, int64_t hidden, uint8_t *__restrict__ out,
-                                                              int out_dtype) {
+                                                              int out_dtype, int64_t n_src) {
     for (int64_t row = blockIdx.x; row < n_out; row += gridDim.x) {
         for (int64_t e = threadIdx.x; e < hidden; e += kBlock) {
             float acc = 0.0f;
             for (int j = 0; j < fan; ++j) {
                 const int64_t from = idx[row * fan + j];
-                if (from < 0) continue;
+                if (!row_in(from, n_src)) continue;
                 float x = load_elem(src + from * src_row_bytes, src_dtype, e, hidden);
                 if (w) x = __fmul_rn(x, load_weight(w, w_dtype, row * fan + j));
                 acc = __fadd_rn(acc, x);
@@ -525,24 +534,24 @@ int launch_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows, 
     return launch_planes<false>(pl, (void *)packed, row_bytes, n_rows, s);
 }
 
-__global__ __launch_bounds__(kBlock) void index_chain_kernel(const int64_t *__restrict__ table,
+__global__ __launch_bounds__(kBlock) void index_chain_kernel(const int64_t *__restrict__ table, int64_t n_table,
                                                              const int64_t *__restrict__ idx, int64_t n,
                                                              int64_t *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     const int64_t a = idx[i];
-    out[i] = a < 0 ? -1 : table[a];
+    out[i] = row_in(a, n_table) ? table[a] : -1;
 }
 
-__global__ __launch_bounds__(kBlock) void index_chain2_kernel(const int64_t *__restrict__ outer,
-                                                              const int64_t *__restrict__ inner,
+__global__ __launch_bounds__(kBlock) void index_chain2_kernel(const int64_t *__restrict__ outer, int64_t n_outer,
+                                                              const int64_t *__restrict__ inner, int64_t n_inner,
                                                               const int64_t *__restrict__ idx, int64_t n,
                                                               int64_t *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     int64_t a = idx[i];
-    if (a >= 0) a = inner[a];
-    out[i] = a < 0 ? -1 : outer[a];
+    a = row_in(a, n_inner) ? inner[a] : -1;
+    out[i] = row_in(a, n_outer) ? outer[a] : -1;
 }
 
 __global__ void send_splits_kernel(const int64_t *__restrict__ node_counts, int world, int rpn, int my_local,
@@ -582,21 +591,21 @@ static int vec_bytes_for(int64_t row_bytes, const void *a, const void *b) {
 
 template <typename V, typename I>
 static void launch_scatter_t(const void *src, void *dst, const I *pos, int64_t n_src, int fan,
-                             int64_t row_vecs, hipStream_t s) {
+                             int64_t row_vecs, int64_t n_dst, hipStream_t s) {
     const int l = tpr_log2_for(row_vecs);
     const int rpi = kBlock >> l;
     const unsigned grid = grid_for(n_src, rpi);
     if (row_vecs > ((int64_t)2 << l))
-        scatter_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l, n_dst);
     else if (row_vecs > ((int64_t)1 << l))
-        scatter_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l, n_dst);
     else
-        scatter_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l);
+        scatter_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)dst, pos, n_src, fan, row_vecs, l, n_dst);
 }
 
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
-                        hipStream_t s) {
+                        int64_t n_dst, hipStream_t s) {
     if (n_src <= 0 || row_bytes <= 0 || fan <= 0) return TERRACE_OK;
     if (n_src > kMaxGridRows) return TERRACE_EINVAL;
     switch (vec_bytes_for(row_bytes, src, dst)) {
@@ -605,78 +614,85 @@ int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src,
             const int head = (int)(((uintptr_t)dst >> 4) & (kWave - 1));
             if (rv % kWave == 0 && head == 0 && n_src * (rv / kWave) <= kMaxBlocks) {
                 scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, 0, s>>>(
-                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)(rv / kWave));
+                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)(rv / kWave), n_dst);
             } else {
                 const int64_t chunks = (rv + 2 * kWave - 2) / kWave;      // most kilobytes one copy can touch
                 if (n_src * chunks <= kMaxBlocks)
                     scatter_rows_aligned_kernel<I><<<(unsigned)(n_src * chunks), kWave, 0, s>>>(
-                        (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)chunks, head);
+                        (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)chunks, head, n_dst);
                 else
-                    launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, rv, s);
+                    launch_scatter_t<u32x4, I>(src, dst, pos, n_src, fan, rv, n_dst, s);
             }
             break;
         }
-        case 8: launch_scatter_t<u32x2, I>(src, dst, pos, n_src, fan, row_bytes / 8, s); break;
-        case 4: launch_scatter_t<uint32_t, I>(src, dst, pos, n_src, fan, row_bytes / 4, s); break;
-        case 2: launch_scatter_t<uint16_t, I>(src, dst, pos, n_src, fan, row_bytes / 2, s); break;
-        default: launch_scatter_t<uint8_t, I>(src, dst, pos, n_src, fan, row_bytes, s); break;
+        case 8: launch_scatter_t<u32x2, I>(src, dst, pos, n_src, fan, row_bytes / 8, n_dst, s); break;
+        case 4: launch_scatter_t<uint32_t, I>(src, dst, pos, n_src, fan, row_bytes / 4, n_dst, s); break;
+        case 2: launch_scatter_t<uint16_t, I>(src, dst, pos, n_src, fan, row_bytes / 2, n_dst, s); break;
+        default: launch_scatter_t<uint8_t, I>(src, dst, pos, n_src, fan, row_bytes, n_dst, s); break;
     }
     return check_launch();
 }
-template int launch_scatter_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int, int64_t, hipStream_t);
-template int launch_scatter_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int, int64_t, hipStream_t);
+template int launch_scatter_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int, int64_t, int64_t,
+                                          hipStream_t);
+template int launch_scatter_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int, int64_t, int64_t,
+                                          hipStream_t);
 
 template <typename V, typename I>
 static void launch_gather_t(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_vecs,
-                            hipStream_t s) {
+                            int64_t n_src, hipStream_t s) {
     const int l = tpr_log2_for(row_vecs);
     const int rpi = kBlock >> l;
     const unsigned grid = grid_for(n_out, rpi);
     if (row_vecs > ((int64_t)2 << l))
-        gather_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+        gather_rows_kernel<V, 4, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l, n_src);
     else if (row_vecs > ((int64_t)1 << l))
-        gather_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+        gather_rows_kernel<V, 2, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l, n_src);
     else
-        gather_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l);
+        gather_rows_kernel<V, 1, I><<<grid, kBlock, 0, s>>>((const V *)src, (V *)out, idx, n_out, row_vecs, l, n_src);
 }
 
 template <typename I>
 static bool launch_gather_sliced(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_vecs,
-                                 hipStream_t s) {
+                                 int64_t n_src, hipStream_t s) {
     const int head = (int)(((uintptr_t)out >> 4) & (kWave - 1));
     const int64_t total = n_out * row_vecs;
     const int64_t blocks = (total + head + kWave - 1) / kWave;
     if (blocks > kMaxBlocks) return false;
     if (row_vecs % kWave == 0 && head == 0) {
         gather_rows_sliced_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, row_vecs,
-                                                                       (uint32_t)(row_vecs / kWave));
+                                                                       (uint32_t)(row_vecs / kWave), n_src);
         return true;
     }
     // rows that are not whole lines: a row's chunks share lines on the source side
     const uint32_t run = (row_vecs % 8) ? (uint32_t)((row_vecs + kWave - 1) / kWave) : 0u;
     gather_rows_flat_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, total, row_vecs,
-                                                                 head, run);
+                                                                 head, run, n_src);
     return true;
 }
 
 template <typename I>
-int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s) {
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, int64_t n_src,
+                       hipStream_t s) {
     if (n_out <= 0 || row_bytes <= 0) return TERRACE_OK;
     if (n_out > kMaxGridRows) return TERRACE_EINVAL;
     switch (vec_bytes_for(row_bytes, src, out)) {
         case 16:
-            if (!launch_gather_sliced<I>(src, out, idx, n_out, row_bytes / 16, s))
-                launch_gather_t<u32x4, I>(src, out, idx, n_out, row_bytes / 16, s);
+            if (!launch_gather_sliced<I>(src, out, idx, n_out, row_bytes / 16, n_src, s))
+                launch_gather_t<u32x4, I>(src, out, idx, n_out, row_bytes / 16, n_src, s);
             break;
-        case 8: launch_gather_t<u32x2, I>(src, out, idx, n_out, row_bytes / 8, s); break;
-        case 4: launch_gather_t<uint32_t, I>(src, out, idx, n_out, row_bytes / 4, s); break;
-        case 2: launch_gather_t<uint16_t, I>(src, out, idx, n_out, row_bytes / 2, s); break;
-        default: launch_gather_t<uint8_t, I>(src, out, idx, n_out, row_bytes, s); break;
+        case 8: launch_gather_t<u32x2, I>(src, out, idx, n_out, row_bytes / 8, n_src, s); break;
+        case 4: launch_gather_t<uint32_t, I>(src, out, idx, n_out, row_bytes / 4, n_src, s); break;
+        case 2: launch_gather_t<uint16_t, I>(src, out, idx, n_out, row_bytes / 2, n_src, s); break;
+        default: launch_gather_t<uint8_t, I>(src, out, idx, n_out, row_bytes, n_src, s); break;
     }
     return check_launch();
 }
-template int launch_gather_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int64_t, hipStream_t);
-template int launch_gather_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int64_t, hipStream_t);
+template int launch_gather_rows<int32_t>(const void *, void *, const int32_t *, int64_t, int64_t, int64_t, hipStream_t);
+template int launch_gather_rows<int64_t>(const void *, void *, const int64_t *, int64_t, int64_t, int64_t, hipStream_t);
+
+__global__ __launch_bounds__(kBlock) void zero_bytes_kernel(uint8_t *__restrict__ p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0;
+}
 
 static int64_t dtype_row_bytes(int dtype, int64_t hidden) {
     switch (dtype) {
@@ -689,8 +705,8 @@ static int64_t dtype_row_bytes(int dtype, int64_t hidden) {
 }
 
 template <int SRC, int OUT>
-static void launch_combine_so(const void *src, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
-                              int fan, int64_t hidden, void *out, hipStream_t s) {
+static void launch_combine_so(const void *src, int64_t n_src, const int64_t *idx, const void *w, int w_dtype,
+                              int64_t n_out, int fan, int64_t hidden, void *out, hipStream_t s) {
     const int64_t chunks = hidden / Chunk<SRC>::N;
     const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
     // one wave per workgroup when a row is a whole number of waves' worth of chunks (a workgroup
@@ -703,36 +719,40 @@ static void launch_combine_so(const void *src, const int64_t *idx, const void *w
     // source rows that are not whole lines (and fp8 rows, whose scales share a line): one XCD per output row
     const uint32_t run = (srb % 128 || SRC == TERRACE_FP8_E4M3_B128) && slices > 1 ? (uint32_t)slices : 0u;
     combine_kernel<SRC, OUT><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, fan, hidden,
-                                                 (uint8_t *)out, orb, slices, run);
+                                                 (uint8_t *)out, orb, slices, run, n_src);
 }
 
 template <int SRC>
-static void launch_combine_s(const void *src, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
-                             int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
-    if (out_dtype == TERRACE_F32) launch_combine_so<SRC, TERRACE_F32>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
-    else if (out_dtype == TERRACE_BF16) launch_combine_so<SRC, TERRACE_BF16>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
-    else launch_combine_so<SRC, TERRACE_F16>(src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+static void launch_combine_s(const void *src, int64_t n_src, const int64_t *idx, const void *w, int w_dtype,
+                             int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
+    if (out_dtype == TERRACE_F32) launch_combine_so<SRC, TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+    else if (out_dtype == TERRACE_BF16) launch_combine_so<SRC, TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+    else launch_combine_so<SRC, TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
 }
 
-int launch_combine(const void *src, int src_dtype, const int64_t *idx, const void *w, int w_dtype, int64_t n_out,
-                   int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
+int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
+                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
     if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
     if (n_out * ((hidden + 1023) / 1024 + 1) > kMaxGridRows) return TERRACE_EINVAL;
     const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
+    if (n_src <= 0) {           // no source rows: every entry is dead and every sum empty (the kernels read row 0)
+        zero_bytes_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)out, n_out * orb);
+        return check_launch();
+    }
     const int n = src_dtype == TERRACE_F32 ? 4 : (src_dtype == TERRACE_FP8_E4M3_B128 ? 16 : 8);
     const bool vec = hidden % n == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                      srb % 16 == 0 && orb % 16 == 0 && ((uintptr_t)w & 3) == 0;   // weights are read as dwords
     if (!vec) {
         const int grid = (int)(n_out > 4096 ? 4096 : n_out);
         combine_elem_kernel<<<grid, kBlock, 0, s>>>((const uint8_t *)src, src_dtype, srb, idx, w, w_dtype, n_out, fan,
-                                                    hidden, (uint8_t *)out, out_dtype);
+                                                    hidden, (uint8_t *)out, out_dtype, n_src);
         return check_launch();
     }
     switch (src_dtype) {
-        case TERRACE_F32: launch_combine_s<TERRACE_F32>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        case TERRACE_BF16: launch_combine_s<TERRACE_BF16>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        case TERRACE_F16: launch_combine_s<TERRACE_F16>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_F32: launch_combine_s<TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_BF16: launch_combine_s<TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_F16: launch_combine_s<TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
     }
     return check_launch();
 }
@@ -753,16 +773,18 @@ int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s) {
     return check_launch();
 }
 
-int launch_index_chain(const int64_t *table, const int64_t *idx, int64_t n, int64_t *out, hipStream_t s) {
+int launch_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n, int64_t *out,
+                       hipStream_t s) {
     if (n <= 0) return TERRACE_OK;
-    index_chain_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(table, idx, n, out);
+    index_chain_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(table, n_table, idx, n, out);
     return check_launch();
 }
 
-int launch_index_chain2(const int64_t *outer, const int64_t *inner, const int64_t *idx, int64_t n, int64_t *out,
-                        hipStream_t s) {
+int launch_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *inner, int64_t n_inner,
+                        const int64_t *idx, int64_t n, int64_t *out, hipStream_t s) {
     if (n <= 0) return TERRACE_OK;
-    index_chain2_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(outer, inner, idx, n, out);
+    index_chain2_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(outer, n_outer, inner, n_inner, idx, n,
+                                                                           out);
     return check_launch();
 }
 

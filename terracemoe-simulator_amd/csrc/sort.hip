@@ -852,7 +852,7 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
                      pos32, meta};
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
-    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
+    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, P, s);
 }
 
 // ---- Hop-B arrival, general branch (pairs listed explicitly) -------------------------------------
@@ -880,7 +880,7 @@ int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_i
     EmitPairs emit{r_in, slot_in, rgate, gate_bytes, gate_width, R, gate_pairs, r_idx, slot_idx, ordo, src32};
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
-    return launch_gather_rows<int32_t>(rx, send_buf, src32, P, row_bytes, s);
+    return launch_gather_rows<int32_t>(rx, send_buf, src32, P, row_bytes, R, s);
 }
 
 // ---- expert-order regroup ---------------------------------------------------------------------
@@ -940,7 +940,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     }
     rc = check_launch();
     if (rc != TERRACE_OK || !node_rx) return rc;
-    return launch_gather_rows<int32_t>(node_rx, permuted, src_of_place, places, row_bytes, s);
+    return launch_gather_rows<int32_t>(node_rx, permuted, src_of_place, places, row_bytes, P, s);
 }
 
 int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
@@ -985,7 +985,7 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
                         pos32, mask_pitch, gate_pitch, gate_pad};
     int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
-    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
+    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
 }
 
 int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
@@ -1042,7 +1042,7 @@ int run_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, in
     const int32_t *pos32 = k2_token_path_applies(k, n_nodes)
                                ? k2_token_positions(ws, T, n_nodes)
                                : (const int32_t *)((const char *)ws + units_table_bytes(make_units(S, n_nodes)));
-    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, s);
+    return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
 }
 
 int run_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int rpn, void *send_buf,
@@ -1054,7 +1054,7 @@ int run_k1_arrival_move(const void *rx, int64_t R, int64_t row_bytes, int quota,
     if (!rx || !send_buf || !ws) return TERRACE_EINVAL;
     if (ws_bytes < k1_workspace(R, quota, rpn)) return TERRACE_ENOSPC;
     const int32_t *pos32 = (const int32_t *)((const char *)ws + units_table_bytes(make_units(P, rpn)));
-    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, s);
+    return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, P, s);
 }
 
 int run_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr, int64_t capacity, void *permuted,
@@ -1073,7 +1073,7 @@ int run_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr,
     if (ws_bytes < regroup_workspace(P, epr, capacity)) return TERRACE_ENOSPC;
     const int32_t *order32 = (const int32_t *)((const char *)ws + units_table_bytes(make_units(P, epr)));
     const int32_t *gidx = (const int32_t *)((const char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
-    return launch_gather_rows<int32_t>(node_rx, permuted, capacity >= 0 ? gidx : order32, places, row_bytes, s);
+    return launch_gather_rows<int32_t>(node_rx, permuted, capacity >= 0 ? gidx : order32, places, row_bytes, P, s);
 }
 
 }  // namespace terrace

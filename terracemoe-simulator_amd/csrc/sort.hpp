@@ -25,11 +25,13 @@ size_t units_table_bytes(const Units &u);
 void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
                  int32_t *status, hipStream_t s);
 
+// n_dst / n_src bound the row ids the movers accept: an id outside [0, bound) is a dead entry.
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
-                        hipStream_t s);
+                        int64_t n_dst, hipStream_t s);
 template <typename I>
-int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, hipStream_t s);
+int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, int64_t n_src,
+                       hipStream_t s);
 
 // Send side with one lane per token (n_nodes <= 64, k <= 16); returns false when the geometry
 // is outside that and the caller must take the (token, run)-item path.

@@ -480,7 +480,8 @@ def regroup_move(node_rx, workspace, epr, capacity=None):
 
 
 def gather_rows(src, idx):
-    """``src[idx]`` for a 2-D ``src``; negative indices give zero rows."""
+    """``src[idx]`` for a 2-D ``src``; indices outside ``[0, len(src))`` (negative ones included) give
+    zero rows -- the kernel never forms an address from them."""
     _require()
     _hip.need_device(src, idx)
     src, idx = src.contiguous(), idx.contiguous().reshape(-1)
@@ -490,15 +491,15 @@ def gather_rows(src, idx):
     row_bytes = src.element_size()
     for d in src.shape[1:]:
         row_bytes *= int(d)
-    _hip.call("terrace_gather_rows", _hip.ptr(src), _hip.ptr(idx), idx.numel(), row_bytes, _hip.ptr(out),
-              _hip.stream(src.device))
+    _hip.call("terrace_gather_rows", _hip.ptr(src), src.shape[0], _hip.ptr(idx), idx.numel(), row_bytes,
+              _hip.ptr(out), _hip.stream(src.device))
     return out
 
 
 def scatter_rows(src, pos, n_dst):
     """``dst[pos[r, f]] = src[r]``: each source row is read once and written ``pos.shape[1]``
-    times (negative places are skipped).  ``dst`` has ``n_dst`` rows; rows no place names are
-    left uninitialised."""
+    times (places outside ``[0, n_dst)`` are skipped).  ``dst`` has ``n_dst`` rows; rows no place
+    names are left uninitialised."""
     _require()
     _hip.need_device(src, pos)
     src, pos = src.contiguous(), pos.contiguous()
@@ -509,29 +510,30 @@ def scatter_rows(src, pos, n_dst):
     for d in src.shape[1:]:
         row_bytes *= int(d)
     _hip.call("terrace_scatter_rows", _hip.ptr(src), _hip.ptr(pos), src.shape[0], pos.shape[1], row_bytes,
-              _hip.ptr(dst), _hip.stream(src.device))
+              _hip.ptr(dst), int(n_dst), _hip.stream(src.device))
     return dst
 
 
 def index_chain(table, idx):
-    """``table[idx]`` over int64 planes (negative entries propagate as -1)."""
+    """``table[idx]`` over int64 planes (entries outside the table, negative ones included, give -1)."""
     _require()
     _hip.need_device(table, idx)
     table, idx = table.contiguous(), idx.contiguous()
     out = torch.empty_like(idx)
-    _hip.call("terrace_index_chain", _hip.ptr(table), _hip.ptr(idx), idx.numel(), _hip.ptr(out),
+    _hip.call("terrace_index_chain", _hip.ptr(table), table.numel(), _hip.ptr(idx), idx.numel(), _hip.ptr(out),
               _hip.stream(idx.device))
     return out
 
 
 def index_chain2(outer, inner, idx):
-    """``outer[inner[idx]]`` over int64 planes in one launch (negative entries propagate as -1)."""
+    """``outer[inner[idx]]`` over int64 planes in one launch (an entry outside its table at either
+    level, negative ones included, gives -1)."""
     _require()
     _hip.need_device(outer, inner, idx)
     outer, inner, idx = outer.contiguous(), inner.contiguous(), idx.contiguous()
     out = torch.empty_like(idx)
-    _hip.call("terrace_index_chain2", _hip.ptr(outer), _hip.ptr(inner), _hip.ptr(idx), idx.numel(), _hip.ptr(out),
-              _hip.stream(idx.device))
+    _hip.call("terrace_index_chain2", _hip.ptr(outer), outer.numel(), _hip.ptr(inner), inner.numel(),
+              _hip.ptr(idx), idx.numel(), _hip.ptr(out), _hip.stream(idx.device))
     return out
 
 
@@ -565,7 +567,7 @@ def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
             raise RuntimeError("combine: weights must match idx")
         w_code = _hip.float_code(weights.dtype)
     out = torch.empty((n_out, hidden), dtype=out_dtype, device=src.device)
-    _hip.call("terrace_combine", _hip.ptr(src), src_code, _hip.ptr(idx), _hip.ptr(weights), w_code, n_out, fan,
+    _hip.call("terrace_combine", _hip.ptr(src), src.shape[0], src_code, _hip.ptr(idx), _hip.ptr(weights), w_code, n_out, fan,
               hidden, _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
     return out
 

@@ -539,6 +539,12 @@ def test_combine_bit_exact_and_within_tolerance(src_fmt, out_fmt, H, fan):
     idx = torch.randint(0, n_src, (n_out, fan), generator=g)
     idx[5, 0] = -1
     idx[6, :] = -1
+    idx[8, fan - 1] = n_src                                          # past the end of src: dead, like a negative id
+    idx[9, 0] = 1 << 41
+    dead_too = idx.clone()
+    idx[idx >= n_src] = -1                                           # what the oracle is given instead
+    got_oob = tops.combine(src.to(DEV), dead_too.to(DEV), None, out_dtype=DT[out_fmt])
+    assert torch.equal(got_oob, tops.combine(src.to(DEV), idx.to(DEV), None, out_dtype=DT[out_fmt]))
     for wfmt in (None, "f32", src_fmt):
         w = None if wfmt is None else rows_of(torch.rand(n_out, fan, generator=g), wfmt)
         got = tops.combine(src.to(DEV), idx.to(DEV), None if w is None else w.to(DEV), out_dtype=DT[out_fmt])
@@ -598,6 +604,18 @@ def test_gather_rows_and_index_chain():
     idx = torch.randint(-1, 100, (4, 7), generator=g)
     want = torch.where(idx < 0, torch.full_like(idx, -1), table[idx.clamp(min=0)])
     assert torch.equal(tops.index_chain(table.to(DEV), idx.to(DEV)).cpu(), want)
+    # ids past the end of a table are dead at either level of the two-step form, and never read
+    inner = torch.randint(-1, 130, (60,), generator=g)               # values 100..129 miss the outer table
+    idx2 = torch.randint(-1, 75, (9, 5), generator=g)                # values 60..74 miss the inner table
+    mid = torch.where((idx2 >= 0) & (idx2 < 60), inner[idx2.clamp(0, 59)], torch.full_like(idx2, -1))
+    want2 = torch.where((mid >= 0) & (mid < 100), table[mid.clamp(0, 99)], torch.full_like(idx2, -1))
+    assert torch.equal(tops.index_chain2(table.to(DEV), inner.to(DEV), idx2.to(DEV)).cpu(), want2)
+    assert torch.equal(tops.index_chain(table.to(DEV), (idx + 101).to(DEV)).cpu(), torch.full_like(idx, -1))
+    empty = torch.zeros(0, dtype=torch.int64, device=DEV)
+    assert bool((tops.index_chain(empty, idx.clamp(min=0).to(DEV)) == -1).all())
+    rows = torch.randn(0, 64, device=DEV)
+    assert not tops.gather_rows(rows, torch.zeros(5, dtype=torch.int64, device=DEV)).any()
+    assert not tops.combine(rows, torch.zeros(5, 3, dtype=torch.int64, device=DEV)).any()
 
 
 # ------------------------------------------------------------------------------- wire containers
@@ -722,28 +740,31 @@ def test_row_movers_at_every_base_alignment(row_bytes):
         src = src_buf[off_src:off_src + n_src * row_bytes].view(n_src, row_bytes)
         idx = torch.randint(0, n_src, (n_out,), generator=g)
         idx[7] = -1
+        idx[9], idx[11] = n_src, 1 << 40                         # past the end of src: dead entries, never addresses
         out_buf = torch.full((pad + n_out * row_bytes + pad,), 0xAB, dtype=torch.uint8, device=DEV)
-        rc = lib.terrace_gather_rows(c_void_p(src.data_ptr()), _hip.ptr(idx.to(DEV)), n_out, row_bytes,
+        rc = lib.terrace_gather_rows(c_void_p(src.data_ptr()), n_src, _hip.ptr(idx.to(DEV)), n_out, row_bytes,
                                      c_void_p(out_buf.data_ptr() + off_dst), stream)
         assert rc == 0
         got = out_buf[off_dst:off_dst + n_out * row_bytes].view(n_out, row_bytes).cpu()
-        want = src.cpu()[idx.clamp(min=0)]
-        want[idx < 0] = 0
+        dead = (idx < 0) | (idx >= n_src)
+        want = src.cpu()[idx.clamp(0, n_src - 1)]
+        want[dead] = 0
         assert torch.equal(got, want), (off_src, off_dst)
         assert bool((out_buf[:off_dst] == 0xAB).all()) and bool((out_buf[off_dst + n_out * row_bytes:] == 0xAB).all())
         # scatter: every destination row named at most once, a few left unnamed
         n_dst = n_src * fan + 5
         pos = torch.randperm(n_dst, generator=g)[:n_src * fan].view(n_src, fan).clone()
         pos[3, 1] = -1
+        pos[5, 0], pos[6, 2] = n_dst, 1 << 40                    # past the end of dst: copies not made
         dst_buf = torch.full((pad + n_dst * row_bytes + pad,), 0xCD, dtype=torch.uint8, device=DEV)
         rc = lib.terrace_scatter_rows(c_void_p(src.data_ptr()), _hip.ptr(pos.to(DEV)), n_src, fan, row_bytes,
-                                      c_void_p(dst_buf.data_ptr() + off_dst), stream)
+                                      c_void_p(dst_buf.data_ptr() + off_dst), n_dst, stream)
         assert rc == 0
         got = dst_buf[off_dst:off_dst + n_dst * row_bytes].view(n_dst, row_bytes).cpu()
         want = torch.full((n_dst, row_bytes), 0xCD, dtype=torch.uint8)
         for r in range(n_src):
             for f in range(fan):
-                if pos[r, f] >= 0:
+                if 0 <= pos[r, f] < n_dst:
                     want[pos[r, f]] = src.cpu()[r]
         assert torch.equal(got, want), (off_src, off_dst)
         assert bool((dst_buf[:off_dst] == 0xCD).all()) and bool((dst_buf[off_dst + n_dst * row_bytes:] == 0xCD).all())
