@@ -392,6 +392,32 @@ def test_malformed_routing_is_contained_and_counted():
         assert torch.isfinite(gate_rows).all()
         if name == "id_range":
             assert fault & _hip.FAULT_ID_RANGE
+    # the (token, run)-item kernels (k > 16, or more than 64 nodes) contain the same breakage: every address they
+    # form comes from an item's sorted position or from a rank below k, never from an id
+    g = torch.Generator().manual_seed(9)
+    for world, rpn, E, T, k, M in [(8, 2, 64, 40, 24, 4), (160, 2, 160, 50, 4, 2)]:
+        n_nodes, slots, q = world // rpn, (E // world) * rpn, k // M
+        e = torch.from_numpy(equal_quota_routing(T, k, E, n_nodes, M, 5, False)).clone()
+        e[1, 0] = E + 7                          # outside [0, E)
+        e[2, 1] = -3
+        e[3, :] = e[3, 0]                        # one expert k times: one node, ranks collide
+        e[4, : k // 2] = e[4, k // 2:][: k // 2] if k % 2 == 0 else e[4, : k // 2]     # duplicates
+        e[5] = torch.randint(0, E, (k,), generator=g)                                  # no quota structure at all
+        x = torch.randn(T, 24, device=DEV)
+        gts = torch.rand(T, k, device=DEV)
+        (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e.to(DEV), gts, world, E, rpn, M, extras=True)
+        torch.cuda.synchronize()
+        fault = ex["status"].tolist()[0]
+        assert fault & _hip.FAULT_ID_RANGE and fault & (_hip.FAULT_FANOUT | _hip.FAULT_QUOTA), fault
+        assert int(counts.sum()) == T * M and bool((counts >= 0).all())
+        assert bool(((u_src >= 0) & (u_src < T)).all())
+        assert bool(((ex["token_rows"] >= 0) & (ex["token_rows"] < T * M)).all())
+        assert bool(((ex["pair_table"] >= -1) & (ex["pair_table"] < T * M * q)).all())
+        # the clean tokens still get their rows right
+        clean = torch.ones(T, dtype=torch.bool)
+        clean[1:6] = False
+        rows_of_clean = ex["token_rows"].cpu()[clean]
+        assert torch.equal(payload.cpu()[rows_of_clean.reshape(-1)], x.cpu()[clean].repeat_interleave(M, 0))
 
 
 def test_hopa_send_splits_literal(literals):
