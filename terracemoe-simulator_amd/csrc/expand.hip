@@ -366,17 +366,35 @@ int run_pair_places(const int64_t *order, const int64_t *r_idx, const int64_t *s
 // is not possible without ordering, so the caller provides them initialised to {INT_MAX, 0}).
 __global__ __launch_bounds__(kBlock) void map_count_kernel(const uint8_t *__restrict__ map, int64_t T, int E,
                                                            int32_t *__restrict__ row_stats) {
+    // a resident grid: every wave walks its share of the tokens keeping a running min / max, the workgroup
+    // folds its four waves, and only then two atomics go out (per-token atomics on the same two words
+    // serialise at about 20 ns each)
+    __shared__ int32_t lo_of[kWavesPerBlock], hi_of[kWavesPerBlock];
     const int lane = lane_id();
-    const int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + wave_in_block();
-    if (t >= T) return;
-    int cnt = 0;
-    for (int e0 = 0; e0 < E; e0 += kWave) {
-        const int e = e0 + lane;
-        cnt += __popcll(__ballot(e < E && map[t * E + e] != 0));
+    const int w = wave_in_block();
+    int lo = 0x7FFFFFFF, hi = 0;
+    const int64_t stride = (int64_t)gridDim.x * kWavesPerBlock;
+    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + w; t < T; t += stride) {
+        int cnt = 0;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            cnt += __popcll(__ballot(e < E && map[t * E + e] != 0));
+        }
+        lo = cnt < lo ? cnt : lo;
+        hi = cnt > hi ? cnt : hi;
     }
     if (lane == 0) {
-        atomicMin(&row_stats[0], cnt);
-        atomicMax(&row_stats[1], cnt);
+        lo_of[w] = lo;
+        hi_of[w] = hi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < kWavesPerBlock; ++i) {
+            lo = lo_of[i] < lo ? lo_of[i] : lo;
+            hi = hi_of[i] > hi ? hi_of[i] : hi;
+        }
+        if (lo != 0x7FFFFFFF) atomicMin(&row_stats[0], lo);
+        if (hi != 0) atomicMax(&row_stats[1], hi);
     }
 }
 
@@ -413,7 +431,9 @@ int run_map_count(const void *map, int64_t T, int E, int32_t *row_stats, hipStre
     map_stats_init_kernel<<<1, 1, 0, s>>>(row_stats);
     if (T > 0) {
         if (!map) return TERRACE_EINVAL;
-        map_count_kernel<<<(unsigned)((T + kWavesPerBlock - 1) / kWavesPerBlock), kBlock, 0, s>>>((const uint8_t *)map, T, E, row_stats);
+        int64_t blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;
+        if (blocks > 1024) blocks = 1024;
+        map_count_kernel<<<(unsigned)blocks, kBlock, 0, s>>>((const uint8_t *)map, T, E, row_stats);
     }
     return check_launch();
 }
