@@ -587,6 +587,22 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
     static constexpr bool kTallies = true;
     typedef NoPre Pre;
     __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    // rank m*quota + i of token t and cell i of its send row `row`: no pair, zero slot, zero gate
+    __device__ __forceinline__ void put_defaults(int64_t t, int m, int32_t row, int i) const {
+        const int64_t at = t * k + (int64_t)m * quota + i;
+        if (pair_table) pair_table[at] = -1;
+        if (sort_order) sort_order[at] = 0;
+        mask[(int64_t)row * mask_pitch + i] = 0;
+        if (!gates) return;
+        const int64_t gcell = (int64_t)row * gate_pitch + i;
+        if (gate_bytes == 4) {
+            ((uint32_t *)gate_rows)[gcell] = 0u;
+            if (gate_sorted) ((uint32_t *)gate_sorted)[at] = 0u;
+        } else {
+            ((uint16_t *)gate_rows)[gcell] = (uint16_t)0;
+            if (gate_sorted) ((uint16_t *)gate_sorted)[at] = (uint16_t)0;
+        }
+    }
     __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, int64_t, Pre, const int32_t *,
                                               int *tally) const {
         const int64_t t = item / groups_m;
@@ -632,12 +648,26 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
         if (u_node) u_node[row] = node;
         if (token_rows) token_rows[item] = row;
         pos32[item] = row;
+        // A run owns ranks [m*quota, (m+1)*quota) of its token's per-rank planes and the quota cells of its
+        // row.  With duplicate ids ranks collide and some of those are claimed by no element: they are given
+        // the defaults below (no pair, zero cells), so every entry is defined whatever the routing.
+        // the row's pad after its quota gates (wire containers).  One loop per element width: with the width test
+        // inside a single loop this toolchain's backend fails to select an instruction at build time.
+        if (gates && gate_bytes == 4)
+            for (int z = 0; z < gate_pad; ++z) ((uint32_t *)gate_rows)[(int64_t)row * gate_pitch + quota + z] = 0u;
+        if (gates && gate_bytes != 4)
+            for (int z = 0; z < gate_pad; ++z) ((uint16_t *)gate_rows)[(int64_t)row * gate_pitch + quota + z] = (uint16_t)0;
+        uint64_t claimed = 0;
+        const bool wide = quota > 64;            // more ranks than the mask holds: defaults first, for all of them
+        if (wide)
+            for (int i = 0; i < quota; ++i) put_defaults(t, m, row, i);
         auto body = [&](int j) {
             const int e = ids.at(j);
             if (e < 0 || e >= n_experts) fault |= TERRACE_FAULT_ID_RANGE;
             const int r = rank_in_row(ids, j);
             if (r / quota != m) return;
             const int i = r - m * quota;
+            if (!wide) claimed |= 1ull << i;
             const int64_t cell = (int64_t)row * quota + i;
             mask[(int64_t)row * mask_pitch + i] = e >= 0 ? e - ids.node(j) * slots : 0;
             if (gates) {
@@ -646,14 +676,10 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
                     const uint32_t gv = ((const uint32_t *)gates)[t * k + j];
                     ((uint32_t *)gate_rows)[gcell] = gv;
                     if (gate_sorted) ((uint32_t *)gate_sorted)[t * k + r] = gv;
-                    if (i == 0)
-                        for (int z = 0; z < gate_pad; ++z) ((uint32_t *)gate_rows)[gcell + quota + z] = 0u;
                 } else {
                     const uint16_t gv = ((const uint16_t *)gates)[t * k + j];
                     ((uint16_t *)gate_rows)[gcell] = gv;
                     if (gate_sorted) ((uint16_t *)gate_sorted)[t * k + r] = gv;
-                    if (i == 0)
-                        for (int z = 0; z < gate_pad; ++z) ((uint16_t *)gate_rows)[gcell + quota + z] = (uint16_t)0;
                 }
             }
             if (inverse) inverse[t * k + j] = row;
@@ -666,6 +692,14 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
                 if (j < k) body(j);
         } else {
             for (int j = 0; j < k; ++j) body(j);
+        }
+        if (!wide) {
+            const uint64_t all = quota == 64 ? ~0ull : (1ull << quota) - 1ull;
+            uint64_t holes = ~claimed & all;
+            while (holes) {
+                put_defaults(t, m, row, __builtin_ctzll(holes));
+                holes &= holes - 1;
+            }
         }
         return fault;
     }

@@ -413,6 +413,8 @@ def test_malformed_routing_is_contained_and_counted():
         assert bool(((u_src >= 0) & (u_src < T)).all())
         assert bool(((ex["token_rows"] >= 0) & (ex["token_rows"] < T * M)).all())
         assert bool(((ex["pair_table"] >= -1) & (ex["pair_table"] < T * M * q)).all())
+        assert bool(((mask >= 0) & (mask < slots)).all()) and bool(torch.isfinite(gate_rows).all())
+        assert bool(((ex["sort_order"] >= 0) & (ex["sort_order"] < k)).all())
         # the clean tokens still get their rows right
         clean = torch.ones(T, dtype=torch.bool)
         clean[1:6] = False
