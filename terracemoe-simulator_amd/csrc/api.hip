@@ -91,7 +91,11 @@ static bool float_dtype(int d) { return d == TERRACE_F32 || d == TERRACE_BF16 ||
 
 extern "C" {
 
-const char *terrace_version(void) { return "terrace-hip 0.1 (gfx950)"; }
+#ifndef TERRACE_SOURCE_HASH
+#define TERRACE_SOURCE_HASH "unstamped"
+#endif
+// ends with the digest of the sources this library was built from (csrc/build.py stamps it)
+const char *terrace_version(void) { return "terrace-hip 0.1 (gfx950) src:" TERRACE_SOURCE_HASH; }
 
 const char *terrace_strerror(int status) {
     switch (status) {

@@ -7,6 +7,8 @@ terracemoe-simulator_amd/lib/ where the ``terrace`` package looks for it.
 """
 from __future__ import annotations
 
+import glob
+import hashlib
 import os
 import subprocess
 import sys
@@ -29,9 +31,23 @@ FLAGS = [
 ]
 
 
+def source_hash() -> str:
+    """Digest of everything the library is compiled from; build() stamps it into the library
+    (terrace_version() ends with it) so that a library older than its sources can be told apart."""
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(HERE, "*.hip")) + glob.glob(os.path.join(HERE, "*.hpp")) +
+                   glob.glob(os.path.join(ROOT, "include", "*.h")))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def _compile(src: str) -> str:
     obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(HERE, src), "-o", obj]
+    stamp = [f'-DTERRACE_SOURCE_HASH="{source_hash()}"'] if src == "api.hip" else []
+    cmd = [HIPCC, *FLAGS, *stamp, "-c", os.path.join(HERE, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode:
         raise RuntimeError(f"hipcc failed on {src}:\n{res.stdout}\n{res.stderr}")

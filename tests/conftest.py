@@ -19,6 +19,29 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a ROCm device (run on the MI355X box)")
 
 
+def pytest_sessionstart(session):
+    """A library built before its sources were last edited must not be tested (least of all on a GPU, where
+    a kernel that lacks a check its test relies on can fault the card): build.py stamps the digest of the
+    sources into the library, and the session stops here when the two differ."""
+    import glob
+    import importlib.util
+    import re
+    libs = sorted(glob.glob(os.path.join(PKG, "lib", "libterrace_hip*.so")))
+    if not libs or os.environ.get("TERRACE_OPS_LIB"):
+        return
+    spec = importlib.util.spec_from_file_location("terrace_build", os.path.join(PKG, "csrc", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    # read the stamp out of the file: loading a HIP library here, before torch has brought in the HIP runtime it
+    # ships, would bind the library to another copy of the runtime and every launch would fail
+    with open(libs[0], "rb") as f:
+        found = re.search(rb"\(gfx950\) src:([0-9a-z]+)", f.read())
+    stamped = found.group(1).decode() if found else "none"
+    if stamped != build.source_hash():
+        pytest.exit(f"{libs[0]} was built from other sources (stamp {stamped}, sources {build.source_hash()}): "
+                    f"run python terracemoe-simulator_amd/csrc/build.py", returncode=3)
+
+
 def pytest_collection_modifyitems(config, items):
     try:
         import torch
