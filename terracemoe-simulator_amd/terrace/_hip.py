@@ -154,7 +154,18 @@ def ptr(t):
     return None if t is None else c_void_p(t.data_ptr())
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream(device) -> c_void_p:
+    """The HIP stream torch currently launches on for ``device``.  The raw-handle accessor is an order of
+    magnitude cheaper than building a ``torch.cuda.Stream`` object, which matters where a step is a dozen
+    launches of a few microseconds each."""
+    if _RAW_STREAM is not None:
+        index = device.index if isinstance(device, torch.device) else torch.device(device).index
+        if index is None:
+            index = torch.cuda.current_device()
+        return c_void_p(_RAW_STREAM(index))
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
