@@ -280,12 +280,15 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
             raw[tl] = (gate_affinity ? gate_affinity : affinity)[tt * E];
         }
         __builtin_amdgcn_wave_barrier();
-        float den = 0.0f;
-        for (int j = 0; j < k; ++j)
-            den = j == 0 ? ((volatile float *)raw)[0] : __fadd_rn(den, ((volatile float *)raw)[j]);
+        // lane j of the token takes pick j into registers (one LDS round trip); the left-to-right sum of the
+        // raw gates then reads lane after lane instead of walking LDS k times, one dependent load after the other
+        const int my_pick = tl < k ? ((volatile int *)sel)[tl] : 0;
+        const float my_raw = tl < k ? ((volatile float *)raw)[tl] : 0.0f;
+        float den = from_lane_f(my_raw, 0);
+        for (int j = 1; j < k; ++j) den = __fadd_rn(den, from_lane_f(my_raw, j));
         if (tl < k && live) {
-            expert_idx[t * k + tl] = ((volatile int *)sel)[tl];
-            store_gate(gates, gate_dtype, t * k + tl, __fdiv_rn(((volatile float *)raw)[tl], den));
+            expert_idx[t * k + tl] = my_pick;
+            store_gate(gates, gate_dtype, t * k + tl, __fdiv_rn(my_raw, den));
         }
         __builtin_amdgcn_wave_barrier();
     }
