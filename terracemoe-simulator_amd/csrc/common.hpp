@@ -18,6 +18,12 @@ __device__ __forceinline__ int wave_in_block() { return threadIdx.x >> 6; }
 
 __device__ __forceinline__ uint64_t lanes_below(int lane) { return (1ull << lane) - 1ull; }
 
+// Wave-private LDS words that lanes of one wave exchange values through.  The pointer carries the LDS address
+// space in its type: a volatile access through a generic pointer is left as a flat instruction by the compiler,
+// through one of these it is a ds_read / ds_write.
+typedef __attribute__((address_space(3))) volatile int32_t lds_i32;
+typedef __attribute__((address_space(3))) volatile float lds_f32;
+
 // Value held by `src_lane` (uniform across the wave).
 __device__ __forceinline__ int read_lane(int v, int src_lane) {
     return __builtin_amdgcn_readlane(v, src_lane);

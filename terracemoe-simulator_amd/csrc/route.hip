@@ -136,8 +136,8 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
     const int tl = lane & (LPT - 1);             // lane within the token
     const int slot = lane / LPT;                 // which of the wave's tokens
     const int lane0 = lane - tl;                 // the token's first lane
-    int *sel = lds + (w * TPW + slot) * 2 * k;   // per token: k chosen ids, then their k raw gates
-    float *raw = (float *)(sel + k);
+    lds_i32 *sel = (lds_i32 *)lds + (w * TPW + slot) * 2 * k;   // per token: k chosen ids, then their k raw gates
+    lds_f32 *raw = (lds_f32 *)(sel + k);
     const int q = k / M;
     const int my_group = tl / LPG;
     float b[VPL];
@@ -275,15 +275,15 @@ __global__ __launch_bounds__(kBlock) void route_wave_kernel(const float *__restr
         }
         __builtin_amdgcn_wave_barrier();
         // slots nobody filed (NaN scores are never picked): expert 0 and its gate
-        if (tl < k && ((volatile int *)sel)[tl] < 0) {
+        if (tl < k && sel[tl] < 0) {
             sel[tl] = 0;
             raw[tl] = (gate_affinity ? gate_affinity : affinity)[tt * E];
         }
         __builtin_amdgcn_wave_barrier();
         // lane j of the token takes pick j into registers (one LDS round trip); the left-to-right sum of the
         // raw gates then reads lane after lane instead of walking LDS k times, one dependent load after the other
-        const int my_pick = tl < k ? ((volatile int *)sel)[tl] : 0;
-        const float my_raw = tl < k ? ((volatile float *)raw)[tl] : 0.0f;
+        const int my_pick = tl < k ? sel[tl] : 0;
+        const float my_raw = tl < k ? raw[tl] : 0.0f;
         float den = from_lane_f(my_raw, 0);
         for (int j = 1; j < k; ++j) den = __fadd_rn(den, from_lane_f(my_raw, j));
         if (tl < k && live) {

@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, in
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
     const int w = wave_in_block();
-    volatile int32_t *hist = lds + w * u.n_buckets;
+    lds_i32 *hist = (lds_i32 *)lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
     const int key_bits = bits_for(u.n_buckets);
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
     const int w = wave_in_block();
-    volatile int32_t *cursor = lds + w * u.n_buckets;
+    lds_i32 *cursor = (lds_i32 *)lds + w * u.n_buckets;
     const int unit = blockIdx.x * kWavesPerBlock + w;
     if (unit >= u.n_units) return;
     const int key_bits = bits_for(u.n_buckets);
