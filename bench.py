@@ -259,11 +259,19 @@ def main():
     kept_pairs = int((state.place >= 0).sum()) if cap is not None else None
     min_bytes = configs.minimum_traffic_bytes(cfg, kept_pairs, None if cap is None else cfg.slots * cap)
     stages = {}
+    # rows a stage writes: send rows, (row, slot) pairs, places of the expert-order buffer, tokens
+    rows_out = {"route": cfg.T, "pack": cfg.send_rows, "arrival": cfg.pairs,
+                "regroup": cfg.pairs if cap is None else cfg.slots * cap, "combine": cfg.T}
     for name, ms in stage_ms.items():
         gbps = nbytes[name] / ms / 1e6
+        min_gbps = min_bytes[name] / ms / 1e6
+        # "GBps" follows the convention that counts a payload row once on the read and once on the write side of
+        # a stage (a scatter that reads a row once for all its copies can thus exceed the peak); "min_traffic"
+        # prices the bytes that must cross HBM
         stages[name] = {"ms": round(ms, 4), "GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
-                        "min_traffic_GBps": round(min_bytes[name] / ms / 1e6, 1)}
-    stages["arrival"]["us_per_row"] = round(stage_ms["arrival"] * 1e3 / cfg.pairs, 6)
+                        "min_traffic_GBps": round(min_gbps, 1),
+                        "min_traffic_frac_hbm_peak": round(min_gbps / HBM_PEAK_GBPS, 4),
+                        "us_per_row": round(ms * 1e3 / max(rows_out[name], 1), 6)}
     stages["arrival"]["reference_target_us_per_row"] = REFERENCE_TARGET_US_PER_ROW
     pc_bytes = nbytes["pack"] + nbytes["combine"]
     pc_ms = stage_ms["pack"] + stage_ms["combine"]
