@@ -334,7 +334,10 @@ def main():
                         "note": "bytes that must cross HBM: a scatter reads each source row once however many "
                                 "copies it writes, a capacity layout reads only the rows it keeps"},
         "pack_plus_combine": {"GBps": round(pc_bytes / pc_ms / 1e6, 1),
-                              "frac_hbm_peak": round(pc_bytes / pc_ms / 1e6 / HBM_PEAK_GBPS, 4)},
+                              "frac_hbm_peak": round(pc_bytes / pc_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                              "min_traffic_GBps": round((min_bytes["pack"] + min_bytes["combine"]) / pc_ms / 1e6, 1),
+                              "min_traffic_frac_hbm_peak": round((min_bytes["pack"] + min_bytes["combine"]) / pc_ms
+                                                                 / 1e6 / HBM_PEAK_GBPS, 4)},
         "arrival_chain_us_per_row": stages["arrival"]["us_per_row"],
         "stages": stages, "kernels": kern, "roofline": roofline,
         "library": os.path.relpath(st.lib, ROOT),
