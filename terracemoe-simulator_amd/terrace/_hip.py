@@ -119,8 +119,26 @@ def load(path: str | None = None):
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype, fn.argtypes = res, args
+    _refuse_stale(lib, path)
     _LIB, _LIB_PATH = lib, path
     return lib
+
+
+def _refuse_stale(lib, path):
+    """In a source tree (csrc/build.py beside the package) the library must carry the digest of the sources
+    that are there now: a kernel older than the host code that calls it can read what it was never given.
+    ``TERRACE_ALLOW_STALE=1`` switches the check off; an installed package without sources has nothing to check."""
+    build_py = os.path.join(os.path.dirname(PKG_DIR), "csrc", "build.py")
+    if not os.path.exists(build_py) or os.environ.get("TERRACE_ALLOW_STALE") == "1":
+        return
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("terrace_csrc_build_check", build_py)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    stamped = lib.terrace_version().decode().rsplit("src:", 1)[-1]
+    if stamped != mod.source_hash():
+        raise LibraryError(f"{path} was built from other sources than those in {os.path.dirname(build_py)} "
+                           f"(stamp {stamped}, sources {mod.source_hash()}): run python {build_py}")
 
 
 def library_path():
