@@ -44,7 +44,8 @@ enum terrace_status {
     TERRACE_OK = 0,
     TERRACE_EINVAL = -22,  /* bad geometry / null pointer / unsupported size */
     TERRACE_ENOSPC = -28,  /* workspace smaller than the matching *_workspace() answer */
-    TERRACE_ELAUNCH = -5   /* the HIP runtime refused a launch (hipGetLastError != 0) */
+    TERRACE_ELAUNCH = -5,  /* the HIP runtime refused a launch (hipGetLastError != 0) */
+    TERRACE_E2BIG = -7     /* input larger than the fixed scratch of terrace_k1_arrival_static */
 };
 
 enum terrace_dtype {
@@ -350,6 +351,25 @@ TERRACE_API int terrace_routing_map_topk(const void *routing_map, const void *pr
  * except send[n*rpn + my_local] = node_counts[n]. */
 TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local,
                              int64_t *send, terrace_stream_t stream);
+
+/* ---- the entry point that brings its own scratch memory ----
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory at all -- code under
+ * HIP graph capture, serving loops that must stay off the allocator, harnesses that forbid hipMalloc -- and so
+ * cannot provide the workspace terrace_k1_arrival asks for.  terrace_k1_arrival_static is terrace_k1_arrival
+ * (same arguments, same outputs, same kernels) with the workspace taken from a device array of
+ * TERRACE_STATIC_SCRATCH_BYTES that is part of the library image: every GPU the library runs on holds that
+ * array until the process ends.  Inputs whose workspace would not fit (terrace_k1_arrival_workspace(R, quota,
+ * rpn) > terrace_static_scratch_bytes(); about 900 thousand pairs) are refused with TERRACE_E2BIG.  The call
+ * allocates and frees nothing.  Unlike the rest of the library it is not reentrant: all calls on one GPU use
+ * that GPU's one array, so two of them must not overlap (same stream, or ordered by events).  The device the
+ * stream belongs to must be current. */
+#define TERRACE_STATIC_SCRATCH_BYTES (4u << 20)
+TERRACE_API size_t terrace_static_scratch_bytes(void);
+TERRACE_API int terrace_k1_arrival_static(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
+                                          int64_t row_bytes, int gate_bytes, int quota, int epr, int rpn,
+                                          int my_local, void *send_buf, void *gate_pairs, int64_t *r_idx,
+                                          int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status,
+                                          terrace_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -103,6 +103,7 @@ const char *terrace_strerror(int status) {
         case TERRACE_EINVAL: return "invalid argument (geometry, null pointer or unsupported size)";
         case TERRACE_ENOSPC: return "workspace too small";
         case TERRACE_ELAUNCH: return "HIP kernel launch failed";
+        case TERRACE_E2BIG: return "input larger than the fixed scratch of the no-allocation entry point";
         default: return "unknown status";
     }
 }

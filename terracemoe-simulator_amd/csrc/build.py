@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 LIB_DIR = os.path.join(os.path.dirname(HERE), "lib")
 OBJ_DIR = os.path.join(HERE, "build")
-SOURCES = ["rows.hip", "sort.hip", "pack.hip", "expand.hip", "route.hip", "api.hip"]
+SOURCES = ["rows.hip", "sort.hip", "pack.hip", "expand.hip", "route.hip", "noalloc.hip", "api.hip"]
 LIB = os.path.join(LIB_DIR, "libterrace_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -17,7 +17,7 @@ ENV_LIB = "TERRACE_OPS_LIB"
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_DIR = os.path.join(os.path.dirname(PKG_DIR), "lib")
 
-OK, EINVAL, ENOSPC, ELAUNCH = 0, -22, -28, -5
+OK, EINVAL, ENOSPC, ELAUNCH, E2BIG = 0, -22, -28, -5, -7
 F32, BF16, F16, FP8_B128 = 0, 1, 2, 3
 MODE_CODES = {"full": 0, "group_limited": 1, "quota_only": 2, "global_topk": 3}
 FORCE_GENERIC = 0x100
@@ -79,6 +79,9 @@ SIGNATURES = {
     "terrace_routing_map_count": (_I, [_P, _L, _I, _P, _P]),
     "terrace_routing_map_topk": (_I, [_P, _P, _I, _L, _I, _I, _P, _P, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
+    "terrace_static_scratch_bytes": (_Z, []),
+    "terrace_k1_arrival_static": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I,
+                                       _P, _P, _P, _P, _P, _P, _P, _P]),
 }
 
 

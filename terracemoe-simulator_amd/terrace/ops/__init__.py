@@ -158,6 +158,31 @@ def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=
     return out + (pair_pos,) if want_pair_pos else out
 
 
+def k1_arrival_static(rx, rslot, rgate, quota, epr, rpn, my_local, out):
+    """The arrival chain through the entry point that allocates nothing: ``out`` is the tuple of caller-made
+    tensors (send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos, status) it fills, and the scratch the kernels
+    need is a fixed array inside the library (so calls on one GPU must not overlap).  Inputs must already be
+    contiguous; nothing here creates a tensor.  Raises RuntimeError when the input is larger than that array holds."""
+    _require()
+    send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos, st = out
+    _hip.need_device(rx, rslot, rgate, *out)
+    _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local)
+    if not all(t.is_contiguous() for t in (rx, rslot, rgate) + tuple(out)):
+        raise RuntimeError("k1_arrival_static: every tensor must be contiguous (the call makes no copies)")
+    R, P = rslot.shape[0], rslot.shape[0] * quota
+    if (tuple(send_buf.shape) != (P, rx.shape[1]) or send_buf.dtype != rx.dtype or gate_pairs.numel() != P
+            or gate_pairs.dtype != rgate.dtype or i_send.numel() != rpn or st.numel() < _hip.STATUS_WORDS
+            or st.dtype != torch.int32
+            or any(t.numel() != P or t.dtype != torch.int64 for t in (r_idx, slot_idx, pair_pos))
+            or i_send.dtype != torch.int64):
+        raise RuntimeError("k1_arrival_static: an output tensor has the wrong shape or dtype")
+    _hip.call("terrace_k1_arrival_static", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R,
+              rx.shape[1] * rx.element_size(), rgate.element_size(), quota, epr, rpn, my_local, _hip.ptr(send_buf),
+              _hip.ptr(gate_pairs), _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(pair_pos),
+              _hip.ptr(st), _hip.stream(rx.device))
+    return out
+
+
 def _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
     """Refusals of terrace/ops/k2_ref.py:87-108 (same exception classes), minus the id-range
     read-back (reported through the status words instead) and the 63-slot mask bound."""
