@@ -174,6 +174,32 @@ TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, con
                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status,
                     void *workspace, size_t workspace_bytes, terrace_stream_t stream);
 
+/* Hop-B local scatter in one pass (north-star stage 4; the arrival-side chain of terrace/ta2a_fwd.py:605-646 when
+ * every expert slot the arriving rows name is local to this GPU -- one GPU per node, or the one-GPU loop-back).
+ * Equals terrace_k1_arrival followed by terrace_regroup(epr = n_local, my_local = 0) without the [P, row_bytes]
+ * buffer between them: a stable sort by owner card and then by local expert is one stable sort by slot, so each
+ * arrived row is read once and written straight to the expert-order place of each of its `quota` pairs.
+ *   rx [R,row_bytes] (NULL: index planes only), rslot [R,quota] i64 with first_slot <= id < first_slot + n_local,
+ *   rgate [R,quota] of gate_bytes-wide elements or NULL.
+ * Pair p = r*quota+i goes to expert x = rslot[p] - first_slot; pairs of one expert keep their order in p.
+ *   capacity < 0: permuted [P,row_bytes]; place[p] = position in that order.
+ *   capacity >= 0: permuted [n_local*capacity,row_bytes]; expert x keeps its first `capacity` pairs at
+ *     x*capacity+rank, later ones are dropped (place[p] = -1, kept[p] = 0), unused places are zero rows.
+ * place [P] i64, kept [P] u8, pair_of_place [places] i64 (-1 on a padding place), permuted_gate [places] (0 on
+ * padding; written when rgate != NULL) may each be NULL.  tokens_per_expert [n_local] i64 counts before the cut;
+ * kept_per_expert [n_local] i64 may be NULL.  With rx == NULL, terrace_hopb_scatter_move moves the rows later
+ * (same geometry, same untouched workspace), like the *_move calls of the other stages. */
+TERRACE_API size_t terrace_hopb_scatter_workspace(int64_t R, int quota, int n_local);
+TERRACE_API int terrace_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
+                                     int64_t row_bytes, int gate_bytes, int quota, int first_slot, int n_local,
+                                     int64_t capacity, void *permuted, void *permuted_gate, int64_t *place,
+                                     uint8_t *kept, int64_t *pair_of_place, int64_t *tokens_per_expert,
+                                     int64_t *kept_per_expert, int32_t *status, void *workspace,
+                                     size_t workspace_bytes, terrace_stream_t stream);
+TERRACE_API int terrace_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local,
+                                          int64_t capacity, void *permuted, const void *workspace,
+                                          size_t workspace_bytes, terrace_stream_t stream);
+
 /* Row ids a caller passes to the four entry points below are never turned into an address unchecked: an id
  * outside [0, n_src) (resp. [0, n_dst), the table length) is a dead entry -- a zero row, a copy not made,
  * no contribution, -1 -- exactly like a negative one.  (The reference's x[u_src] / index_add would raise.) */

@@ -434,6 +434,46 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None):
     return padded, dest, kept, counts, np.minimum(counts, capacity)
 
 
+def hopb_local_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None):
+    """The arrival chain and the expert-order regroup of a rank whose node's slots are all local, as the
+    reference composes them (terrace/ta2a_fwd.py:605-646): ``k1_arrival`` with ``epr*rpn = n_local``, then
+    ``regroup`` over all ``n_local`` slots of what arrived.  Returned per PAIR ``p = r*quota + i`` (the
+    enumeration before the arrival reorder), which is what a one-pass kernel can know:
+
+    (permuted, place [P] i64 (-1 dropped), kept [P] bool, tokens_per_expert, kept_per_expert,
+     permuted_gate [places], pair_of_place [places] i64 (-1 on padding)).
+
+    The owner-card split is immaterial to the result (a stable sort by ``slot // epr`` then by ``slot`` is a
+    stable sort by ``slot``); it is taken with ``rpn = n_local`` cards of one expert each.
+    """
+    rslot = np.asarray(rslot, dtype=np.int64)
+    R, q = rslot.shape
+    P = R * q
+    local = rslot - first_slot
+    send_buf, gate_pairs, r_idx, slot_idx, _ = k1_arrival(rx, local, rgate, quota, 1, n_local)
+    pos = arrival_positions(local, 1, n_local)                 # pair p -> arrival position
+    ordo = np.empty_like(pos)
+    ordo[pos] = np.arange(P)                                   # arrival position -> pair
+    if capacity is None:
+        permuted, order, counts = regroup(send_buf, slot_idx, n_local)
+        place_arr = np.empty(P, dtype=np.int64)
+        place_arr[order] = np.arange(P)
+        kept_arr = np.ones(P, dtype=bool)
+        kept_per = counts.copy()
+        n_places = P
+    else:
+        permuted, place_arr, kept_arr, counts, kept_per = regroup(send_buf, slot_idx, n_local, capacity=capacity)
+        n_places = n_local * capacity
+    place = place_arr[pos]
+    kept = kept_arr[pos]
+    pair_of_place = np.full(n_places, -1, dtype=np.int64)
+    pair_of_place[place_arr[kept_arr]] = ordo[kept_arr]
+    g = np.asarray(rgate)
+    permuted_gate = np.zeros(n_places, dtype=g.dtype)
+    permuted_gate[place_arr[kept_arr]] = gate_pairs[kept_arr]
+    return permuted, place, kept, counts, kept_per, permuted_gate, pair_of_place
+
+
 # --------------------------------------------------------------------------------------
 # (5) combine -- terrace/ta2a_fwd.py:658-670 ; one level: terrace/ep_dist.py:121-122
 # --------------------------------------------------------------------------------------

@@ -38,6 +38,14 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
                 int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
                 int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
                 int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, hipStream_t s);
+size_t hopb_workspace(int64_t R, int quota, int n_local);
+int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                     int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
+                     void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
+                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *ws, size_t ws_bytes,
+                     hipStream_t s);
+int run_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local, int64_t capacity,
+                          void *permuted, const void *ws, size_t ws_bytes, hipStream_t s);
 size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m);
 int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
                 int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
@@ -229,6 +237,24 @@ int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta, int64_t P,
     return run_regroup(node_rx, my_meta, gate_plane, P, row_bytes, gate_bytes, epr, my_local, capacity, permuted,
                        permuted_gate, order, dest, kept, tokens_per_expert, kept_per_expert, status, workspace,
                        workspace_bytes, 2, 2 * (8 / gate_bytes), (hipStream_t)stream);
+}
+
+size_t terrace_hopb_scatter_workspace(int64_t R, int quota, int n_local) { return hopb_workspace(R, quota, n_local); }
+
+int terrace_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                         int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
+                         void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
+                         int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *workspace,
+                         size_t workspace_bytes, terrace_stream_t stream) {
+    return run_hopb_scatter(rx, rslot, rgate, R, row_bytes, gate_bytes, quota, first_slot, n_local, capacity, permuted,
+                            permuted_gate, place, kept, pair_of_place, tokens_per_expert, kept_per_expert, status,
+                            workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int terrace_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local, int64_t capacity,
+                              void *permuted, const void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    return run_hopb_scatter_move(rx, R, row_bytes, quota, n_local, capacity, permuted, workspace, workspace_bytes,
+                                 (hipStream_t)stream);
 }
 
 int terrace_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, int n_nodes, int groups_m,

@@ -7,39 +7,68 @@
 //   expert card item = received row   key = local expert          (expert-order regroup)
 // Unordered atomic cursors cannot give a stable order, so placement is
 //   dest = start[key] + (items with that key in earlier units) + (rank inside the unit),
-// built in three launches:
-//   count  each wave owns a contiguous "unit" of items and histograms it in wave-private LDS;
-//   scan   one workgroup turns the [unit][bucket] counts into exclusive cursors (bucket-major);
-//   rank   each wave replays its unit, ranks items with wave ballots, and emits the outputs.
+// built in two launches (three for very large tables):
+//   count  each wave owns a contiguous "unit" of items and histograms it in wave-private LDS; the workgroup
+//          leaves each unit's prefix inside the workgroup and the workgroup's totals;
+//   rank   each workgroup adds up the totals before it (a few KB from L2), each wave replays its unit, ranks
+//          items with wave ballots, and emits the outputs.
+//   (scan  tables too large for every rank workgroup to re-read: one workgroup turns the plain [unit][bucket]
+//          counts into exclusive cursors between the two.)
 // The row payload itself is moved afterwards by the scatter/gather kernels of rows.hip.
 #include "sort.hpp"
 
 namespace terrace {
 
+void finish_units(Units &u) {
+    // direct: 16-wave workgroups keep the number of workgroup totals a rank workgroup re-reads small
+    u.wpb = u.n_units >= 64 ? 16 : 4;
+    u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
+    u.direct = u.n_buckets <= kDirectMaxBuckets && (int64_t)u.n_buckets * u.n_blocks <= kDirectMaxWords;
+    if (!u.direct) {
+        u.wpb = 4;
+        u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
+    }
+}
+
 Units make_units(int64_t n_items, int n_buckets) {
     Units u;
     u.n_items = n_items;
     u.n_buckets = n_buckets;
-    // Unit size: a chunk more per wave costs the count and rank passes about 1 us, a count table four
-    // times larger costs the one-workgroup scan about 6 us (16K entries 5.5 us, 64K entries 12 us).
-    // So one chunk per wave while the table stays within 16K entries, four while it stays within 64K,
-    // sixteen beyond.
+    // Unit size.  A chunk more per wave costs the count and rank passes about 1 us; more units cost the direct
+    // path more workgroup totals to re-read and the scan path a larger table (16K entries 5.5 us, 64K entries
+    // 12 us).  One chunk per wave up to 2048 units, then four, then sixteen; when even that leaves a table
+    // the scan path must take, the scan path's own limits (16K / 64K entries) choose.
     u.chunks = 16;
-    const int64_t limit[] = {16384, 65536};
-    const int choice[] = {1, 4};
-    for (int i = 0; i < 2; ++i) {
-        if ((n_items + 64 * choice[i] - 1) / (64 * choice[i]) * n_buckets <= limit[i]) {
-            u.chunks = choice[i];
+    for (int c : {1, 4}) {
+        if ((n_items + 64 * c - 1) / (64 * c) <= 2048) {
+            u.chunks = c;
             break;
         }
     }
     u.n_units = (int)((n_items + 64 * u.chunks - 1) / (64 * u.chunks));
     if (u.n_units < 1) u.n_units = 1;
+    finish_units(u);
+    if (!u.direct) {
+        u.chunks = 16;
+        const int64_t limit[] = {16384, 65536};
+        const int choice[] = {1, 4};
+        for (int i = 0; i < 2; ++i) {
+            if ((n_items + 64 * choice[i] - 1) / (64 * choice[i]) * n_buckets <= limit[i]) {
+                u.chunks = choice[i];
+                break;
+            }
+        }
+        u.n_units = (int)((n_items + 64 * u.chunks - 1) / (64 * u.chunks));
+        if (u.n_units < 1) u.n_units = 1;
+        finish_units(u);
+    }
     return u;
 }
 
 size_t units_table_bytes(const Units &u) {
-    return align_up(((size_t)u.n_units * u.n_buckets + u.n_buckets + 1) * sizeof(int32_t), 256);
+    const size_t words = (size_t)u.n_units * u.n_buckets + u.n_buckets + 1 +
+                         (u.direct ? (size_t)u.n_buckets * u.n_blocks : 0);
+    return align_up(words * sizeof(int32_t), 256);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -70,7 +99,13 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
 };
 
 // A token's k expert ids and their nodes, in registers when k <= KMAX (KMAX > 0), else re-read
-// through L1.  Padding entries hold INT_MAX so they rank after every real id.
+// through L1.  Padding entries hold INT_MAX so they rank after every real id.  An id is narrowed only after its
+// 64-bit value has been bounded: a negative one becomes -1 and one beyond the int range INT_MAX - 1, so neither
+// can alias a valid expert and both are reported as out of range by whoever tests the id.
+__device__ __forceinline__ int narrow_id(int64_t x) {
+    return x < 0 ? -1 : (x > 0x7FFFFFFE ? 0x7FFFFFFE : (int)x);
+}
+
 template <int KMAX>
 struct RowIds {
     int v[KMAX > 0 ? KMAX : 1];
@@ -84,35 +119,43 @@ struct RowIds {
         if constexpr (KMAX > 0) {
 #pragma unroll
             for (int j = 0; j < KMAX; ++j) {
-                v[j] = j < k ? (int)r[j] : 0x7FFFFFFF;
-                nd[j] = j < k ? v[j] / slots : 0x7FFFFFFF;
+                v[j] = j < k ? narrow_id(r[j]) : 0x7FFFFFFF;
+                nd[j] = j < k ? (v[j] < 0 ? -1 : v[j] / slots) : 0x7FFFFFFF;
             }
         }
     }
     __device__ __forceinline__ int at(int j) const {
         if constexpr (KMAX > 0) return v[j];
-        else return (int)row[j];
+        else return narrow_id(row[j]);
     }
     __device__ __forceinline__ int node(int j) const {
         if constexpr (KMAX > 0) return nd[j];
-        else return (int)row[j] / slots;
+        else {
+            const int e = narrow_id(row[j]);
+            return e < 0 ? -1 : e / slots;
+        }
     }
 };
 
+// Ascending rank of column j inside the row by (id, column): equal ids keep their column order, so the ranks of a
+// row are always a permutation of 0..k-1.
 template <int KMAX>
 __device__ __forceinline__ int rank_in_row(const RowIds<KMAX> &ids, int j) {
     const int e = ids.at(j);
     int r = 0;
     if constexpr (KMAX > 0) {
 #pragma unroll
-        for (int i = 0; i < KMAX; ++i) r += (ids.v[i] < e) ? 1 : 0;
+        for (int i = 0; i < KMAX; ++i) r += (ids.v[i] < e || (ids.v[i] == e && i < j)) ? 1 : 0;
     } else {
-        for (int i = 0; i < ids.k; ++i) r += (ids.at(i) < e) ? 1 : 0;
+        for (int i = 0; i < ids.k; ++i) {
+            const int o = ids.at(i);
+            r += (o < e || (o == e && i < j)) ? 1 : 0;
+        }
     }
     return r;
 }
 
-// Column of the element whose ascending rank inside the row is `want` (-1 if none: duplicates).
+// Column of the element whose ascending rank inside the row is `want`.
 template <int KMAX>
 __device__ __forceinline__ int column_with_rank(const RowIds<KMAX> &ids, int want) {
     int found = -1;
@@ -178,41 +221,52 @@ __device__ __forceinline__ int bits_for(int n_buckets) { return n_buckets <= 1 ?
 // count: table is bucket-major, table[b * n_units + unit]
 // ---------------------------------------------------------------------------------------------
 template <typename KeyFn, int CH>
-__global__ __launch_bounds__(kBlock) void count_kernel(KeyFn key_of, Units u, int32_t *__restrict__ table) {
+__global__ __launch_bounds__(kSortBlockMax) void count_kernel(KeyFn key_of, Units u, int32_t *__restrict__ table,
+                                                              int32_t *__restrict__ status) {
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
     const int w = wave_in_block();
     lds_i32 *hist = (lds_i32 *)lds + w * u.n_buckets;
-    const int unit = blockIdx.x * kWavesPerBlock + w;
-    if (unit >= u.n_units) return;
-    const int key_bits = bits_for(u.n_buckets);
-    const int64_t first = (int64_t)unit * CH * kWave;
-    int64_t fetched[CH];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {       // every chunk's load is issued before any key is computed
-        const int64_t item = first + (int64_t)c * kWave + lane;
-        fetched[c] = key_of.fetch(item < u.n_items ? item : u.n_items - 1);
-    }
-    int keys[CH];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int64_t item = first + (int64_t)c * kWave + lane;
-        bool bad = false;
-        const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
-        keys[c] = item < u.n_items ? key : -1;
-    }
+    const int unit = blockIdx.x * u.wpb + w;
+    const bool active = unit < u.n_units;           // an idle wave of the last workgroup still holds zero counts
+    if (!active && !u.direct) return;
     for (int b = lane; b < u.n_buckets; b += kWave) hist[b] = 0;
     __builtin_amdgcn_wave_barrier();
+    if (active) {
+        const int key_bits = bits_for(u.n_buckets);
+        const int64_t first = (int64_t)unit * CH * kWave;
+        int64_t fetched[CH];
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int key = keys[c];
-        const bool valid = key >= 0;
-        const uint64_t peers = same_key_lanes(key, valid, key_bits);
-        // the lowest lane of each key adds the key's count: distinct keys, distinct words
-        if (valid && lane == __builtin_ctzll(peers)) hist[key] = hist[key] + __popcll(peers);
-        __builtin_amdgcn_wave_barrier();
+        for (int c = 0; c < CH; ++c) {       // every chunk's load is issued before any key is computed
+            const int64_t item = first + (int64_t)c * kWave + lane;
+            fetched[c] = key_of.fetch(item < u.n_items ? item : u.n_items - 1);
+        }
+        int keys[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int64_t item = first + (int64_t)c * kWave + lane;
+            bool bad = false;
+            const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
+            keys[c] = item < u.n_items ? key : -1;
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int key = keys[c];
+            const bool valid = key >= 0;
+            const uint64_t peers = same_key_lanes(key, valid, key_bits);
+            // the lowest lane of each key adds the key's count: distinct keys, distinct words
+            if (valid && lane == __builtin_ctzll(peers)) hist[key] = hist[key] + __popcll(peers);
+            __builtin_amdgcn_wave_barrier();
+        }
     }
-    for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)b * u.n_units + unit] = hist[b];
+    if (!u.direct) {
+        for (int b = lane; b < u.n_buckets; b += kWave) table[(int64_t)b * u.n_units + unit] = hist[b];
+        return;
+    }
+    // the rank launch accumulates into the status block; nothing but this launch is ordered before it
+    if (status && blockIdx.x == 0 && threadIdx.x < TERRACE_STATUS_WORDS) status[threadIdx.x] = 0;
+    __syncthreads();
+    direct_block_counts(u, table, (lds_i32 *)lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -384,15 +438,19 @@ void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_
 // rank
 // ---------------------------------------------------------------------------------------------
 template <typename KeyFn, typename EmitFn, int CH>
-__global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit, Units u,
-                                                      const int32_t *__restrict__ table,
-                                                      int32_t *__restrict__ status) {
+__global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitFn emit, Units u,
+                                                             int32_t *__restrict__ table,
+                                                             int64_t *__restrict__ hist_i64,
+                                                             float *__restrict__ hist_f32,
+                                                             int64_t *__restrict__ offsets_i64,
+                                                             int32_t *__restrict__ status) {
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
     const int w = wave_in_block();
     lds_i32 *cursor = (lds_i32 *)lds + w * u.n_buckets;
-    const int unit = blockIdx.x * kWavesPerBlock + w;
-    if (unit >= u.n_units) return;
+    const int unit = blockIdx.x * u.wpb + w;
+    const bool active = unit < u.n_units;
+    if (!active && !u.direct) return;
     const int key_bits = bits_for(u.n_buckets);
     const int64_t first = (int64_t)unit * CH * kWave;
     int fault = 0;
@@ -406,6 +464,31 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
         fetched[c] = key_of.fetch(safe);
         pre[c] = emit.fetch(safe);
     }
+    const int32_t *start = table + units_start_at(u);
+    if (u.direct) {
+        // this unit's prefixes inside its workgroup: loaded now, with the keys, so that the only memory round trip
+        // of the kernel is the one the workgroup totals below share with them
+        constexpr int kTabRegs = kDirectMaxBuckets / kWave;
+        int32_t tab[kTabRegs];
+#pragma unroll
+        for (int i = 0; i < kTabRegs; ++i) {
+            const int b = lane + i * kWave;
+            tab[i] = (active && b < u.n_buckets) ? table[(int64_t)b * u.n_units + unit] : 0;
+        }
+        lds_i32 *shared = (lds_i32 *)lds + u.wpb * u.n_buckets;          // tot, base, start
+        lds_i32 *base = shared + u.n_buckets, *lstart = base + u.n_buckets;
+        direct_block_base(u, table, (int)blockIdx.x, blockIdx.x == 0, shared, base, lstart, hist_i64, hist_f32,
+                          offsets_i64);
+        if (!active) return;
+#pragma unroll
+        for (int i = 0; i < kTabRegs; ++i) {
+            const int b = lane + i * kWave;
+            if (b < u.n_buckets) cursor[b] = base[b] + tab[i];
+        }
+        start = (const int32_t *)lstart;
+    } else {
+        for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)b * u.n_units + unit];
+    }
     int keys[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -415,9 +498,7 @@ __global__ __launch_bounds__(kBlock) void rank_kernel(KeyFn key_of, EmitFn emit,
         keys[c] = item < u.n_items ? key : -1;
         if (bad && item < u.n_items) fault |= TERRACE_FAULT_ID_RANGE;
     }
-    for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)b * u.n_units + unit];
     __builtin_amdgcn_wave_barrier();
-    const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
     int tally[2] = {0, 0};
     // phase 2: places, in registers
     int32_t dests[CH];
@@ -517,6 +598,83 @@ struct EmitArrival {         // terrace/ops/__init__.py:287-299
         return 0;
     }
 };
+
+struct EmitHopB {            // arrival + expert-order regroup in one placement (all of the node's slots local)
+    const void *rgate;       // [R, quota] at row pitch gate_pitch (gate elements), or NULL
+    int gate_bytes, quota;
+    int64_t gate_pitch;
+    int64_t capacity;        // < 0: drop-less
+    int64_t *place;          // [P]: where pair p sits in the expert-order buffer, -1 = dropped
+    uint8_t *kept;           // [P]
+    int64_t *pair_of_place;  // [places]: the pair behind each place
+    void *permuted_gate;     // [places]
+    int32_t *pos32;          // [P]: `place` for the row mover
+    static constexpr bool kTallies = false;
+    struct Pre { uint32_t gbits; };
+    __device__ __forceinline__ Pre fetch(int64_t p) const {
+        Pre pre{0u};
+        if (rgate) {
+            const uint32_t r = (uint32_t)p / (uint32_t)quota;
+            const int64_t at = (int64_t)r * gate_pitch + (int64_t)((uint32_t)p - r * (uint32_t)quota);
+            pre.gbits = gate_bytes == 4 ? ((const uint32_t *)rgate)[at] : (uint32_t)((const uint16_t *)rgate)[at];
+        }
+        return pre;
+    }
+    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre pre,
+                                              const int32_t *start, int *) const {
+        int64_t d = dest;
+        bool keep = true;
+        if (capacity >= 0) {
+            const int64_t rank = dest - start[key];
+            keep = rank < capacity;
+            d = keep ? key * capacity + rank : -1;
+        }
+        pos32[p] = (int32_t)d;
+        if (place) place[p] = d;
+        if (kept) kept[p] = keep ? 1 : 0;
+        if (keep) {
+            if (pair_of_place) pair_of_place[d] = p;
+            if (rgate && permuted_gate) {
+                if (gate_bytes == 4) ((uint32_t *)permuted_gate)[d] = pre.gbits;
+                else ((uint16_t *)permuted_gate)[d] = (uint16_t)pre.gbits;
+            }
+        }
+        return 0;
+    }
+};
+
+// The places of a capacity layout that hold no row: zero rows, zero gates, no pair.  blockIdx.x = x * chunks + c
+// looks after places [c * kPadRows, (c + 1) * kPadRows) of expert x and leaves at once when they are all in use;
+// the first workgroup of an expert also writes kept_per_expert.
+constexpr int kPadRows = 16;
+template <typename V>
+__global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restrict__ start, int epr, int64_t capacity,
+                                                          int chunks, V *__restrict__ rows, int64_t row_vecs,
+                                                          void *__restrict__ gate_plane, int gate_bytes,
+                                                          int64_t *__restrict__ pair_of_place,
+                                                          int64_t *__restrict__ kept_per_expert) {
+    const int x = blockIdx.x / chunks, c = blockIdx.x - x * chunks;
+    const int64_t count = start[x + 1] - start[x];
+    const int64_t used = count < capacity ? count : capacity;
+    if (c == 0 && threadIdx.x == 0 && kept_per_expert) kept_per_expert[x] = used;
+    int64_t lo = (int64_t)c * kPadRows, hi = lo + kPadRows;
+    if (lo < used) lo = used;
+    if (hi > capacity) hi = capacity;
+    if (lo >= hi) return;
+    const int64_t first = x * capacity + lo, n = hi - lo;
+    for (int64_t i = threadIdx.x; i < n; i += kBlock) {
+        if (pair_of_place) pair_of_place[first + i] = -1;
+        if (gate_plane) {
+            if (gate_bytes == 4) ((uint32_t *)gate_plane)[first + i] = 0u;
+            else ((uint16_t *)gate_plane)[first + i] = (uint16_t)0;
+        }
+    }
+    if (!rows) return;
+    V *o = rows + first * row_vecs;
+    V z;
+    __builtin_memset(&z, 0, sizeof(V));
+    for (int64_t i = threadIdx.x; i < n * row_vecs; i += kBlock) __builtin_nontemporal_store(z, o + i);
+}
 
 struct EmitPairs {           // terrace/ta2a_fwd.py:605-628, general branch: pairs come as (row, slot) lists
     const int64_t *r_in, *slot_in;
@@ -728,6 +886,10 @@ __global__ __launch_bounds__(kBlock) void fill_zero_kernel(uint8_t *__restrict__
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0;
 }
 
+__global__ __launch_bounds__(kBlock) void fill_minus_one_kernel(int64_t *__restrict__ p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = -1;
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gather_elems_kernel(const T *__restrict__ src,
                                                               const int32_t *__restrict__ idx, int64_t n,
@@ -801,22 +963,29 @@ __global__ __launch_bounds__(kBlock) void pack_quota_wire_kernel(const int64_t *
 // ---------------------------------------------------------------------------------------------
 // host drivers
 // ---------------------------------------------------------------------------------------------
-static int blocks_for_units(const Units &u) { return (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock; }
-static size_t lds_for(const Units &u) { return (size_t)kWavesPerBlock * u.n_buckets * sizeof(int32_t); }
+static size_t lds_count(const Units &u) { return (size_t)u.wpb * u.n_buckets * sizeof(int32_t); }
+static size_t lds_rank(const Units &u) {
+    return ((size_t)u.wpb * u.n_buckets + (u.direct ? 3 * (size_t)u.n_buckets + 1 : 0)) * sizeof(int32_t);
+}
 
 template <typename KeyFn, typename EmitFn>
-static int run_sort(const KeyFn &key, const EmitFn &emit, const Units &u, int32_t *table, int64_t *hist,
+static int run_sort(const KeyFn &key, const EmitFn &emit, Units u, int32_t *table, int64_t *hist,
                     float *hist_f, int64_t *offsets, int32_t *status, bool do_rank, hipStream_t s) {
-    const int blocks = blocks_for_units(u);
-    const size_t lds = lds_for(u);
-    if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, kBlock, lds, s>>>(key, u, table);
-    else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, kBlock, lds, s>>>(key, u, table);
-    else count_kernel<KeyFn, 16><<<blocks, kBlock, lds, s>>>(key, u, table);
-    launch_scan(u, table, hist, hist_f, offsets, status, s);
+    if (!do_rank && u.direct) {          // the histogram alone: the scan launch writes it, so take that path
+        u.direct = 0;                    // (the table region of a direct layout is large enough for it)
+        u.wpb = 4;
+        u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
+    }
+    const int blocks = u.n_blocks, threads = u.wpb * kWave;
+    const size_t lc = lds_count(u), lr = lds_rank(u);
+    if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, threads, lc, s>>>(key, u, table, status);
+    else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, threads, lc, s>>>(key, u, table, status);
+    else count_kernel<KeyFn, 16><<<blocks, threads, lc, s>>>(key, u, table, status);
+    if (!u.direct) launch_scan(u, table, hist, hist_f, offsets, status, s);
     if (do_rank) {
-        if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
-        else if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
-        else rank_kernel<KeyFn, EmitFn, 16><<<blocks, kBlock, lds, s>>>(key, emit, u, table, status);
+        if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
+        else if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
+        else rank_kernel<KeyFn, EmitFn, 16><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
     }
     return check_launch();
 }
@@ -917,6 +1086,115 @@ int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_i
     return launch_gather_rows<int32_t>(rx, send_buf, src32, P, row_bytes, R, s);
 }
 
+// ---- Hop-B local scatter in one pass ------------------------------------------------------------
+// = run_k1_arrival followed by run_regroup over all n_local slots of the node, without the buffer between them:
+// a stable sort by owner card and then by local expert is one stable sort by slot.
+typedef uint32_t pad_u32x4 __attribute__((ext_vector_type(4)));
+
+size_t hopb_workspace(int64_t R, int quota, int n_local) {
+    const int64_t P = R * quota;
+    if (P <= 0 || n_local <= 0 || n_local > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(P, n_local)) + align_up((size_t)P * sizeof(int32_t), 256);
+}
+
+static int launch_zero_pad(const int32_t *start, int epr, int64_t capacity, void *rows, int64_t row_bytes,
+                           void *gate_plane, int gate_bytes, int64_t *pair_of_place, int64_t *kept_per_expert,
+                           hipStream_t s) {
+    if (epr <= 0) return TERRACE_OK;
+    const int chunks = capacity > 0 ? (int)((capacity + kPadRows - 1) / kPadRows) : 1;
+    const int64_t blocks = (int64_t)epr * chunks;
+    if (blocks >= (int64_t)1 << 31) return TERRACE_EINVAL;
+    if (!rows || row_bytes == 0) {
+        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, nullptr, 0,
+                                                                    gate_plane, gate_bytes, pair_of_place,
+                                                                    kept_per_expert);
+    } else if ((((uintptr_t)rows | (uintptr_t)row_bytes) & 15) == 0) {
+        zero_pad_kernel<pad_u32x4><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, (pad_u32x4 *)rows,
+                                                                      row_bytes / 16, gate_plane, gate_bytes,
+                                                                      pair_of_place, kept_per_expert);
+    } else {
+        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, (uint8_t *)rows,
+                                                                    row_bytes, gate_plane, gate_bytes, pair_of_place,
+                                                                    kept_per_expert);
+    }
+    return check_launch();
+}
+
+int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
+                     int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
+                     void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
+                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *ws, size_t ws_bytes,
+                     hipStream_t s) {
+    if (R < 0 || quota <= 0 || n_local <= 0 || n_local > kMaxBuckets || first_slot < 0 || !tokens_per_expert ||
+        (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0 ||
+        (capacity >= 0 && (int64_t)n_local * capacity >= (int64_t)1 << 31))
+        return TERRACE_EINVAL;
+    if (R > (((int64_t)1 << 31) - 1) / quota) return TERRACE_EINVAL;
+    const int64_t P = R * quota;
+    const int64_t places = capacity >= 0 ? (int64_t)n_local * capacity : P;
+    if (places > 0 && rx && !permuted) return TERRACE_EINVAL;
+    if (P == 0) {
+        int rc = empty_outputs(tokens_per_expert, nullptr, kept_per_expert, n_local, status, s);
+        if (rc != TERRACE_OK || places == 0) return rc;
+        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        if (permuted_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
+        if (pair_of_place) fill_minus_one_kernel<<<64, kBlock, 0, s>>>(pair_of_place, places);
+        return check_launch();
+    }
+    if (!rslot || !ws) return TERRACE_EINVAL;
+    const Units u = make_units(P, n_local);
+    const size_t table_bytes = units_table_bytes(u);
+    if (ws_bytes < hopb_workspace(R, quota, n_local)) return TERRACE_ENOSPC;
+    int32_t *table = (int32_t *)ws;
+    int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
+    KeyAffine key{rslot, (int64_t)first_slot, 1, n_local, quota, (int64_t)quota};
+    EmitHopB emit{rgate, gate_bytes, quota, (int64_t)quota, capacity, place, kept, pair_of_place,
+                  rgate ? permuted_gate : nullptr, pos32};
+    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
+    if (rc != TERRACE_OK) return rc;
+    const int32_t *start = table + units_start_at(u);
+    if (capacity >= 0) {
+        // padding planes now; the padding rows with the row mover (they may be moved later, by the _move call)
+        rc = launch_zero_pad(start, n_local, capacity, rx ? permuted : nullptr, rx ? row_bytes : 0,
+                             rgate ? permuted_gate : nullptr, gate_bytes, pair_of_place, kept_per_expert, s);
+        if (rc != TERRACE_OK) return rc;
+    } else if (kept_per_expert) {
+        capacity_index_kernel<<<(n_local + kBlock - 1) / kBlock, kBlock, 0, s>>>(nullptr, start, n_local, INT64_MAX, 0,
+                                                                                nullptr, kept_per_expert);
+        rc = check_launch();
+        if (rc != TERRACE_OK) return rc;
+    }
+    if (!rx) return rc;
+    return launch_scatter_rows<int32_t>(rx, permuted, pos32, R, quota, row_bytes, places, s);
+}
+
+int run_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local, int64_t capacity,
+                          void *permuted, const void *ws, size_t ws_bytes, hipStream_t s) {
+    if (R < 0 || quota <= 0 || n_local <= 0 || n_local > kMaxBuckets || row_bytes < 0 ||
+        (capacity >= 0 && (int64_t)n_local * capacity >= (int64_t)1 << 31))
+        return TERRACE_EINVAL;
+    if (R > (((int64_t)1 << 31) - 1) / quota) return TERRACE_EINVAL;
+    const int64_t P = R * quota;
+    const int64_t places = capacity >= 0 ? (int64_t)n_local * capacity : P;
+    if (places == 0 || row_bytes == 0) return TERRACE_OK;
+    if (!permuted) return TERRACE_EINVAL;
+    if (P == 0) {       // all padding
+        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        return check_launch();
+    }
+    if (!rx || !ws) return TERRACE_EINVAL;
+    if (ws_bytes < hopb_workspace(R, quota, n_local)) return TERRACE_ENOSPC;
+    const Units u = make_units(P, n_local);
+    const int32_t *table = (const int32_t *)ws;
+    const int32_t *pos32 = (const int32_t *)((const char *)ws + units_table_bytes(u));
+    if (capacity >= 0) {
+        int rc = launch_zero_pad(table + units_start_at(u), n_local, capacity, permuted, row_bytes, nullptr, 4, nullptr,
+                                 nullptr, s);
+        if (rc != TERRACE_OK) return rc;
+    }
+    return launch_scatter_rows<int32_t>(rx, permuted, pos32, R, quota, row_bytes, places, s);
+}
+
 // ---- expert-order regroup ---------------------------------------------------------------------
 size_t regroup_workspace(int64_t P, int epr, int64_t capacity) {
     if (P <= 0 || epr <= 0 || epr > kMaxBuckets) return 256;
@@ -955,7 +1233,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *src_of_place = order32;
-    const int32_t *start = table + (int64_t)u.n_units * u.n_buckets;
+    const int32_t *start = table + units_start_at(u);
     if (capacity >= 0) {
         const int64_t n = places > epr ? places : epr;
         capacity_index_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(order32, start, epr, capacity,
@@ -1001,7 +1279,7 @@ size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m) {
     const int64_t S = T * groups_m;
     if (S <= 0 || n_nodes <= 0 || n_nodes > kMaxBuckets) return 256;
     const size_t item_path = units_table_bytes(make_units(S, n_nodes)) + align_up((size_t)S * sizeof(int32_t), 256);
-    const size_t token_path = k2_token_path_applies(k, n_nodes) ? k2_token_workspace(T, n_nodes, groups_m) : 0;
+    const size_t token_path = k2_token_path_applies(T, k, n_nodes) ? k2_token_workspace(T, n_nodes, groups_m) : 0;
     return item_path > token_path ? item_path : token_path;
 }
 
@@ -1040,7 +1318,7 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
     if (S == 0) return empty_outputs(node_counts, nullptr, node_offsets, n_nodes, status, s);
     if (!expert_idx || !mask || !u_src || !ws || (hidden && !payload) || (gates && !gate_rows)) return TERRACE_EINVAL;
     if (ws_bytes < k2_workspace(T, k, n_nodes, groups_m)) return TERRACE_ENOSPC;
-    if (k2_token_path_applies(k, n_nodes))
+    if (k2_token_path_applies(T, k, n_nodes))
         return run_k2_token(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts,
                             groups_m, payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets,
                             pair_table, sort_order, token_rows, gate_sorted, status, ws, mask_pitch, gate_pitch,
@@ -1073,7 +1351,7 @@ int run_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, in
     if (S == 0 || row_bytes == 0) return TERRACE_OK;
     if (!hidden || !payload || !ws) return TERRACE_EINVAL;
     if (ws_bytes < k2_workspace(T, k, n_nodes, groups_m)) return TERRACE_ENOSPC;
-    const int32_t *pos32 = k2_token_path_applies(k, n_nodes)
+    const int32_t *pos32 = k2_token_path_applies(T, k, n_nodes)
                                ? k2_token_positions(ws, T, n_nodes)
                                : (const int32_t *)((const char *)ws + units_table_bytes(make_units(S, n_nodes)));
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);

@@ -8,22 +8,121 @@ namespace terrace {
 constexpr int kMaxBuckets = 2048;
 constexpr int kScanThreads = 1024;
 
-// A "unit" is the contiguous run of items one wave owns: chunks * 64 of them.
+// A "unit" is the contiguous run of items one wave owns: chunks * 64 of them.  The count and rank kernels
+// run `wpb` waves (units) per workgroup.
+//
+// Two ways from counts to cursors:
+//   direct  the count kernel leaves, per unit, the exclusive prefix of the counts inside its workgroup and, per
+//           workgroup, the workgroup's totals (blocktot, bucket-major); every rank workgroup then adds up the
+//           totals of all buckets before its own and of the workgroups before itself -- n_buckets * n_blocks
+//           words from L2 -- and no launch stands between count and rank;
+//   scan    the count kernel leaves plain per-unit counts and a one-workgroup scan launch turns the whole table
+//           into cursors (tables too large for every workgroup to re-read).
 struct Units {
     int64_t n_items;
     int chunks;       // 64-item chunks per unit: 1, 4 or 16, growing with the item count
     int n_units;
     int n_buckets;
+    int wpb;          // waves per workgroup of the count / rank kernels (4 or 16)
+    int n_blocks;     // their grid
+    int direct;       // 1: no scan launch (see above)
 };
 
-Units make_units(int64_t n_items, int n_buckets);
-size_t units_table_bytes(const Units &u);
+constexpr int kDirectMaxBuckets = 256;
+constexpr int kDirectMaxWords = 16384;   // n_buckets * n_blocks a rank workgroup may re-read
 
-// Exclusive prefix over the bucket-major count table table[b * n_units + unit], in place; also
+Units make_units(int64_t n_items, int n_buckets);
+// Fills wpb / n_blocks / direct from n_units and n_buckets.
+void finish_units(Units &u);
+size_t units_table_bytes(const Units &u);
+// Words of the table region: [n_units * n_buckets] counts or prefixes, then start[n_buckets + 1], then (direct)
+// blocktot[n_buckets * n_blocks].
+__host__ __device__ inline int64_t units_start_at(const Units &u) { return (int64_t)u.n_units * u.n_buckets; }
+__host__ __device__ inline int64_t units_blocktot_at(const Units &u) { return units_start_at(u) + u.n_buckets + 1; }
+
+// Scan path: exclusive prefix over the bucket-major count table table[b * n_units + unit], in place; also
 // start[b] (n_buckets + 1 int32 right after the table), the optional histogram / offsets planes
 // and a zeroed status block.
 void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
                  int32_t *status, hipStream_t s);
+
+constexpr int kSortBlockMax = 1024;      // 16 waves: the widest count / rank workgroup
+
+// Direct path, rank side: called by every thread of a workgroup (any whole number of waves) before it places
+// anything of count workgroup `me`.  From the workgroup totals the count kernel left it derives, into LDS,
+//   start[b]  first place of bucket b (n_buckets + 1 entries, the last one the item total),
+//   base[b]   first place of the items of bucket b that count workgroup `me` holds,
+// using tot[n_buckets] as scratch; with `publish` it also writes start[] after the table and fills the caller's
+// histogram / offsets planes (exactly one workgroup of a launch does).  A unit's cursor is then
+// base[b] + table[b * n_units + unit].
+__device__ __forceinline__ void direct_block_base(const Units &u, int32_t *__restrict__ table, int me, bool publish,
+                                                  lds_i32 *tot, lds_i32 *base, lds_i32 *start,
+                                                  int64_t *__restrict__ hist_i64, float *__restrict__ hist_f32,
+                                                  int64_t *__restrict__ offsets_i64) {
+    const int lane = lane_id(), w = wave_in_block(), nw = (int)(blockDim.x >> 6);
+    const int32_t *blocktot = table + units_blocktot_at(u);
+    for (int b = w; b < u.n_buckets; b += nw) {            // one wave per bucket: no two waves share a word
+        int t = 0, before = 0;
+        for (int blk = lane; blk < u.n_blocks; blk += kWave) {
+            const int v = blocktot[(int64_t)b * u.n_blocks + blk];
+            t += v;
+            before += blk < me ? v : 0;
+        }
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            t += __shfl_xor(t, d, kWave);
+            before += __shfl_xor(before, d, kWave);
+        }
+        if (lane == 0) {
+            tot[b] = t;
+            base[b] = before;
+        }
+    }
+    __syncthreads();
+    if (w == 0) {
+        int carry = 0;
+        for (int b0 = 0; b0 < u.n_buckets; b0 += kWave) {
+            const int b = b0 + lane;
+            const int v = b < u.n_buckets ? tot[b] : 0;
+            const int incl = wave_inclusive_scan(v);
+            if (b < u.n_buckets) {
+                start[b] = carry + incl - v;
+                base[b] = base[b] + carry + incl - v;
+            }
+            carry += __shfl(incl, kWave - 1, kWave);
+        }
+        if (lane == 0) start[u.n_buckets] = carry;
+    }
+    __syncthreads();
+    if (publish) {
+        int32_t *start_out = table + units_start_at(u);
+        for (int b = threadIdx.x; b <= u.n_buckets; b += blockDim.x) {
+            const int32_t s0 = start[b];
+            start_out[b] = s0;
+            if (b == u.n_buckets) break;
+            const int32_t c = tot[b];
+            if (hist_i64) hist_i64[b] = c;
+            if (hist_f32) hist_f32[b] = (float)c;
+            if (offsets_i64) offsets_i64[b] = s0;
+        }
+    }
+}
+
+// Direct path, count side: called by every thread of a count workgroup once its waves' per-bucket counts sit in
+// LDS (counts[wave * n_buckets + b], idle waves hold zeros) and a __syncthreads() has passed.  Writes each unit's
+// exclusive prefix inside the workgroup and the workgroup's totals.
+__device__ __forceinline__ void direct_block_counts(const Units &u, int32_t *__restrict__ table, lds_i32 *counts) {
+    const int nw = (int)(blockDim.x >> 6), me = (int)blockIdx.x;
+    int32_t *blocktot = table + units_blocktot_at(u);
+    for (int i = threadIdx.x; i < nw * u.n_buckets; i += blockDim.x) {
+        const int ww = i / u.n_buckets, b = i - ww * u.n_buckets;
+        int run = 0;
+        for (int x = 0; x < ww; ++x) run += counts[x * u.n_buckets + b];
+        const int un = me * nw + ww;
+        if (un < u.n_units) table[(int64_t)b * u.n_units + un] = run;
+        if (ww == nw - 1) blocktot[(int64_t)b * u.n_blocks + me] = run + counts[ww * u.n_buckets + b];
+    }
+}
 
 // n_dst / n_src bound the row ids the movers accept: an id outside [0, bound) is a dead entry.
 template <typename I>
@@ -33,9 +132,10 @@ template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, int64_t n_src,
                        hipStream_t s);
 
-// Send side with one lane per token (n_nodes <= 64, k <= 16); returns false when the geometry
-// is outside that and the caller must take the (token, run)-item path.
-bool k2_token_path_applies(int k, int n_nodes);
+// Send side with a token's node set in one 64-bit word (n_nodes <= 64, k <= 16, a count table small enough for
+// the direct path); returns false when the geometry is outside that and the caller must take the (token, run)-item
+// path.
+bool k2_token_path_applies(int64_t T, int k, int n_nodes);
 size_t k2_token_workspace(int64_t T, int n_nodes, int groups_m);
 // Where run_k2_token leaves the [T, groups_m] int32 send-row positions inside its workspace.
 const int32_t *k2_token_positions(const void *ws, int64_t T, int n_nodes);

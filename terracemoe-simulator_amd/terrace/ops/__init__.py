@@ -420,6 +420,77 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
     return out + (pgate,) if my_gate is not None else out
 
 
+def hopb_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None, want_pairs=False,
+                 workspace_out=None):
+    """Hop-B local scatter in one pass: what ``k1_arrival`` followed by ``regroup(epr=n_local)`` produce when
+    every slot the arrived rows name is local to this GPU, without the send buffer between them.
+
+    Returns a dict: ``permuted`` ([P, H], or [n_local*capacity, H] with zero padding rows), ``place`` [P]
+    (where pair ``p = r*quota + i`` sits in ``permuted``; -1 = dropped), ``kept`` [P] bool (None drop-less),
+    ``tokens_per_expert`` / ``kept_per_expert`` [n_local], ``permuted_gate`` (the gate of each place, when
+    ``rgate`` is given) and, with ``want_pairs``, ``pair_of_place`` (-1 on padding).
+
+    ``rx`` None: the index planes only; the workspace :func:`hopb_scatter_move` needs is appended to
+    ``workspace_out``."""
+    _require()
+    _hip.need_device(rx, rslot, rgate)
+    if rslot.dim() != 2 or rslot.dtype != torch.int64 or rslot.shape[1] != quota:
+        raise RuntimeError("hopb_scatter: rslot must be an int64 [R, quota] table")
+    if rx is not None and (rx.dim() != 2 or rx.shape[0] != rslot.shape[0]):
+        raise RuntimeError(f"hopb_scatter: rx {tuple(rx.shape)} does not have one row per row of rslot")
+    if rgate is not None and (tuple(rgate.shape) != tuple(rslot.shape) or rgate.element_size() not in (2, 4)):
+        raise RuntimeError("hopb_scatter: rgate must match rslot and hold 2- or 4-byte elements")
+    if not (quota > 0 and n_local > 0 and first_slot >= 0):
+        raise RuntimeError("hopb_scatter: bad geometry scalars")
+    rslot = rslot.contiguous()
+    dev = rslot.device
+    R = rslot.shape[0]
+    P = R * quota
+    cap = -1 if capacity is None else int(capacity)
+    places = P if capacity is None else n_local * cap
+    i64 = dict(dtype=torch.int64, device=dev)
+    permuted, row_bytes = None, 0
+    if rx is not None:
+        rx = rx.contiguous()
+        row_bytes = rx.shape[1] * rx.element_size()
+        permuted = torch.empty((places, rx.shape[1]), dtype=rx.dtype, device=dev)
+    pgate, gate_bytes = None, 4
+    if rgate is not None:
+        rgate = rgate.contiguous()
+        gate_bytes = rgate.element_size()
+        pgate = torch.empty((places,), dtype=rgate.dtype, device=dev)
+    place = torch.empty((P,), **i64)
+    kept = torch.empty((P,), dtype=torch.uint8, device=dev) if capacity is not None else None
+    pairs = torch.empty((places,), **i64) if want_pairs else None
+    tpe, kpe = torch.empty((n_local,), **i64), torch.empty((n_local,), **i64)
+    st = _hip.new_status(dev)
+    ws = _hip.workspace(_hip.query("terrace_hopb_scatter_workspace", R, quota, n_local), dev)
+    _hip.call("terrace_hopb_scatter", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, row_bytes, gate_bytes, quota,
+              first_slot, n_local, cap, _hip.ptr(permuted), _hip.ptr(pgate), _hip.ptr(place), _hip.ptr(kept),
+              _hip.ptr(pairs), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    if workspace_out is not None:
+        workspace_out.append(ws)
+    return {"permuted": permuted, "place": place, "kept": None if kept is None else kept.view(torch.bool),
+            "tokens_per_expert": tpe, "kept_per_expert": kpe, "permuted_gate": pgate, "pair_of_place": pairs,
+            "status": st}
+
+
+def hopb_scatter_move(rx, workspace, quota, n_local, capacity=None):
+    """Second phase of :func:`hopb_scatter` called with ``rx=None``: the expert-order buffer."""
+    _require()
+    _hip.need_device(rx, workspace)
+    if rx.dim() != 2:
+        raise RuntimeError("hopb_scatter: rx must be 2-D")
+    rx = rx.contiguous()
+    R, H = rx.shape
+    cap = -1 if capacity is None else int(capacity)
+    places = R * quota if capacity is None else n_local * cap
+    permuted = torch.empty((places, H), dtype=rx.dtype, device=rx.device)
+    _hip.call("terrace_hopb_scatter_move", _hip.ptr(rx), R, H * rx.element_size(), quota, n_local, cap,
+              _hip.ptr(permuted), _hip.ptr(workspace), workspace.numel(), _hip.stream(rx.device))
+    return permuted
+
+
 # ---- the stage operators in two phases (index planes first, rows later) -----------------------------
 def k2_pack_index(expert_idx, gates, world, n_experts, rpn, groups_m):
     """First phase of :func:`k2_pack_raw`: every index plane, no rows.  Returns
@@ -1002,5 +1073,6 @@ __all__ = [
     "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
     "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
     "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table", "pair_places",
-    "wire_words", "k2_pack_wire", "k1_arrival_wire", "regroup_wire",
+    "wire_words", "k2_pack_wire", "k1_arrival_wire", "regroup_wire", "hopb_scatter", "hopb_scatter_move",
+    "k1_arrival_static",
 ]

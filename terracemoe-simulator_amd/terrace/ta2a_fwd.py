@@ -124,6 +124,23 @@ class LoopbackState:
     capacity: int | None
 
 
+@dataclass
+class OnePassState:
+    """Dispatch state when Hop B ran as one pass (:func:`loopback_dispatch_onepass`): no arrival-order send
+    buffer exists, so ``place`` is indexed by Hop-A pair ``row*quota + i`` directly."""
+    payload: torch.Tensor
+    mask: torch.Tensor
+    gate_rows: torch.Tensor
+    u_src: torch.Tensor
+    node_counts: torch.Tensor
+    extras: dict
+    permuted: torch.Tensor
+    tokens_per_expert: torch.Tensor
+    place: torch.Tensor            # [P] by pair; -1 = dropped
+    kept: torch.Tensor | None
+    capacity: int | None
+
+
 _INDEX_STREAMS: dict = {}
 
 
@@ -211,6 +228,22 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
                          slot_idx, i_send, pair_pos, permuted, rg["tokens_per_expert"], place, rg["kept"], capacity)
 
 
+def loopback_dispatch_onepass(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8, groups_m: int = 1,
+                              capacity: int | None = None) -> OnePassState:
+    """Stages 2-4 on one GPU with Hop B as ONE pass: index build + Hop-A pack, then every packed row written
+    straight to the expert-order (capacity-padded) place of each of its pairs (``ops.hopb_scatter``).  Same
+    ``permuted`` / ``tokens_per_expert`` as :func:`loopback_dispatch` and ``place == its place[its pair_pos]``;
+    the arrival-order planes (send_buf, r_idx, slot_idx, i_send) are never formed."""
+    epr = n_experts // world
+    slots = epr * rpn
+    quota = expert_idx.shape[1] // groups_m
+    (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
+        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+    hb = _ops.hopb_scatter(payload, mask, None, quota, slots, 0, capacity)
+    return OnePassState(payload, mask, gate_rows, u_src, node_counts, extras, hb["permuted"], hb["tokens_per_expert"],
+                        hb["place"], hb["kept"], capacity)
+
+
 def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
     """Drop-less regroup that also returns each input row's place (the inverse of ``order``):
     (permuted, order, tokens_per_expert, place[, permuted_gate])."""
@@ -237,7 +270,7 @@ def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
     return out + (pgate,) if my_gate is not None else out
 
 
-def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, weights=None):
+def loopback_combine(ye, st, out_dtype=None, fp8_hidden=None, weights=None):
     """Stage 5, fused: ``y[t] = sum_s gate[t,s] * ye[place of (t, s-th smallest expert)]``.
 
     The k rows of a token are added in ascending expert id -- slot ascending inside a send row,
@@ -246,7 +279,10 @@ def loopback_combine(ye, st: LoopbackState, out_dtype=None, fp8_hidden=None, wei
     """
     where = st.extras.get("where")
     if where is None:
-        where = _ops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
+        if isinstance(st, OnePassState):
+            where = _ops.index_chain(st.place, st.extras["pair_table"])
+        else:
+            where = _ops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
     w = st.extras["gate_sorted"] if weights is None else weights
     return _ops.combine(ye, where, w, out_dtype=out_dtype, fp8_hidden=fp8_hidden)
 
@@ -262,9 +298,11 @@ def twolevel_combine(ye, st: LoopbackState, out_dtype=None):
 
 
 def ta2a_loopback_forward(x, expert_idx, gates, expert_fn, world: int, n_experts: int, rpn: int = 8,
-                          groups_m: int = 1, capacity: int | None = None):
-    """dispatch -> ``expert_fn(permuted, tokens_per_expert) -> ye`` -> combine, on one GPU."""
-    st = loopback_dispatch(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity)
+                          groups_m: int = 1, capacity: int | None = None, onepass: bool = False):
+    """dispatch -> ``expert_fn(permuted, tokens_per_expert) -> ye`` -> combine, on one GPU.  ``onepass`` runs
+    Hop B as one scatter (same ``permuted``, no arrival-order planes in the returned state)."""
+    dispatch = loopback_dispatch_onepass if onepass else loopback_dispatch
+    st = dispatch(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity)
     ye = expert_fn(st.permuted, st.tokens_per_expert)
     return loopback_combine(ye, st), st
 

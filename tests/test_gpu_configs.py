@@ -125,6 +125,20 @@ def _check_every_plane(cfg):
         if cfg.name.startswith("c4"):
             assert 0 < kept.sum() < kept.size, "the skewed workload must overflow some expert but not all"
     same(st.permuted, perm, "permuted"), same(st.place, place, "place"), same(st.tokens_per_expert, tpe, "tokens_per_expert")
+    # ---- the same Hop B as one pass: identical expert-order buffer, places named by pair
+    import terrace.ops as tops
+    from terrace.ta2a_fwd import loopback_dispatch_onepass
+    hb = tops.hopb_scatter(st.payload, st.mask, st.gate_rows, cfg.quota, cfg.slots, 0, cap, want_pairs=True)
+    o_perm, o_place, o_kept, o_tpe, o_kpe, o_pgate, o_pairs = orc.hopb_local_scatter(
+        payload, mask, gate_rows, cfg.quota, cfg.slots, 0, cap)
+    assert np.array_equal(o_perm, perm) and np.array_equal(o_place, place[pos])
+    same(hb["permuted"], perm, "one-pass permuted"), same(hb["place"], o_place, "one-pass place")
+    same(hb["tokens_per_expert"], tpe, "one-pass tokens_per_expert"), same(hb["pair_of_place"], o_pairs, "pair_of_place")
+    same(hb["permuted_gate"], o_pgate, "one-pass permuted_gate"), same(hb["kept_per_expert"], o_kpe, "kept_per_expert")
+    if cap is not None:
+        same(hb["kept"], o_kept, "one-pass kept")
+    st1 = loopback_dispatch_onepass(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    assert torch.equal(st1.permuted, st.permuted) and torch.equal(st1.place, st.place[st.pair_pos])
     # ---- experts: row * (expert id + 1) / E, or fresh fp8 rows for the fp8 workload
     n_places = perm.shape[0]
     if cfg.fmt == "fp8":
@@ -148,6 +162,8 @@ def _check_every_plane(cfg):
     want = orc.combine(ye_rows, where, wf, fmt_in, out_fmt, hidden=cfg.hidden)
     got = loopback_combine(ye, st, out_dtype=cfg.out_dtype, fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None)
     same(got, want, "combine")
+    same(loopback_combine(ye, st1, out_dtype=cfg.out_dtype, fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None), want,
+         "combine after the one-pass dispatch")
     # ---- the stated tolerance against float64
     src64 = orc.decode_rows(ye_rows, fmt_in, cfg.hidden).astype(np.float64)
     ref = np.zeros((cfg.T, cfg.hidden))
@@ -166,7 +182,7 @@ def _check_every_plane(cfg):
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
 def test_full_size_index_planes_and_round_trip(name):
     from terrace import configs
-    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, loopback_dispatch_onepass
     cfg = configs.CONFIGS[name]
     announce("full", cfg.name, cfg.T)
     inp = configs.make_inputs(cfg)
@@ -211,6 +227,13 @@ def test_full_size_index_planes_and_round_trip(name):
         used = torch.zeros(st.permuted.shape[0], dtype=torch.bool, device=DEV)
         used[pk] = True
         assert not st.permuted[~used].any(), "capacity padding rows must be zero"
+    # ---- Hop B as one pass gives the same buffer and the same places
+    st1 = loopback_dispatch_onepass(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    assert torch.equal(st1.permuted, st.permuted), "one-pass expert-order buffer differs"
+    assert torch.equal(st1.place, st.place[st.pair_pos]) and torch.equal(st1.tokens_per_expert, st.tokens_per_expert)
+    if cap is not None:
+        assert torch.equal(st1.kept, st.kept[st.pair_pos])
+    del st1
     # ---- round trip with identity experts: y[t] = x[t] * (sum of the token's kept gates)
     got = loopback_combine(st.permuted, st, out_dtype=cfg.out_dtype,
                            fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None).float()

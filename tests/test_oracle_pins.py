@@ -512,3 +512,159 @@ def test_route_gates_against_the_library_composition(E, Ng, k, M):
     local = sg.gather(1, grp[:, :, None].expand(-1, -1, E // Ng)).topk(k // M, dim=-1).indices
     want = (grp[:, :, None] * (E // Ng) + local).reshape(-1, k)
     assert np.array_equal(e, want.numpy())
+
+
+# ----------------------------------------------------------------------------- the other routing modes, pool > 2
+
+def _modes_brute(aff, bias, E, Ng, k, M, pool, mode):
+    """Definition of the three other modes and of any pool, token by token, with Python sorting on
+    (-value, index): values descending, lowest index first among equals."""
+    g = E // Ng
+    rows, grps = [], []
+    for t in range(aff.shape[0]):
+        s = [np.float32(aff[t, e]) + np.float32(bias[e]) for e in range(E)]
+        by_value = lambda ids: sorted(ids, key=lambda e: (-s[e], e))
+        if mode == "global_topk":
+            row = by_value(range(E))[:k]
+            grp = [e // g for e in row]
+        elif mode == "quota_only":
+            row = []
+            for G in range(Ng):
+                row += by_value(range(G * g, (G + 1) * g))[:k // Ng]
+            grp = list(range(Ng))
+        else:
+            score = []
+            for G in range(Ng):
+                top = sorted(s[G * g:(G + 1) * g], reverse=True)[:min(pool, g)]
+                acc = np.float32(top[0])
+                for v in top[1:]:
+                    acc = np.float32(acc + v)
+                score.append(np.float32(acc / np.float32(len(top))))
+            grp = sorted(range(Ng), key=lambda G: (-score[G], G))[:M]
+            if mode == "group_limited":
+                # candidates in the order the reference concatenates them: chosen groups in score order
+                cand = [e for G in grp for e in range(G * g, (G + 1) * g)]
+                order = sorted(range(len(cand)), key=lambda i: (-s[cand[i]], i))[:k]
+                row = [cand[i] for i in order]
+            else:
+                row = []
+                for G in grp:
+                    row += by_value(range(G * g, (G + 1) * g))[:k // M]
+        rows.append(row)
+        grps.append(grp)
+    return np.array(rows, dtype=np.int64), np.array(grps, dtype=np.int64)
+
+
+@pytest.mark.parametrize("mode", ["quota_only", "group_limited", "global_topk", "full"])
+@pytest.mark.parametrize("E,Ng,k,M,pool", [(16, 4, 4, 2, 2), (24, 3, 6, 3, 3), (32, 4, 8, 2, 4), (32, 4, 8, 4, 1),
+                                           (40, 5, 5, 1, 8), (12, 2, 4, 2, 6)])
+def test_route_every_mode_and_pool_equals_brute_force(mode, E, Ng, k, M, pool):
+    """Exact ids IN ORDER, not as sets: a version that took the lowest scores of a group, or that returned
+    group_limited's picks in index order instead of value order, fails here."""
+    if mode == "quota_only" and k % Ng:
+        pytest.skip("quota_only needs k divisible by the group count")
+    rng = np.random.default_rng(E * 7 + k + pool)
+    aff = rng.random((29, E)).astype(np.float32)
+    aff[3] = 0.25                                     # an all-tied token: lowest index first everywhere
+    aff[4, ::2] = 0.5
+    bias = (rng.standard_normal(E) * 0.3).astype(np.float32)
+    e, _, grp = orc.t_route(aff, bias, E, Ng, k, M, pool=pool, mode=mode)
+    be, bgrp = _modes_brute(aff, bias, E, Ng, k, M, pool, mode)
+    assert np.array_equal(e, be), mode
+    assert np.array_equal(grp, bgrp), mode
+
+
+@pytest.mark.parametrize("E,Ng,k,M", [(64, 8, 8, 4), (256, 8, 8, 4), (128, 16, 16, 2), (96, 8, 8, 2)])
+def test_route_other_modes_against_the_library_composition(E, Ng, k, M):
+    """quota_only and group_limited as the reference composes them from topk / gather
+    (terrace/routing.py:75-85, 99-109), evaluated by the installed torch on untied seeded inputs: exact expert
+    ids in the reference's order."""
+    g = torch.Generator().manual_seed(E * 3 + k)
+    T, gs = 2048, E // Ng
+    aff = torch.rand(T, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.1
+    s = aff + bias
+    sg = s.view(T, Ng, gs)
+    # quota_only (:99-109): top-(k/N_g) inside every group, groups ascending
+    per = k // Ng
+    local = sg.topk(per, -1).indices
+    want = (torch.arange(Ng)[None, :, None] * gs + local).reshape(T, -1)
+    e, gates, grp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, mode="quota_only")
+    assert np.array_equal(e, want.numpy())
+    assert np.array_equal(grp, torch.arange(Ng)[None].expand(T, -1).numpy())
+    raw = aff.gather(1, want)
+    lib = (raw / raw.sum(-1, keepdim=True)).numpy()
+    assert np.all(np.abs(gates - lib) <= 1e-6 * np.abs(lib))
+    # group_limited (:77-85): top-M groups by the mean of their top-2, then a free top-k over their M*g candidates
+    gsc = sg.topk(min(2, gs), -1).values.mean(-1)
+    group_idx = gsc.topk(M, -1).indices
+    cand = sg.gather(1, group_idx[..., None].expand(-1, -1, gs)).reshape(T, -1)
+    loc = cand.topk(k, -1).indices
+    flat_base = (group_idx * gs)[..., None].expand(-1, -1, gs).reshape(T, -1)
+    want = flat_base.gather(1, loc) + (loc % gs)
+    e, _, grp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, mode="group_limited")
+    assert np.array_equal(grp, group_idx.numpy())
+    assert np.array_equal(e, want.numpy())
+
+
+@pytest.mark.parametrize("pool", [3, 4, 8])
+def test_group_score_pool_beyond_two_against_the_library(pool):
+    """mean of the top-min(pool, g) (terrace/routing.py:24,88): the chosen groups are the library's on untied
+    inputs, and the score is its mean to one unit in the last place (the library's order inside a 3- to 8-term
+    sum is its own; the oracle adds from the largest down)."""
+    E, Ng, k, M = 128, 8, 8, 4
+    g = torch.Generator().manual_seed(pool)
+    aff = torch.rand(1024, E, generator=g)
+    bias = torch.zeros(E)
+    sg = (aff + bias).view(1024, Ng, E // Ng)
+    gsc = sg.topk(min(pool, E // Ng), -1).values.mean(-1)
+    mine = orc._group_scores(sg.numpy(), pool)
+    assert np.all(np.abs(mine - gsc.numpy()) <= 2e-7 * np.abs(gsc.numpy()))
+    group_idx = gsc.topk(M, -1).indices.numpy()
+    _, _, grp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, pool=pool)
+    # a last-place difference in a score can swap two groups only where two scores nearly tie
+    close = np.abs(np.sort(gsc.numpy(), axis=1)[:, 1:] - np.sort(gsc.numpy(), axis=1)[:, :-1]).min(axis=1) < 1e-6
+    assert np.array_equal(grp[~close], group_idx[~close])
+    assert (~close).sum() > 1000
+
+
+# ----------------------------------------------------------------------------- one-pass Hop-B
+
+@pytest.mark.parametrize("capacity", [None, 0, 3, 1000])
+def test_hopb_local_scatter_is_one_stable_sort_by_slot(capacity):
+    """The composition arrival chain -> expert-order regroup, against its definition written out pair by pair:
+    pairs in ascending (slot, p) order, expert x keeping its first `capacity`."""
+    rng = np.random.default_rng(17)
+    R, q, n_local, first = 37, 3, 12, 5
+    rslot = np.stack([np.sort(rng.permutation(n_local)[:q]) for _ in range(R)]) + first
+    rx = rng.integers(0, 1 << 16, (R, 6)).astype(np.uint16)
+    rgate = rng.random((R, q)).astype(np.float32)
+    permuted, place, kept, counts, kept_per, pgate, pairs = orc.hopb_local_scatter(rx, rslot, rgate, q, n_local, first,
+                                                                                  capacity)
+    P = R * q
+    by_expert = {x: [] for x in range(n_local)}
+    for p in range(P):
+        by_expert[int(rslot.reshape(-1)[p]) - first].append(p)
+    want_place = np.full(P, -1, dtype=np.int64)
+    at = 0
+    for x in range(n_local):
+        for rank, p in enumerate(by_expert[x]):
+            if capacity is None:
+                want_place[p] = at + rank
+            elif rank < capacity:
+                want_place[p] = x * capacity + rank
+        at += len(by_expert[x])
+    n_places = P if capacity is None else n_local * capacity
+    assert np.array_equal(place, want_place) and np.array_equal(kept, want_place >= 0)
+    assert counts.tolist() == [len(by_expert[x]) for x in range(n_local)]
+    assert kept_per.tolist() == [len(v) if capacity is None else min(len(v), capacity) for v in by_expert.values()]
+    want_rows = np.zeros((n_places, 6), dtype=np.uint16)
+    want_gate = np.zeros(n_places, dtype=np.float32)
+    want_pairs = np.full(n_places, -1, dtype=np.int64)
+    for p in range(P):
+        if want_place[p] >= 0:
+            want_rows[want_place[p]] = rx[p // q]
+            want_gate[want_place[p]] = rgate.reshape(-1)[p]
+            want_pairs[want_place[p]] = p
+    assert np.array_equal(permuted, want_rows) and np.array_equal(pgate, want_gate)
+    assert np.array_equal(pairs, want_pairs)
