@@ -130,7 +130,8 @@ TERRACE_API int terrace_k2_pack(const void *hidden, const int64_t *expert_idx, c
                     int groups_m, void *payload, int64_t *mask, void *gate_rows, int64_t *u_src,
                     int64_t *node_counts, int64_t *u_node, int64_t *inverse, int64_t *node_offsets,
                     int64_t *pair_table, int64_t *sort_order, int64_t *token_rows, void *gate_sorted,
-                    int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+                    int64_t *pair_src, int64_t *combine_table, int32_t *status, void *workspace,
+                    size_t workspace_bytes, terrace_stream_t stream);
 
 /* _pack_quota_wire (terrace/ta2a_fwd.py:177-249) for a caller that already holds `inverse`:
  * for the token's s-th smallest expert (column j), run m = s/q, i = s%q:
@@ -149,13 +150,16 @@ TERRACE_API int terrace_pack_quota_wire(const int64_t *expert_idx, const void *g
  *   gate_bytes-wide elements (NULL: gate_pairs ignored).
  * Pairs p = r*quota+i are placed in stable ascending order of rslot[p]/epr.  Writes send_buf
  * [P,row_bytes], gate_pairs [P], r_idx [P] i64, slot_idx [P] i64, i_send [rpn] i64 and, when
- * not NULL, pair_pos [P] i64 (the place pair p landed at: the inverse permutation). */
+ * not NULL, pair_pos [P] i64 (the place pair p landed at: the inverse permutation).
+ * Tags: with tags_in [P] i64 and tags_out [P] i64 both given, a caller's tag rides with each pair:
+ * tags_out[place of p] = tags_in[p] (no counterpart in the reference; it lets a later stage name what it
+ * placed in the caller's own terms without a look-up launch). */
 TERRACE_API size_t terrace_k1_arrival_workspace(int64_t R, int quota, int rpn);
 TERRACE_API int terrace_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
                        int64_t row_bytes, int gate_bytes, int quota, int epr, int rpn, int my_local,
                        void *send_buf, void *gate_pairs, int64_t *r_idx, int64_t *slot_idx,
-                       int64_t *i_send, int64_t *pair_pos, int32_t *status, void *workspace,
-                       size_t workspace_bytes, terrace_stream_t stream);
+                       int64_t *i_send, int64_t *pair_pos, const int64_t *tags_in, int64_t *tags_out,
+                       int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream);
 
 /* Expert-order regroup on the expert card (terrace/ta2a_fwd.py:641-646), optionally with a
  * per-expert capacity (no counterpart in the reference, which is drop-less:
@@ -166,13 +170,18 @@ TERRACE_API int terrace_k1_arrival(const void *rx, const int64_t *rslot, const v
  *     place or -1 for a dropped row; kept [P] u8.
  * tokens_per_expert [epr] i64 counts before the cut; kept_per_expert [epr] i64 (may be NULL).
  * node_rx NULL: index planes only.  gate planes ride along when my_gate != NULL:
- * permuted_gate has one gate_bytes-wide element per permuted row. */
+ * permuted_gate has one gate_bytes-wide element per permuted row.
+ * Tags: with tags_in [P] i64 and place_by_tag [n_tags] i64 given, place_by_tag[tags_in[p]] = place of row p
+ * (-1 when dropped; tags outside [0, n_tags) are skipped).  Fed with the tags terrace_k1_arrival carried from
+ * terrace_k2_pack's pair_src, place_by_tag is the combine's [T,k] table (terrace_combine's idx), with no
+ * look-up launch between dispatch and combine. */
 TERRACE_API size_t terrace_regroup_workspace(int64_t P, int epr, int64_t capacity);
 TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P,
                     int64_t row_bytes, int gate_bytes, int epr, int my_local, int64_t capacity,
                     void *permuted, void *permuted_gate, int64_t *order, int64_t *dest, uint8_t *kept,
-                    int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status,
-                    void *workspace, size_t workspace_bytes, terrace_stream_t stream);
+                    int64_t *tokens_per_expert, int64_t *kept_per_expert, const int64_t *tags_in,
+                    int64_t *place_by_tag, int64_t n_tags, int32_t *status, void *workspace,
+                    size_t workspace_bytes, terrace_stream_t stream);
 
 /* Hop-B local scatter in one pass (north-star stage 4; the arrival-side chain of terrace/ta2a_fwd.py:605-646 when
  * every expert slot the arriving rows name is local to this GPU -- one GPU per node, or the one-GPU loop-back).
@@ -187,15 +196,17 @@ TERRACE_API int terrace_regroup(const void *node_rx, const int64_t *my_slot, con
  *     x*capacity+rank, later ones are dropped (place[p] = -1, kept[p] = 0), unused places are zero rows.
  * place [P] i64, kept [P] u8, pair_of_place [places] i64 (-1 on a padding place), permuted_gate [places] (0 on
  * padding; written when rgate != NULL) may each be NULL.  tokens_per_expert [n_local] i64 counts before the cut;
- * kept_per_expert [n_local] i64 may be NULL.  With rx == NULL, terrace_hopb_scatter_move moves the rows later
+ * kept_per_expert [n_local] i64 may be NULL.  tags_in [P] / place_by_tag [n_tags] as in terrace_regroup:
+ * place_by_tag[tags_in[p]] = place[p].  With rx == NULL, terrace_hopb_scatter_move moves the rows later
  * (same geometry, same untouched workspace), like the *_move calls of the other stages. */
 TERRACE_API size_t terrace_hopb_scatter_workspace(int64_t R, int quota, int n_local);
 TERRACE_API int terrace_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
                                      int64_t row_bytes, int gate_bytes, int quota, int first_slot, int n_local,
                                      int64_t capacity, void *permuted, void *permuted_gate, int64_t *place,
                                      uint8_t *kept, int64_t *pair_of_place, int64_t *tokens_per_expert,
-                                     int64_t *kept_per_expert, int32_t *status, void *workspace,
-                                     size_t workspace_bytes, terrace_stream_t stream);
+                                     int64_t *kept_per_expert, const int64_t *tags_in, int64_t *place_by_tag,
+                                     int64_t n_tags, int32_t *status, void *workspace, size_t workspace_bytes,
+                                     terrace_stream_t stream);
 TERRACE_API int terrace_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local,
                                           int64_t capacity, void *permuted, const void *workspace,
                                           size_t workspace_bytes, terrace_stream_t stream);
@@ -382,7 +393,7 @@ TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, 
  * No counterpart in the reference.  It is for callers that cannot allocate device memory at all -- code under
  * HIP graph capture, serving loops that must stay off the allocator, harnesses that forbid hipMalloc -- and so
  * cannot provide the workspace terrace_k1_arrival asks for.  terrace_k1_arrival_static is terrace_k1_arrival
- * (same arguments, same outputs, same kernels) with the workspace taken from a device array of
+ * (its arguments without the tags and the workspace, same outputs, same kernels) with the workspace taken from a device array of
  * TERRACE_STATIC_SCRATCH_BYTES that is part of the library image: every GPU the library runs on holds that
  * array until the process ends.  Inputs whose workspace would not fit (terrace_k1_arrival_workspace(R, quota,
  * rpn) > terrace_static_scratch_bytes(); about 900 thousand pairs) are refused with TERRACE_E2BIG.  The call

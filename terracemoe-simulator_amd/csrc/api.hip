@@ -32,17 +32,20 @@ size_t k1_workspace(int64_t R, int quota, int rpn);
 int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                    int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
                    int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
-                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, hipStream_t s);
+                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, const int64_t *tags_in,
+                   int64_t *tags_out, hipStream_t s);
 size_t regroup_workspace(int64_t P, int epr, int64_t capacity);
 int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
                 int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
                 int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
-                int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, hipStream_t s);
+                int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch,
+                const int64_t *tags_in, int64_t *place_by_tag, int64_t n_tags, hipStream_t s);
 size_t hopb_workspace(int64_t R, int quota, int n_local);
 int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                      int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
                      void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
-                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *ws, size_t ws_bytes,
+                     int64_t *tokens_per_expert, int64_t *kept_per_expert, const int64_t *tags_in,
+                     int64_t *place_by_tag, int64_t n_tags, int32_t *status, void *ws, size_t ws_bytes,
                      hipStream_t s);
 int run_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local, int64_t capacity,
                           void *permuted, const void *ws, size_t ws_bytes, hipStream_t s);
@@ -51,8 +54,8 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
                 int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
                 void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node, int64_t *inverse,
                 int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order, int64_t *token_rows,
-                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, int64_t mask_pitch, int64_t gate_pitch,
-                int gate_pad, hipStream_t s);
+                void *gate_sorted, int64_t *pair_src, int64_t *combine_table, int32_t *status, void *ws,
+                size_t ws_bytes, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s);
 int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
                         int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
                         int32_t *status, hipStream_t s);
@@ -155,12 +158,12 @@ int terrace_k2_pack(const void *hidden, const int64_t *expert_idx, const void *g
                     int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload,
                     int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                     int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                    int64_t *token_rows, void *gate_sorted, int32_t *status, void *workspace,
-                    size_t workspace_bytes, terrace_stream_t stream) {
+                    int64_t *token_rows, void *gate_sorted, int64_t *pair_src, int64_t *combine_table,
+                    int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
     return run_k2_pack(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, world, n_experts, rpn, groups_m,
                        payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets, pair_table,
-                       sort_order, token_rows, gate_sorted, status, workspace, workspace_bytes, 0, 0, 0,
-                       (hipStream_t)stream);
+                       sort_order, token_rows, gate_sorted, pair_src, combine_table, status, workspace,
+                       workspace_bytes, 0, 0, 0, (hipStream_t)stream);
 }
 
 // Words of one Hop-A small container row holding `quota` slot ids and `quota` gates.
@@ -179,7 +182,8 @@ int terrace_k2_pack_wire(const void *hidden, const int64_t *expert_idx, const vo
     void *gate_plane = (void *)(wire + quota);                 // the gates start on the word after the ids
     return run_k2_pack(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, world, n_experts, rpn, groups_m,
                        payload, wire, gate_plane, u_src, node_counts, u_node, inverse, node_offsets, pair_table,
-                       sort_order, token_rows, gate_sorted, status, workspace, workspace_bytes, wire_words,
+                       sort_order, token_rows, gate_sorted, nullptr, nullptr, status, workspace, workspace_bytes,
+                       wire_words,
                        (int64_t)wire_words * per_word, (wire_words - quota) * per_word - quota, (hipStream_t)stream);
 }
 
@@ -194,11 +198,12 @@ size_t terrace_k1_arrival_workspace(int64_t R, int quota, int rpn) { return k1_w
 
 int terrace_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                        int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
-                       int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status,
-                       void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+                       int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, const int64_t *tags_in,
+                       int64_t *tags_out, int32_t *status, void *workspace, size_t workspace_bytes,
+                       terrace_stream_t stream) {
     return run_k1_arrival(rx, rslot, rgate, R, row_bytes, gate_bytes, quota, epr, rpn, my_local, send_buf,
                           gate_pairs, r_idx, slot_idx, i_send, pair_pos, status, workspace, workspace_bytes, quota,
-                          quota, nullptr, (hipStream_t)stream);
+                          quota, nullptr, tags_in, tags_out, (hipStream_t)stream);
 }
 
 int terrace_k1_arrival_wire(const void *rx, const int64_t *rwire, int wire_words, int64_t R, int64_t row_bytes,
@@ -211,7 +216,8 @@ int terrace_k1_arrival_wire(const void *rx, const int64_t *rwire, int wire_words
     const void *gate_plane = rwire ? (const void *)(rwire + quota) : nullptr;
     return run_k1_arrival(rx, rwire, gate_plane, R, row_bytes, gate_bytes, quota, epr, rpn, my_local, send_buf,
                           gate_pairs, r_idx, slot_idx, i_send, pair_pos, status, workspace, workspace_bytes,
-                          wire_words, (int64_t)wire_words * (8 / gate_bytes), meta, (hipStream_t)stream);
+                          wire_words, (int64_t)wire_words * (8 / gate_bytes), meta, nullptr, nullptr,
+                          (hipStream_t)stream);
 }
 
 size_t terrace_regroup_workspace(int64_t P, int epr, int64_t capacity) { return regroup_workspace(P, epr, capacity); }
@@ -219,11 +225,11 @@ size_t terrace_regroup_workspace(int64_t P, int epr, int64_t capacity) { return 
 int terrace_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
                     int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
                     int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert,
-                    int64_t *kept_per_expert, int32_t *status, void *workspace, size_t workspace_bytes,
-                    terrace_stream_t stream) {
+                    int64_t *kept_per_expert, const int64_t *tags_in, int64_t *place_by_tag, int64_t n_tags,
+                    int32_t *status, void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
     return run_regroup(node_rx, my_slot, my_gate, P, row_bytes, gate_bytes, epr, my_local, capacity, permuted,
                        permuted_gate, order, dest, kept, tokens_per_expert, kept_per_expert, status, workspace,
-                       workspace_bytes, 1, 1, (hipStream_t)stream);
+                       workspace_bytes, 1, 1, tags_in, place_by_tag, n_tags, (hipStream_t)stream);
 }
 
 int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta, int64_t P, int64_t row_bytes, int gate_bytes,
@@ -236,7 +242,7 @@ int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta, int64_t P,
     const void *gate_plane = (permuted_gate && my_meta) ? (const void *)(my_meta + 1) : nullptr;
     return run_regroup(node_rx, my_meta, gate_plane, P, row_bytes, gate_bytes, epr, my_local, capacity, permuted,
                        permuted_gate, order, dest, kept, tokens_per_expert, kept_per_expert, status, workspace,
-                       workspace_bytes, 2, 2 * (8 / gate_bytes), (hipStream_t)stream);
+                       workspace_bytes, 2, 2 * (8 / gate_bytes), nullptr, nullptr, 0, (hipStream_t)stream);
 }
 
 size_t terrace_hopb_scatter_workspace(int64_t R, int quota, int n_local) { return hopb_workspace(R, quota, n_local); }
@@ -244,11 +250,12 @@ size_t terrace_hopb_scatter_workspace(int64_t R, int quota, int n_local) { retur
 int terrace_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                          int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
                          void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
-                         int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *workspace,
+                         int64_t *tokens_per_expert, int64_t *kept_per_expert, const int64_t *tags_in,
+                         int64_t *place_by_tag, int64_t n_tags, int32_t *status, void *workspace,
                          size_t workspace_bytes, terrace_stream_t stream) {
     return run_hopb_scatter(rx, rslot, rgate, R, row_bytes, gate_bytes, quota, first_slot, n_local, capacity, permuted,
-                            permuted_gate, place, kept, pair_of_place, tokens_per_expert, kept_per_expert, status,
-                            workspace, workspace_bytes, (hipStream_t)stream);
+                            permuted_gate, place, kept, pair_of_place, tokens_per_expert, kept_per_expert, tags_in,
+                            place_by_tag, n_tags, status, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 int terrace_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quota, int n_local, int64_t capacity,

@@ -20,7 +20,8 @@ size_t k1_workspace(int64_t R, int quota, int rpn);
 int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                    int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
                    int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
-                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, hipStream_t s);
+                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, const int64_t *tags_in,
+                   int64_t *tags_out, hipStream_t s);
 }  // namespace terrace
 
 static __device__ __align__(256) unsigned char scratch[TERRACE_STATIC_SCRATCH_BYTES];
@@ -70,7 +71,8 @@ int terrace_k1_arrival_static(const void *rx, const int64_t *rslot, const void *
     if (!ws) return rc;
     return terrace::run_k1_arrival(rx, rslot, rgate, R, row_bytes, gate_bytes, quota, epr, rpn, my_local, send_buf,
                                    gate_pairs, r_idx, slot_idx, i_send, pair_pos, status, ws,
-                                   (size_t)TERRACE_STATIC_SCRATCH_BYTES, quota, quota, nullptr, (hipStream_t)stream);
+                                   (size_t)TERRACE_STATIC_SCRATCH_BYTES, quota, quota, nullptr, nullptr, nullptr,
+                                   (hipStream_t)stream);
 }
 
 }  // extern "C"

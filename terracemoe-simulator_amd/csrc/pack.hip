@@ -27,27 +27,33 @@ namespace terrace {
 
 constexpr int kTokUnit = kWave;          // tokens per unit
 
-static Units token_units(int64_t T, int n_nodes) {
+// Lanes per token of the two kernels: the smallest of 4, 8, 16 that holds the token's k ids.
+static int lanes_per_token(int k) { return k <= 4 ? 4 : (k <= 8 ? 8 : 16); }
+
+// One count workgroup is kSortBlockMax lanes = 1024 / LPT tokens = 16 / LPT units.
+static Units token_units(int64_t T, int k, int n_nodes) {
     Units u;
     u.n_items = T;
     u.n_buckets = n_nodes;
     u.chunks = 1;
     u.n_units = (int)((T + kTokUnit - 1) / kTokUnit);
     if (u.n_units < 1) u.n_units = 1;
-    finish_units(u);
+    u.wpb = 16 / lanes_per_token(k);
+    u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
+    u.direct = n_nodes <= kDirectMaxBuckets && (int64_t)n_nodes * u.n_blocks <= kDirectMaxWords;
     return u;
 }
 
 bool k2_token_path_applies(int64_t T, int k, int n_nodes) {
-    return k <= 16 && n_nodes <= 64 && token_units(T, n_nodes).direct;
+    return k <= 16 && n_nodes <= 64 && token_units(T, k, n_nodes).direct;
 }
 
-const int32_t *k2_token_positions(const void *ws, int64_t T, int n_nodes) {
-    return (const int32_t *)((const char *)ws + units_table_bytes(token_units(T, n_nodes)));
+const int32_t *k2_token_positions(const void *ws, int64_t T, int k, int n_nodes) {
+    return (const int32_t *)((const char *)ws + units_table_bytes(token_units(T, k, n_nodes)));
 }
 
-size_t k2_token_workspace(int64_t T, int n_nodes, int groups_m) {
-    return units_table_bytes(token_units(T, n_nodes)) + align_up((size_t)T * groups_m * sizeof(int32_t), 256);
+size_t k2_token_workspace(int64_t T, int k, int n_nodes, int groups_m) {
+    return units_table_bytes(token_units(T, k, n_nodes)) + align_up((size_t)T * groups_m * sizeof(int32_t), 256);
 }
 
 // The lowest M set bits of a node set: the nodes that get a send row.
@@ -67,37 +73,89 @@ __device__ __forceinline__ uint64_t read_lane64(uint64_t v, int src_lane) {
     return ((uint64_t)hi << 32) | lo;
 }
 
-template <int KMAX>
-__global__ __launch_bounds__(kSortBlockMax) void k2_count_kernel(const int64_t *__restrict__ expert_idx, int64_t T,
-                                                                 int k, int slots, int n_experts, int M, Units u,
-                                                                 int32_t *__restrict__ table,
-                                                                 int32_t *__restrict__ status) {
-    extern __shared__ int32_t lds[];
-    const int lane = lane_id(), w = wave_in_block();
-    const int unit = blockIdx.x * u.wpb + w;
-    const int64_t t = (int64_t)unit * kTokUnit + lane;
-    uint64_t occ = 0;
-    if (unit < u.n_units && t < T) {
-        const int64_t *row = expert_idx + t * k;
-        int64_t v[KMAX];
+// What lane (token, column) knows once the token's ids are shared inside its group of LPT lanes.
+template <int LPT>
+struct TokenView {
+    int e, nd;                  // the lane's expert and node, -1 when the column is padding or out of range
+    bool ok;
+    uint64_t all, occ;          // every node the token touches; the lowest M of them (identical in the group)
+    int rank, within;           // of the lane's expert among the token's by (id, column); among those of its node
+    bool first_of_node, bad_pair;
+    __device__ __forceinline__ void build(int64_t v, bool has_col, int col, int tok_lane, int slots, int n_experts,
+                                          int M, int quota) {
+        ok = has_col && v >= 0 && v < n_experts;
+        e = ok ? (int)v : -1;
+        nd = ok ? e / slots : -1;
+        int E[LPT], N[LPT];
 #pragma unroll
-        for (int j = 0; j < KMAX; ++j) v[j] = row[j < k ? j : 0];
-        uint64_t all = 0;
+        for (int i = 0; i < LPT; ++i) {
+            E[i] = __shfl(e, tok_lane + i, kWave);
+            N[i] = __shfl(nd, tok_lane + i, kWave);
+        }
+        all = 0;
 #pragma unroll
-        for (int j = 0; j < KMAX; ++j)
-            if (j < k && v[j] >= 0 && v[j] < n_experts) all |= 1ull << ((int)v[j] / slots);
+        for (int i = 0; i < LPT; ++i)
+            if (N[i] >= 0) all |= 1ull << N[i];
         occ = lowest_bits(all, M);
+        rank = within = 0;
+        int same = 0, earlier = 0;
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const bool lower = E[i] >= 0 && (E[i] < e || (E[i] == e && i < col));
+            const bool hit = N[i] == nd;
+            rank += lower ? 1 : 0;
+            within += (lower && hit) ? 1 : 0;
+            same += hit ? 1 : 0;
+            earlier += (hit && i < col) ? 1 : 0;
+        }
+        first_of_node = ok && earlier == 0;
+        bad_pair = first_of_node && same != quota;
     }
-    int mine = 0;                       // lane n counts node n
-    for (int n = 0; n < u.n_buckets; ++n) {
-        const int cnt = __popcll(__ballot((occ >> n) & 1ull));
-        if (lane == n) mine = cnt;
-    }
-    lds_i32 *counts = (lds_i32 *)lds;
-    if (lane < u.n_buckets) counts[w * u.n_buckets + lane] = mine;
-    if (status && blockIdx.x == 0 && threadIdx.x < TERRACE_STATUS_WORDS) status[threadIdx.x] = 0;
+};
+
+// Count: 1024 lanes per workgroup, LPT lanes per token (lane = token * LPT + column, so the ids are read with
+// consecutive lanes on consecutive words), 16 / LPT units per workgroup.  Also takes the census the guard of
+// terrace/ta2a.py:170-204 reads -- occupied (token, node) pairs, pairs holding other than k/M experts, the fault
+// bits -- and leaves it per workgroup beside the totals: the place kernel's first workgroup adds the few entries up
+// and stores the status block, so no workgroup ever waits on an atomic to a word every other workgroup adds to.
+template <int LPT>
+__global__ __launch_bounds__(kSortBlockMax) void k2_count_kernel(const int64_t *__restrict__ expert_idx, int64_t T,
+                                                                 int k, int slots, int n_experts, int M, int quota,
+                                                                 Units u, int32_t *__restrict__ table) {
+    constexpr int kTpw = kWave / LPT;               // tokens per wave
+    constexpr int kWpu = LPT;                       // waves per unit
+    __shared__ int32_t s_counts[16 / LPT * 64];     // [unit in block][node]
+    __shared__ int32_t s_census[4];
+    const int lane = lane_id(), w = wave_in_block();
+    const int n_nodes = u.n_buckets;
+    const int col = lane & (LPT - 1), tok_lane = lane & ~(LPT - 1);
+    const int unit_in_block = w / kWpu;
+    const int64_t t = ((int64_t)blockIdx.x * u.wpb + unit_in_block) * kTokUnit + (w % kWpu) * kTpw + lane / LPT;
+    const bool live = t < T, has_col = live && col < k;
+    const int64_t v = has_col ? expert_idx[t * k + col] : -1;
+    for (int i = threadIdx.x; i < u.wpb * n_nodes; i += blockDim.x) s_counts[i] = 0;
+    if (threadIdx.x < 4) s_census[threadIdx.x] = 0;
     __syncthreads();
-    direct_block_counts(u, table, counts);
+    TokenView<LPT> tv;
+    tv.build(v, has_col, col, tok_lane, slots, n_experts, M, quota);
+    int wave_cnt = 0;                               // lane n: tokens of this wave on node n
+#pragma unroll
+    for (int i = 0; i < kTpw; ++i) wave_cnt += (int)((read_lane64(tv.occ, i * LPT) >> lane) & 1ull);
+    if (lane < n_nodes && wave_cnt) atomicAdd(&s_counts[unit_in_block * n_nodes + lane], wave_cnt);
+    int fault = (has_col && !tv.ok) ? TERRACE_FAULT_ID_RANGE : 0;
+    if (live && col == 0 && __popcll(tv.all) != M) fault |= TERRACE_FAULT_FANOUT;
+    if (tv.bad_pair) fault |= TERRACE_FAULT_QUOTA;
+    const int occupied = __popcll(__ballot(tv.first_of_node)), off_quota = __popcll(__ballot(tv.bad_pair));
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) fault |= __shfl_xor(fault, d, kWave);
+    if (lane == 0) {
+        if (fault) atomicOr(&s_census[0], fault);
+        if (occupied) atomicAdd(&s_census[1], occupied);
+        if (off_quota) atomicAdd(&s_census[2], off_quota);
+    }
+    __syncthreads();
+    direct_block_counts(u, table, (lds_i32 *)s_counts);
+    if (threadIdx.x < 4) table[units_census_at(u) + 4 * (int64_t)blockIdx.x + threadIdx.x] = s_census[threadIdx.x];
 }
 
 // LPT lanes per token (k <= LPT), 64 tokens per workgroup: blockDim = 64 * LPT, thread = token_local * LPT + column.
@@ -107,14 +165,14 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     int M, int quota, Units u, int32_t *__restrict__ table, int64_t *__restrict__ mask, G *__restrict__ gate_rows,
     int64_t *__restrict__ u_src, int64_t *__restrict__ u_node, int64_t *__restrict__ inverse,
     int64_t *__restrict__ pair_table, int64_t *__restrict__ sort_order, int64_t *__restrict__ token_rows,
-    G *__restrict__ gate_sorted, int32_t *__restrict__ pos32, int64_t *__restrict__ node_counts,
-    int64_t *__restrict__ node_offsets, int32_t *__restrict__ status, int64_t mask_pitch, int64_t gate_pitch,
-    int gate_pad) {
+    G *__restrict__ gate_sorted, int64_t *__restrict__ pair_src, int64_t *__restrict__ combine_table,
+    int32_t *__restrict__ pos32, int64_t *__restrict__ node_counts, int64_t *__restrict__ node_offsets,
+    int32_t *__restrict__ status, int64_t mask_pitch, int64_t gate_pitch, int gate_pad) {
     constexpr int kWaves = LPT;                     // waves per workgroup
     constexpr int kTpw = kWave / LPT;               // tokens per wave
     __shared__ int32_t s_tot[64], s_base[64], s_start[65], s_tab[64];
     __shared__ int32_t s_wcnt[kWaves][64];
-    __shared__ int32_t s_census[kWaves][4];
+    __shared__ int32_t s_dirty[kWaves];
     const int lane = lane_id(), w = wave_in_block();
     const int unit = blockIdx.x;
     const int n_nodes = u.n_buckets;
@@ -136,50 +194,24 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     const int me = unit / u.wpb;
     direct_block_base(u, table, me, unit == 0, (lds_i32 *)s_tot, (lds_i32 *)s_base, (lds_i32 *)s_start, node_counts,
                       nullptr, node_offsets);
-    // ---- the token's ids, shared inside the group ----
-    const bool ok = has_col && v >= 0 && v < n_experts;
-    const int e = ok ? (int)v : -1;
-    const int nd = ok ? e / slots : -1;
-    int fault = (has_col && !ok) ? TERRACE_FAULT_ID_RANGE : 0;
-    int E[LPT], N[LPT];
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-        E[i] = __shfl(e, tok_lane + i, kWave);
-        N[i] = __shfl(nd, tok_lane + i, kWave);
-    }
-    uint64_t all = 0;
-#pragma unroll
-    for (int i = 0; i < LPT; ++i)
-        if (N[i] >= 0) all |= 1ull << N[i];
-    const uint64_t occ = lowest_bits(all, M);       // identical in the lanes of a token
-    // ranks by (id, column); census of the lane's own element (terrace/ta2a.py:170-204)
-    int rank = 0, within = 0, same = 0, earlier = 0;
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-        const bool lower = E[i] >= 0 && (E[i] < e || (E[i] == e && i < col));
-        const bool hit = N[i] == nd;
-        rank += lower ? 1 : 0;
-        within += (lower && hit) ? 1 : 0;
-        same += hit ? 1 : 0;
-        earlier += (hit && i < col) ? 1 : 0;
-    }
-    const bool first_of_node = ok && earlier == 0;
-    const bool bad_pair = first_of_node && same != quota;
-    const int n_all = __popcll(all);
+    // ---- the token's ids, shared inside the group; ranks by (id, column) ----
+    TokenView<LPT> tv;
+    tv.build(v, has_col, col, tok_lane, slots, n_experts, M, quota);
+    const bool ok = tv.ok;
+    const int e = tv.e, nd = tv.nd, rank = tv.rank, within = tv.within;
+    const uint64_t occ = tv.occ;
     // a token is clean when it touches exactly M nodes, each with exactly `quota` in-range experts
-    const uint64_t dirty_lanes = __ballot(bad_pair || (has_col && !ok));
+    const uint64_t dirty_lanes = __ballot(tv.bad_pair || (has_col && !ok));
     const bool dirty_group = ((dirty_lanes >> tok_lane) & ((LPT == 64 ? 0 : (1ull << LPT)) - 1ull)) != 0;
-    const bool clean = live && n_all == M && !dirty_group;
-    if (live && col == 0 && n_all != M) fault |= TERRACE_FAULT_FANOUT;
-    if (bad_pair) fault |= TERRACE_FAULT_QUOTA;
-    int occupied = first_of_node ? 1 : 0, off_quota = bad_pair ? 1 : 0;
+    const bool clean = live && __popcll(tv.all) == M && !dirty_group;
     // a token that is not clean starts from a defined state: its per-column cells first, ordered before the
-    // stores that fill cells by the two barriers below
+    // stores that fill cells by the barrier below
     if (has_col && !clean) {
         if (pair_table) pair_table[t * k + col] = -1;
         if (sort_order) sort_order[t * k + col] = 0;
         if (inverse) inverse[t * k + col] = -1;
         if (gates && gate_sorted) gate_sorted[t * k + col] = G(0);
+        if (combine_table) combine_table[t * k + col] = -1;
     }
     // ---- tokens of this wave per node (lane n counts node n); the owner lanes count their earlier peers ----
     const bool owner = live && col < M;             // lane (token, m) owns the token's m-th send row
@@ -198,33 +230,33 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     }
     if (lane < n_nodes) s_wcnt[w][lane] = wave_cnt;
     if (threadIdx.x < n_nodes) s_tab[threadIdx.x] = tab;
-    // ---- census: one atomic per workgroup and word, issued before the stores so that nothing waits on it ----
+    // ---- does any token of the workgroup start from defaults?  (uniform across the workgroup after the barrier) ----
     const uint64_t any_dirty = __ballot(live && !clean);
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        fault |= __shfl_xor(fault, d, kWave);
-        occupied += __shfl_xor(occupied, d, kWave);
-        off_quota += __shfl_xor(off_quota, d, kWave);
-    }
-    if (lane == 0) {
-        s_census[w][0] = fault;
-        s_census[w][1] = occupied;
-        s_census[w][2] = off_quota;
-        s_census[w][3] = any_dirty != 0;
-    }
+    if (lane == 0) s_dirty[w] = any_dirty != 0;
     __syncthreads();
-    bool dirty_block = false;                       // uniform across the workgroup
-    for (int x = 0; x < kWaves; ++x) dirty_block = dirty_block || s_census[x][3];
-    if (threadIdx.x == 0 && status) {
+    bool dirty_block = false;
+    for (int x = 0; x < kWaves; ++x) dirty_block = dirty_block || s_dirty[x];
+    // ---- the status block: the count kernel's per-workgroup census, added up and stored by the first workgroup ----
+    if (unit == 0 && w == 0 && status) {
+        const int32_t *census = table + units_census_at(u);
         int f = 0, o = 0, q = 0;
-        for (int x = 0; x < kWaves; ++x) {
-            f |= s_census[x][0];
-            o += s_census[x][1];
-            q += s_census[x][2];
+        for (int b = lane; b < u.n_blocks; b += kWave) {
+            f |= census[4 * b + 0];
+            o += census[4 * b + 1];
+            q += census[4 * b + 2];
         }
-        if (f) atomicOr(&status[0], f);
-        if (o) atomicAdd(&status[1], o);
-        if (q) atomicAdd(&status[2], q);
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) {
+            f |= __shfl_xor(f, d, kWave);
+            o += __shfl_xor(o, d, kWave);
+            q += __shfl_xor(q, d, kWave);
+        }
+        if (lane == 0) {
+            status[0] = f;
+            status[1] = o;
+            status[2] = q;
+            status[3] = 0;
+        }
     }
     int r = -1;
     if (my_node >= 0) {
@@ -239,6 +271,7 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
             for (int i = 0; i < quota; ++i) {
                 mask[(int64_t)r * mask_pitch + i] = 0;
                 if (gates) gate_rows[(int64_t)r * gate_pitch + i] = G(0);
+                if (pair_src) pair_src[(int64_t)r * quota + i] = -1;
             }
     }
     if (owner) {
@@ -251,7 +284,10 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
         for (int64_t x = used + threadIdx.x; x < S; x += blockDim.x) {
             u_src[x] = 0;
             if (u_node) u_node[x] = 0;
-            for (int i = 0; i < quota; ++i) mask[x * mask_pitch + i] = 0;
+            for (int i = 0; i < quota; ++i) {
+                mask[x * mask_pitch + i] = 0;
+                if (pair_src) pair_src[x * quota + i] = -1;
+            }
             if (gates)
                 for (int i = 0; i < quota + gate_pad; ++i) gate_rows[x * gate_pitch + i] = G(0);
         }
@@ -268,6 +304,7 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
         if (gates) gate_rows[(int64_t)row * gate_pitch + within] = gate;
         if (inverse) inverse[t * k + col] = row;
         if (pair_table) pair_table[t * k + rank] = (int64_t)row * quota + within;
+        if (pair_src) pair_src[(int64_t)row * quota + within] = t * k + rank;
         if (sort_order) sort_order[t * k + rank] = col;
         if (gates && gate_sorted) gate_sorted[t * k + rank] = gate;
     }
@@ -277,35 +314,35 @@ template <int LPT, typename G>
 static void launch_place(const int64_t *expert_idx, const void *gates, int64_t T, int k, int slots, int n_experts,
                          int M, const Units &u, int32_t *table, int64_t *mask, void *gate_rows, int64_t *u_src,
                          int64_t *u_node, int64_t *inverse, int64_t *pair_table, int64_t *sort_order,
-                         int64_t *token_rows, void *gate_sorted, int32_t *pos32, int64_t *node_counts,
-                         int64_t *node_offsets, int32_t *status, int64_t mask_pitch, int64_t gate_pitch, int gate_pad,
-                         hipStream_t s) {
+                         int64_t *token_rows, void *gate_sorted, int64_t *pair_src, int64_t *combine_table,
+                         int32_t *pos32, int64_t *node_counts, int64_t *node_offsets, int32_t *status,
+                         int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
     k2_place_kernel<LPT, G><<<u.n_units, kWave * LPT, 0, s>>>(
         expert_idx, (const G *)gates, T, k, slots, n_experts, M, k / M, u, table, mask, (G *)gate_rows, u_src, u_node,
-        inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pos32, node_counts, node_offsets, status,
-        mask_pitch, gate_pitch, gate_pad);
+        inverse, pair_table, sort_order, token_rows, (G *)gate_sorted, pair_src, combine_table, pos32, node_counts,
+        node_offsets, status, mask_pitch, gate_pitch, gate_pad);
 }
 
 int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
                  int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                  int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                  int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, int64_t mask_pitch,
-                 int64_t gate_pitch, int gate_pad, hipStream_t s) {
-    const Units u = token_units(T, n_nodes);
+                 int64_t *token_rows, void *gate_sorted, int64_t *pair_src, int64_t *combine_table, int32_t *status,
+                 void *ws, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
+    const Units u = token_units(T, k, n_nodes);
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + units_table_bytes(u));
-    const size_t lds = (size_t)u.wpb * n_nodes * sizeof(int32_t);
-    if (k <= 8)
-        k2_count_kernel<8><<<u.n_blocks, u.wpb * kWave, lds, s>>>(expert_idx, T, k, slots, n_experts, groups_m, u, table,
-                                                                 status);
-    else
-        k2_count_kernel<16><<<u.n_blocks, u.wpb * kWave, lds, s>>>(expert_idx, T, k, slots, n_experts, groups_m, u,
-                                                                  table, status);
+#define TERRACE_COUNT(L)                                                                                          \
+    k2_count_kernel<L><<<u.n_blocks, kSortBlockMax, 0, s>>>(expert_idx, T, k, slots, n_experts, groups_m, k / groups_m, \
+                                                           u, table)
+    if (k <= 4) TERRACE_COUNT(4);
+    else if (k <= 8) TERRACE_COUNT(8);
+    else TERRACE_COUNT(16);
+#undef TERRACE_COUNT
 #define TERRACE_PLACE(L, G)                                                                                        \
     launch_place<L, G>(expert_idx, gates, T, k, slots, n_experts, groups_m, u, table, mask, gate_rows, u_src, u_node, \
-                       inverse, pair_table, sort_order, token_rows, gate_sorted, pos32, node_counts, node_offsets,  \
-                       status, mask_pitch, gate_pitch, gate_pad, s)
+                       inverse, pair_table, sort_order, token_rows, gate_sorted, pair_src, combine_table, pos32,    \
+                       node_counts, node_offsets, status, mask_pitch, gate_pitch, gate_pad, s)
     if (k <= 4) {
         if (gate_bytes == 4) TERRACE_PLACE(4, uint32_t);
         else TERRACE_PLACE(4, uint16_t);

@@ -67,7 +67,7 @@ Units make_units(int64_t n_items, int n_buckets) {
 
 size_t units_table_bytes(const Units &u) {
     const size_t words = (size_t)u.n_units * u.n_buckets + u.n_buckets + 1 +
-                         (u.direct ? (size_t)u.n_buckets * u.n_blocks : 0);
+                         (u.direct ? (size_t)u.n_buckets * u.n_blocks + 4 * (size_t)u.n_blocks : 0);
     return align_up(words * sizeof(int32_t), 256);
 }
 
@@ -569,20 +569,24 @@ struct EmitArrival {         // terrace/ops/__init__.py:287-299
     int64_t *r_idx, *slot_idx, *pair_pos;
     int32_t *pos32;
     int64_t *meta;           // Hop-B container [P, 2]: word 0 the slot id, word 1 the gate then zeros; or NULL
+    const int64_t *tags_in;  // [P] a caller's tag per pair, carried to the pair's place: tags_out[dest] = tags_in[p]
+    int64_t *tags_out;
     static constexpr bool kTallies = false;
-    struct Pre { uint32_t gbits; };
+    struct Pre { uint32_t gbits; int64_t tag; };
     __device__ __forceinline__ Pre fetch(int64_t p) const {
-        Pre pre{0u};
+        Pre pre{0u, -1};
         if (rgate) {
             const uint32_t r = (uint32_t)p / (uint32_t)quota;
             const int64_t at = (int64_t)r * gate_pitch + (int64_t)((uint32_t)p - r * (uint32_t)quota);
             pre.gbits = gate_bytes == 4 ? ((const uint32_t *)rgate)[at] : (uint32_t)((const uint16_t *)rgate)[at];
         }
+        if (tags_in) pre.tag = tags_in[p];
         return pre;
     }
     // `slot` is the value the key was computed from: rslot[r, i]
     __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, int64_t slot, Pre pre, const int32_t *,
                                               int *) const {
+        if (tags_out) tags_out[dest] = pre.tag;
         r_idx[dest] = (int64_t)((uint32_t)p / (uint32_t)quota);
         if (slot_idx) slot_idx[dest] = slot;
         if (rgate && gate_pairs) {
@@ -609,15 +613,19 @@ struct EmitHopB {            // arrival + expert-order regroup in one placement 
     int64_t *pair_of_place;  // [places]: the pair behind each place
     void *permuted_gate;     // [places]
     int32_t *pos32;          // [P]: `place` for the row mover
+    const int64_t *tags_in;  // [P] a caller's tag per pair: place_by_tag[tags_in[p]] = place of p (-1 dropped)
+    int64_t *place_by_tag;
+    int64_t n_tags;
     static constexpr bool kTallies = false;
-    struct Pre { uint32_t gbits; };
+    struct Pre { uint32_t gbits; int64_t tag; };
     __device__ __forceinline__ Pre fetch(int64_t p) const {
-        Pre pre{0u};
+        Pre pre{0u, -1};
         if (rgate) {
             const uint32_t r = (uint32_t)p / (uint32_t)quota;
             const int64_t at = (int64_t)r * gate_pitch + (int64_t)((uint32_t)p - r * (uint32_t)quota);
             pre.gbits = gate_bytes == 4 ? ((const uint32_t *)rgate)[at] : (uint32_t)((const uint16_t *)rgate)[at];
         }
+        if (tags_in) pre.tag = tags_in[p];
         return pre;
     }
     __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre pre,
@@ -632,6 +640,7 @@ struct EmitHopB {            // arrival + expert-order regroup in one placement 
         pos32[p] = (int32_t)d;
         if (place) place[p] = d;
         if (kept) kept[p] = keep ? 1 : 0;
+        if (place_by_tag && (uint64_t)pre.tag < (uint64_t)n_tags) place_by_tag[pre.tag] = d;
         if (keep) {
             if (pair_of_place) pair_of_place[d] = p;
             if (rgate && permuted_gate) {
@@ -710,22 +719,26 @@ struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
     int64_t *order, *dest_out;
     uint8_t *kept;
     int32_t *order32;
+    const int64_t *tags_in;  // [P] a caller's tag per row: place_by_tag[tags_in[p]] = place of row p (-1 dropped)
+    int64_t *place_by_tag;
+    int64_t n_tags;
     static constexpr bool kTallies = false;
-    typedef NoPre Pre;
-    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
-    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre, const int32_t *start,
-                                              int *) const {
+    struct Pre { int64_t tag; };
+    __device__ __forceinline__ Pre fetch(int64_t p) const { return Pre{tags_in ? tags_in[p] : -1}; }
+    __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre pre,
+                                              const int32_t *start, int *) const {
         order32[dest] = (int32_t)p;
         if (order) order[dest] = p;
+        int64_t d = dest;
+        bool keep = true;
         if (capacity >= 0) {
             const int64_t rank = dest - start[key];
-            const bool keep = rank < capacity;
-            if (dest_out) dest_out[p] = keep ? key * capacity + rank : -1;
-            if (kept) kept[p] = keep ? 1 : 0;
-        } else {
-            if (dest_out) dest_out[p] = dest;
-            if (kept) kept[p] = 1;
+            keep = rank < capacity;
+            d = keep ? key * capacity + rank : -1;
         }
+        if (dest_out) dest_out[p] = d;
+        if (kept) kept[p] = keep ? 1 : 0;
+        if (place_by_tag && (uint64_t)pre.tag < (uint64_t)n_tags) place_by_tag[pre.tag] = d;
         return 0;
     }
 };
@@ -738,6 +751,8 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
     int64_t *mask, *u_src, *u_node, *inverse, *pair_table, *sort_order, *token_rows;
     void *gate_rows, *gate_sorted;
     int32_t *pos32;
+    int64_t *pair_src;                   // [T*M*quota]: t*k + rank behind each Hop-A pair, -1 where none
+    int64_t *combine_table;              // [T, k]: ranks that own no pair are set to -1 here
     int64_t mask_pitch, gate_pitch;      // row pitches of the mask / gate_rows planes, in their own elements
     int gate_pad;                        // gate elements to zero after a row's quota gates
     // status word 1 receives the number of occupied (token, node) pairs, word 2 the number of
@@ -750,6 +765,8 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
         const int64_t at = t * k + (int64_t)m * quota + i;
         if (pair_table) pair_table[at] = -1;
         if (sort_order) sort_order[at] = 0;
+        if (combine_table) combine_table[at] = -1;
+        if (pair_src) pair_src[(int64_t)row * quota + i] = -1;
         mask[(int64_t)row * mask_pitch + i] = 0;
         if (!gates) return;
         const int64_t gcell = (int64_t)row * gate_pitch + i;
@@ -843,6 +860,7 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
             if (inverse) inverse[t * k + j] = row;
             if (pair_table) pair_table[t * k + r] = cell;
             if (sort_order) sort_order[t * k + r] = j;
+            if (pair_src) pair_src[cell] = t * k + r;
         };
         if constexpr (KMAX > 0) {
 #pragma unroll
@@ -1036,7 +1054,8 @@ size_t k1_workspace(int64_t R, int quota, int rpn) {
 int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                    int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf, void *gate_pairs,
                    int64_t *r_idx, int64_t *slot_idx, int64_t *i_send, int64_t *pair_pos, int32_t *status, void *ws,
-                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, hipStream_t s) {
+                   size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, int64_t *meta, const int64_t *tags_in,
+                   int64_t *tags_out, hipStream_t s) {
     if (R < 0 || quota <= 0 || epr <= 0 || rpn <= 0 || rpn > kMaxBuckets || my_local < 0 || my_local >= rpn ||
         !i_send || (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0 || slot_pitch < quota || gate_pitch < quota)
         return TERRACE_EINVAL;
@@ -1052,7 +1071,7 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
     int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
     KeyAffine key{rslot, 0, epr, rpn, quota, slot_pitch};
     EmitArrival emit{rslot, rgate, gate_bytes, quota, slot_pitch, gate_pitch, gate_pairs, r_idx, slot_idx, pair_pos,
-                     pos32, meta};
+                     pos32, meta, tags_out ? tags_in : nullptr, tags_in ? tags_out : nullptr};
     int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, P, s);
@@ -1123,7 +1142,8 @@ static int launch_zero_pad(const int32_t *start, int epr, int64_t capacity, void
 int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                      int gate_bytes, int quota, int first_slot, int n_local, int64_t capacity, void *permuted,
                      void *permuted_gate, int64_t *place, uint8_t *kept, int64_t *pair_of_place,
-                     int64_t *tokens_per_expert, int64_t *kept_per_expert, int32_t *status, void *ws, size_t ws_bytes,
+                     int64_t *tokens_per_expert, int64_t *kept_per_expert, const int64_t *tags_in,
+                     int64_t *place_by_tag, int64_t n_tags, int32_t *status, void *ws, size_t ws_bytes,
                      hipStream_t s) {
     if (R < 0 || quota <= 0 || n_local <= 0 || n_local > kMaxBuckets || first_slot < 0 || !tokens_per_expert ||
         (gate_bytes != 2 && gate_bytes != 4) || row_bytes < 0 ||
@@ -1148,8 +1168,10 @@ int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, in
     int32_t *table = (int32_t *)ws;
     int32_t *pos32 = (int32_t *)((char *)ws + table_bytes);
     KeyAffine key{rslot, (int64_t)first_slot, 1, n_local, quota, (int64_t)quota};
+    const bool tagged = tags_in && place_by_tag && n_tags > 0;
     EmitHopB emit{rgate, gate_bytes, quota, (int64_t)quota, capacity, place, kept, pair_of_place,
-                  rgate ? permuted_gate : nullptr, pos32};
+                  rgate ? permuted_gate : nullptr, pos32, tagged ? tags_in : nullptr,
+                  tagged ? place_by_tag : nullptr, n_tags};
     int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *start = table + units_start_at(u);
@@ -1206,7 +1228,8 @@ size_t regroup_workspace(int64_t P, int epr, int64_t capacity) {
 int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate, int64_t P, int64_t row_bytes,
                 int gate_bytes, int epr, int my_local, int64_t capacity, void *permuted, void *permuted_gate,
                 int64_t *order, int64_t *dest, uint8_t *kept, int64_t *tokens_per_expert, int64_t *kept_per_expert,
-                int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch, hipStream_t s) {
+                int32_t *status, void *ws, size_t ws_bytes, int64_t slot_pitch, int64_t gate_pitch,
+                const int64_t *tags_in, int64_t *place_by_tag, int64_t n_tags, hipStream_t s) {
     if (P < 0 || epr <= 0 || epr > kMaxBuckets || my_local < 0 || !tokens_per_expert || row_bytes < 0 ||
         slot_pitch < 1 || gate_pitch < 1 ||
         (gate_bytes != 2 && gate_bytes != 4) || P >= (int64_t)1 << 31 ||
@@ -1229,7 +1252,9 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     int32_t *order32 = (int32_t *)((char *)ws + table_bytes);
     int32_t *gidx = (int32_t *)((char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
     KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr, 1, slot_pitch};
-    EmitRegroup emit{capacity, order, dest, kept, order32};
+    const bool tagged = tags_in && place_by_tag && n_tags > 0;
+    EmitRegroup emit{capacity, order, dest, kept, order32, tagged ? tags_in : nullptr,
+                     tagged ? place_by_tag : nullptr, n_tags};
     int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *src_of_place = order32;
@@ -1279,7 +1304,7 @@ size_t k2_workspace(int64_t T, int k, int n_nodes, int groups_m) {
     const int64_t S = T * groups_m;
     if (S <= 0 || n_nodes <= 0 || n_nodes > kMaxBuckets) return 256;
     const size_t item_path = units_table_bytes(make_units(S, n_nodes)) + align_up((size_t)S * sizeof(int32_t), 256);
-    const size_t token_path = k2_token_path_applies(T, k, n_nodes) ? k2_token_workspace(T, n_nodes, groups_m) : 0;
+    const size_t token_path = k2_token_path_applies(T, k, n_nodes) ? k2_token_workspace(T, k, n_nodes, groups_m) : 0;
     return item_path > token_path ? item_path : token_path;
 }
 
@@ -1288,13 +1313,14 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
                     int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                     int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                     int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                    int64_t *token_rows, void *gate_sorted, int32_t *status, const Units &u, int32_t *table,
-                    int32_t *pos32, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
+                    int64_t *token_rows, void *gate_sorted, int64_t *pair_src, int64_t *combine_table,
+                    int32_t *status, const Units &u, int32_t *table, int32_t *pos32, int64_t mask_pitch,
+                    int64_t gate_pitch, int gate_pad, hipStream_t s) {
     const int quota = k / groups_m;
     KeyRun<KMAX> key{expert_idx, k, groups_m, quota, slots, n_nodes};
     EmitPack<KMAX> emit{expert_idx, gates, gate_bytes, k, groups_m, quota, slots, n_experts,
                         mask, u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_rows, gate_sorted,
-                        pos32, mask_pitch, gate_pitch, gate_pad};
+                        pos32, pair_src, combine_table, mask_pitch, gate_pitch, gate_pad};
     int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
@@ -1304,8 +1330,8 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
                 int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, void *payload, int64_t *mask,
                 void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node, int64_t *inverse,
                 int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order, int64_t *token_rows,
-                void *gate_sorted, int32_t *status, void *ws, size_t ws_bytes, int64_t mask_pitch, int64_t gate_pitch,
-                int gate_pad, hipStream_t s) {
+                void *gate_sorted, int64_t *pair_src, int64_t *combine_table, int32_t *status, void *ws,
+                size_t ws_bytes, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s) {
     if (mask_pitch <= 0) mask_pitch = groups_m > 0 ? k / groups_m : 0;       // dense planes
     if (gate_pitch <= 0) gate_pitch = groups_m > 0 ? k / groups_m : 0;
     if (T < 0 || k <= 0 || world <= 0 || rpn <= 0 || n_experts <= 0 || groups_m <= 0 || world % rpn ||
@@ -1321,8 +1347,8 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
     if (k2_token_path_applies(T, k, n_nodes))
         return run_k2_token(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts,
                             groups_m, payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets,
-                            pair_table, sort_order, token_rows, gate_sorted, status, ws, mask_pitch, gate_pitch,
-                            gate_pad, s);
+                            pair_table, sort_order, token_rows, gate_sorted, pair_src, combine_table, status, ws,
+                            mask_pitch, gate_pitch, gate_pad, s);
     const Units u = make_units(S, n_nodes);
     const size_t table_bytes = units_table_bytes(u);
     int32_t *table = (int32_t *)ws;
@@ -1330,7 +1356,8 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
 #define TERRACE_K2(KM)                                                                                        \
     run_k2_t<KM>(hidden, expert_idx, gates, T, row_bytes, gate_bytes, k, slots, n_nodes, n_experts, groups_m, \
                  payload, mask, gate_rows, u_src, node_counts, u_node, inverse, node_offsets, pair_table,     \
-                 sort_order, token_rows, gate_sorted, status, u, table, pos32, mask_pitch, gate_pitch, gate_pad, s)
+                 sort_order, token_rows, gate_sorted, pair_src, combine_table, status, u, table, pos32, mask_pitch,   \
+                 gate_pitch, gate_pad, s)
     if (k <= 8) return TERRACE_K2(8);
     if (k <= 16) return TERRACE_K2(16);
     return TERRACE_K2(0);
@@ -1352,7 +1379,7 @@ int run_k2_pack_move(const void *hidden, int64_t T, int64_t row_bytes, int k, in
     if (!hidden || !payload || !ws) return TERRACE_EINVAL;
     if (ws_bytes < k2_workspace(T, k, n_nodes, groups_m)) return TERRACE_ENOSPC;
     const int32_t *pos32 = k2_token_path_applies(T, k, n_nodes)
-                               ? k2_token_positions(ws, T, n_nodes)
+                               ? k2_token_positions(ws, T, k, n_nodes)
                                : (const int32_t *)((const char *)ws + units_table_bytes(make_units(S, n_nodes)));
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
 }

@@ -36,9 +36,12 @@ Units make_units(int64_t n_items, int n_buckets);
 void finish_units(Units &u);
 size_t units_table_bytes(const Units &u);
 // Words of the table region: [n_units * n_buckets] counts or prefixes, then start[n_buckets + 1], then (direct)
-// blocktot[n_buckets * n_blocks].
+// blocktot[n_buckets * n_blocks], then census[n_blocks * 4] (the send side's per-workgroup guard quantities).
 __host__ __device__ inline int64_t units_start_at(const Units &u) { return (int64_t)u.n_units * u.n_buckets; }
 __host__ __device__ inline int64_t units_blocktot_at(const Units &u) { return units_start_at(u) + u.n_buckets + 1; }
+__host__ __device__ inline int64_t units_census_at(const Units &u) {
+    return units_blocktot_at(u) + (int64_t)u.n_buckets * u.n_blocks;
+}
 
 // Scan path: exclusive prefix over the bucket-major count table table[b * n_units + unit], in place; also
 // start[b] (n_buckets + 1 int32 right after the table), the optional histogram / offsets planes
@@ -108,11 +111,11 @@ __device__ __forceinline__ void direct_block_base(const Units &u, int32_t *__res
     }
 }
 
-// Direct path, count side: called by every thread of a count workgroup once its waves' per-bucket counts sit in
-// LDS (counts[wave * n_buckets + b], idle waves hold zeros) and a __syncthreads() has passed.  Writes each unit's
-// exclusive prefix inside the workgroup and the workgroup's totals.
+// Direct path, count side: called by every thread of a count workgroup once the per-bucket counts of its u.wpb
+// units sit in LDS (counts[unit_in_block * n_buckets + b], units past the end hold zeros) and a __syncthreads() has
+// passed.  Writes each unit's exclusive prefix inside the workgroup and the workgroup's totals.
 __device__ __forceinline__ void direct_block_counts(const Units &u, int32_t *__restrict__ table, lds_i32 *counts) {
-    const int nw = (int)(blockDim.x >> 6), me = (int)blockIdx.x;
+    const int nw = u.wpb, me = (int)blockIdx.x;
     int32_t *blocktot = table + units_blocktot_at(u);
     for (int i = threadIdx.x; i < nw * u.n_buckets; i += blockDim.x) {
         const int ww = i / u.n_buckets, b = i - ww * u.n_buckets;
@@ -136,14 +139,14 @@ int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, 
 // the direct path); returns false when the geometry is outside that and the caller must take the (token, run)-item
 // path.
 bool k2_token_path_applies(int64_t T, int k, int n_nodes);
-size_t k2_token_workspace(int64_t T, int n_nodes, int groups_m);
+size_t k2_token_workspace(int64_t T, int k, int n_nodes, int groups_m);
 // Where run_k2_token leaves the [T, groups_m] int32 send-row positions inside its workspace.
-const int32_t *k2_token_positions(const void *ws, int64_t T, int n_nodes);
+const int32_t *k2_token_positions(const void *ws, int64_t T, int k, int n_nodes);
 int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
                  int gate_bytes, int k, int slots, int n_nodes, int n_experts, int groups_m, void *payload,
                  int64_t *mask, void *gate_rows, int64_t *u_src, int64_t *node_counts, int64_t *u_node,
                  int64_t *inverse, int64_t *node_offsets, int64_t *pair_table, int64_t *sort_order,
-                 int64_t *token_rows, void *gate_sorted, int32_t *status, void *ws, int64_t mask_pitch,
-                 int64_t gate_pitch, int gate_pad, hipStream_t s);
+                 int64_t *token_rows, void *gate_sorted, int64_t *pair_src, int64_t *combine_table, int32_t *status,
+                 void *ws, int64_t mask_pitch, int64_t gate_pitch, int gate_pad, hipStream_t s);
 
 }  // namespace terrace

@@ -39,17 +39,17 @@ SIGNATURES = {
     "terrace_argsort_small": (_I, [_P, _L, _I, _P, _P, _P, _P, _Z, _P]),
     "terrace_k2_pack_workspace": (_Z, [_L, _I, _I, _I]),
     "terrace_k2_pack": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I,
-                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_pack_quota_wire": (_I, [_P, _P, _P, _L, _I, _I, _L, _I, _I, _P, _P, _P, _P]),
     "terrace_k1_arrival_workspace": (_Z, [_L, _I, _I]),
     "terrace_k1_arrival": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I,
-                                _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+                                _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_regroup_workspace": (_Z, [_L, _I, _L]),
     "terrace_regroup": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _L,
-                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+                             _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _Z, _P]),
     "terrace_hopb_scatter_workspace": (_Z, [_L, _I, _I]),
     "terrace_hopb_scatter": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _L,
-                                  _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+                                  _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _P, _Z, _P]),
     "terrace_hopb_scatter_move": (_I, [_P, _L, _L, _I, _I, _L, _P, _P, _Z, _P]),
     "terrace_gather_rows": (_I, [_P, _L, _P, _L, _L, _P, _P]),
     "terrace_scatter_rows": (_I, [_P, _P, _L, _I, _L, _P, _L, _P]),

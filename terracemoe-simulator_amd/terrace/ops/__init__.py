@@ -124,11 +124,12 @@ def _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local):
 
 
 def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=False, status_out=None,
-                   workspace_out=None):
+                   workspace_out=None, tags=None, tags_out=None):
     """(send_buf, gate_pairs, r_idx, slot_idx, i_send[, pair_pos]) -- one library call.
 
     ``rx`` None: the index planes only (``send_buf`` is None); the workspace, which then holds what
-    :func:`k1_arrival_move` needs, is appended to the list ``workspace_out``."""
+    :func:`k1_arrival_move` needs, is appended to the list ``workspace_out``.  ``tags`` ([P] int64, one per pair):
+    the same values in arrival order are appended to the list ``tags_out``."""
     _require()
     _hip.need_device(rx, rslot, rgate)
     _check_k1(rx, rslot, rgate, quota, epr, rpn, my_local)
@@ -146,16 +147,35 @@ def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=
     slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
     pair_pos = torch.empty((P,), dtype=torch.int64, device=dev) if want_pair_pos else None
+    carried = None
+    if tags is not None:
+        tags = _tag_plane(tags, P, dev)
+        carried = torch.empty((P,), dtype=torch.int64, device=dev)
     st = status_out if status_out is not None else _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
     _hip.call("terrace_k1_arrival", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, row_bytes,
               rgate.element_size(), quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(gate_pairs),
-              _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(st),
-              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+              _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(tags),
+              _hip.ptr(carried), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     if workspace_out is not None:
         workspace_out.append(ws)
+    if tags_out is not None:
+        tags_out.append(carried)
     out = (send_buf, gate_pairs, r_idx, slot_idx, i_send)
     return out + (pair_pos,) if want_pair_pos else out
+
+
+def _tag_plane(tags, n, dev):
+    tags = tags.contiguous().reshape(-1)
+    if tags.dtype != torch.int64 or tags.numel() != n or tags.device != dev:
+        raise RuntimeError(f"tags must be an int64 plane of {n} entries on {dev}")
+    return tags
+
+
+def _table_plane(table):
+    if table.dtype != torch.int64 or not table.is_contiguous():
+        raise RuntimeError("the table the tags index must be a contiguous int64 tensor")
+    return table
 
 
 def k1_arrival_static(rx, rslot, rgate, quota, epr, rpn, my_local, out):
@@ -206,19 +226,27 @@ def _check_k2(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
                          f"groups_m={groups_m} not divisible")
 
 
-def _k2_extras(T, k, n_nodes, groups_m, gate_dtype, dev):
-    """The send side's optional planes: what plan_ta2a returns beside u_src, and the combine's per-token tables."""
+def _k2_extras(T, k, n_nodes, groups_m, gate_dtype, dev, combine_table=False):
+    """The send side's optional planes: what plan_ta2a returns beside u_src, and the combine's per-token tables.
+    With ``combine_table`` also ``pair_src`` (entry t*k+s behind each Hop-A pair) and ``where`` [T, k], the
+    combine's place table, which the send side only pre-sets (-1) where a malformed routing leaves a rank without
+    a pair: a later stage fills it through the pairs' tags."""
     i64 = dict(dtype=torch.int64, device=dev)
-    return {"u_node": torch.empty((T * groups_m,), **i64), "inverse": torch.empty((T * k,), **i64),
-            "node_offsets": torch.empty((n_nodes,), **i64), "pair_table": torch.empty((T, k), **i64),
-            "sort_order": torch.empty((T, k), **i64), "token_rows": torch.empty((T, groups_m), **i64),
-            "gate_sorted": torch.empty((T, k), dtype=gate_dtype, device=dev)}
+    ex = {"u_node": torch.empty((T * groups_m,), **i64), "inverse": torch.empty((T * k,), **i64),
+          "node_offsets": torch.empty((n_nodes,), **i64), "pair_table": torch.empty((T, k), **i64),
+          "sort_order": torch.empty((T, k), **i64), "token_rows": torch.empty((T, groups_m), **i64),
+          "gate_sorted": torch.empty((T, k), dtype=gate_dtype, device=dev)}
+    if combine_table:
+        ex["pair_src"] = torch.empty((T * k,), **i64)
+        ex["where"] = torch.empty((T, k), **i64)
+    return ex
 
 
-def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=False, status_out=None):
+def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=False, status_out=None,
+                combine_table=False):
     """(payload, mask, gate_rows, u_src, node_counts) and, with ``extras``, a dict holding
     u_node, inverse, node_offsets, pair_table, sort_order, token_rows, gate_sorted and the
-    status words.
+    status words (with ``combine_table`` also pair_src and the pre-set ``where`` table, see ``_k2_extras``).
 
     ``hidden`` None: the index planes only (``payload`` is None); ``extras["workspace"]`` then
     holds what :func:`k2_pack_move` needs."""
@@ -238,7 +266,7 @@ def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extr
     gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
     u_src = torch.empty((S,), dtype=torch.int64, device=dev)
     node_counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
-    ex = _k2_extras(T, k, n_nodes, groups_m, gates.dtype, dev) if extras else {}
+    ex = _k2_extras(T, k, n_nodes, groups_m, gates.dtype, dev, combine_table) if extras else {}
     st = status_out if status_out is not None else _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
     _hip.call("terrace_k2_pack", _hip.ptr(hidden), _hip.ptr(expert_idx), _hip.ptr(gates), T,
@@ -246,7 +274,8 @@ def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extr
               _hip.ptr(payload), _hip.ptr(mask), _hip.ptr(gate_rows), _hip.ptr(u_src), _hip.ptr(node_counts),
               _hip.ptr(ex.get("u_node")), _hip.ptr(ex.get("inverse")), _hip.ptr(ex.get("node_offsets")),
               _hip.ptr(ex.get("pair_table")), _hip.ptr(ex.get("sort_order")), _hip.ptr(ex.get("token_rows")),
-              _hip.ptr(ex.get("gate_sorted")), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+              _hip.ptr(ex.get("gate_sorted")), _hip.ptr(ex.get("pair_src")), _hip.ptr(ex.get("where")), _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     out = (payload, mask, gate_rows, u_src, node_counts)
     if extras:
         ex["status"] = st
@@ -369,13 +398,16 @@ def plan_raw(expert_idx, world, n_experts, rpn, groups_m):
     ws = _hip.workspace(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m), dev)
     _hip.call("terrace_k2_pack", None, _hip.ptr(expert_idx), None, T, 0, 4, k, world, n_experts, rpn, groups_m,
               None, _hip.ptr(mask), None, _hip.ptr(u_src), _hip.ptr(counts), _hip.ptr(u_node),
-              _hip.ptr(inverse), None, None, None, None, None, _hip.ptr(st), _hip.ptr(ws), ws.numel(),
+              _hip.ptr(inverse), None, None, None, None, None, None, None, _hip.ptr(st), _hip.ptr(ws), ws.numel(),
               _hip.stream(dev))
     return u_src, u_node, counts, inverse, mask, st
 
 
-def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
+def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None, tags=None, table=None):
     """Expert-order regroup of the rows an expert card received.
+
+    ``tags`` ([P] int64) with ``table`` (int64, any shape): ``table.view(-1)[tags[p]]`` is set to the place of
+    row p (-1 when dropped), in place.
 
     Drop-less (``capacity=None``; terrace/ta2a_fwd.py:641-646 of the reference):
     returns ``(permuted, order, tokens_per_expert)`` (+ ``permuted_gate`` when ``my_gate``).
@@ -407,12 +439,16 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
         my_gate = my_gate.contiguous().reshape(-1)
         gate_bytes = my_gate.element_size()
         pgate = torch.empty((places,), dtype=my_gate.dtype, device=dev)
+    n_tags = 0
+    if tags is not None:
+        tags, table = _tag_plane(tags, P, dev), _table_plane(table)
+        n_tags = table.numel()
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, cap), dev)
     _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), _hip.ptr(my_gate), P,
               H * node_rx.element_size(), gate_bytes, epr, my_local, cap, _hip.ptr(permuted), _hip.ptr(pgate),
-              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st),
-              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(tags),
+              _hip.ptr(table), n_tags, _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     if capacity is None:
         out = (permuted, order, tpe)
     else:
@@ -421,7 +457,7 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None):
 
 
 def hopb_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None, want_pairs=False,
-                 workspace_out=None):
+                 workspace_out=None, tags=None, table=None):
     """Hop-B local scatter in one pass: what ``k1_arrival`` followed by ``regroup(epr=n_local)`` produce when
     every slot the arrived rows name is local to this GPU, without the send buffer between them.
 
@@ -431,7 +467,7 @@ def hopb_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None, 
     ``rgate`` is given) and, with ``want_pairs``, ``pair_of_place`` (-1 on padding).
 
     ``rx`` None: the index planes only; the workspace :func:`hopb_scatter_move` needs is appended to
-    ``workspace_out``."""
+    ``workspace_out``.  ``tags`` ([P] int64) with ``table`` (int64): ``table.view(-1)[tags[p]] = place[p]``, in place."""
     _require()
     _hip.need_device(rx, rslot, rgate)
     if rslot.dim() != 2 or rslot.dtype != torch.int64 or rslot.shape[1] != quota:
@@ -463,11 +499,16 @@ def hopb_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None, 
     kept = torch.empty((P,), dtype=torch.uint8, device=dev) if capacity is not None else None
     pairs = torch.empty((places,), **i64) if want_pairs else None
     tpe, kpe = torch.empty((n_local,), **i64), torch.empty((n_local,), **i64)
+    n_tags = 0
+    if tags is not None:
+        tags, table = _tag_plane(tags, P, dev), _table_plane(table)
+        n_tags = table.numel()
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_hopb_scatter_workspace", R, quota, n_local), dev)
     _hip.call("terrace_hopb_scatter", _hip.ptr(rx), _hip.ptr(rslot), _hip.ptr(rgate), R, row_bytes, gate_bytes, quota,
               first_slot, n_local, cap, _hip.ptr(permuted), _hip.ptr(pgate), _hip.ptr(place), _hip.ptr(kept),
-              _hip.ptr(pairs), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+              _hip.ptr(pairs), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(tags), _hip.ptr(table), n_tags, _hip.ptr(st),
+              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     if workspace_out is not None:
         workspace_out.append(ws)
     return {"permuted": permuted, "place": place, "kept": None if kept is None else kept.view(torch.bool),
@@ -553,8 +594,8 @@ def regroup_index(my_slot, epr, my_local=0, capacity=None):
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, cap), dev)
     _hip.call("terrace_regroup", None, _hip.ptr(my_slot), None, P, 0, 4, epr, my_local, cap, None, None,
-              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(st),
-              _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+              _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), None, None, 0,
+              _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     return {"tokens_per_expert": tpe, "kept_per_expert": kpe, "dest": dest, "order": order,
             "kept": None if kept is None else kept.view(torch.bool), "workspace": ws}
 

@@ -185,15 +185,21 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
     if overlap is None:
         overlap = os.environ.get("TERRACE_OVERLAP", "0") == "1"
     if not overlap or x.shape[0] == 0:
+        # the combine's [T, k] place table is filled on the way: every Hop-A pair carries the entry it answers
+        # (pair_src) through the arrival reorder, and the regroup writes the pair's place there
         (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
-            x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+            x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True, combine_table=True)
+        carried = []
         send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = _ops.k1_arrival_raw(
-            payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True)
+            payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True, tags=extras["pair_src"],
+            tags_out=carried)
         if capacity is None:
-            permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots)
+            permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots, tags=carried[0],
+                                                              table=extras["where"])
             kept = None
         else:
-            permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity)
+            permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity,
+                                                            tags=carried[0], table=extras["where"])
         return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
                              slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
 
@@ -238,15 +244,16 @@ def loopback_dispatch_onepass(x, expert_idx, gates, world: int, n_experts: int, 
     slots = epr * rpn
     quota = expert_idx.shape[1] // groups_m
     (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
-        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
-    hb = _ops.hopb_scatter(payload, mask, None, quota, slots, 0, capacity)
+        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True, combine_table=True)
+    hb = _ops.hopb_scatter(payload, mask, None, quota, slots, 0, capacity, tags=extras["pair_src"],
+                           table=extras["where"])
     return OnePassState(payload, mask, gate_rows, u_src, node_counts, extras, hb["permuted"], hb["tokens_per_expert"],
                         hb["place"], hb["kept"], capacity)
 
 
-def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
+def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None, tags=None, table=None):
     """Drop-less regroup that also returns each input row's place (the inverse of ``order``):
-    (permuted, order, tokens_per_expert, place[, permuted_gate])."""
+    (permuted, order, tokens_per_expert, place[, permuted_gate]).  ``tags`` / ``table`` as in ``ops.regroup``."""
     _ops._require()
     node_rx, my_slot = node_rx.contiguous(), my_slot.contiguous().reshape(-1)
     dev = my_slot.device
@@ -260,12 +267,16 @@ def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None):
         my_gate = my_gate.contiguous().reshape(-1)
         gate_bytes = my_gate.element_size()
         pgate = torch.empty((P,), dtype=my_gate.dtype, device=dev)
+    n_tags = 0
+    if tags is not None:
+        tags, table = _ops._tag_plane(tags, P, dev), _ops._table_plane(table)
+        n_tags = table.numel()
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, -1), dev)
     _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), _hip.ptr(my_gate), P,
               H * node_rx.element_size(), gate_bytes, epr, my_local, -1, _hip.ptr(permuted), _hip.ptr(pgate),
-              _hip.ptr(order), _hip.ptr(place), None, _hip.ptr(tpe), None, _hip.ptr(st), _hip.ptr(ws), ws.numel(),
-              _hip.stream(dev))
+              _hip.ptr(order), _hip.ptr(place), None, _hip.ptr(tpe), None, _hip.ptr(tags), _hip.ptr(table), n_tags,
+              _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     out = (permuted, order, tpe, place)
     return out + (pgate,) if my_gate is not None else out
 

@@ -139,6 +139,14 @@ def _check_every_plane(cfg):
         same(hb["kept"], o_kept, "one-pass kept")
     st1 = loopback_dispatch_onepass(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
     assert torch.equal(st1.permuted, st.permuted) and torch.equal(st1.place, st.place[st.pair_pos])
+    # ---- the combine's place table, filled on the way through the pairs' tags (no look-up launch)
+    o_pair_tab, _ = orc.token_pair_table(oe, inverse, cfg.quota)
+    o_where = place[pos[o_pair_tab]]
+    o_pair_src = np.empty(cfg.pairs, dtype=np.int64)
+    o_pair_src[o_pair_tab.reshape(-1)] = np.arange(cfg.T * cfg.top_k)
+    same(st.extras["pair_src"], o_pair_src, "pair_src")
+    same(st.extras["where"], o_where, "where (two-step dispatch)"), same(st1.extras["where"], o_where, "where (one pass)")
+    assert torch.equal(st.extras["where"], tops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"]))
     # ---- experts: row * (expert id + 1) / E, or fresh fp8 rows for the fp8 workload
     n_places = perm.shape[0]
     if cfg.fmt == "fp8":
@@ -233,7 +241,10 @@ def test_full_size_index_planes_and_round_trip(name):
     assert torch.equal(st1.place, st.place[st.pair_pos]) and torch.equal(st1.tokens_per_expert, st.tokens_per_expert)
     if cap is not None:
         assert torch.equal(st1.kept, st.kept[st.pair_pos])
-    del st1
+    import terrace.ops as tops
+    looked_up = tops.index_chain2(st.place, st.pair_pos, st.extras["pair_table"])
+    assert torch.equal(st.extras["where"], looked_up) and torch.equal(st1.extras["where"], looked_up)
+    del st1, looked_up
     # ---- round trip with identity experts: y[t] = x[t] * (sum of the token's kept gates)
     got = loopback_combine(st.permuted, st, out_dtype=cfg.out_dtype,
                            fp8_hidden=cfg.hidden if cfg.fmt == "fp8" else None).float()

@@ -106,8 +106,8 @@ def test_hopb_scatter_refuses_bad_arguments_and_contains_bad_ids():
     ws = torch.zeros(1 << 16, dtype=torch.uint8, device=DEV)
     st = torch.zeros(4, dtype=torch.int32, device=DEV)
     args = lambda R, quota, n_local, cap, ws_bytes: (None, _hip.ptr(i64), None, R, 0, 4, quota, 0, n_local, cap, None,
-                                                     None, _hip.ptr(i64), None, None, _hip.ptr(i64), None, _hip.ptr(st),
-                                                     _hip.ptr(ws), ws_bytes, s)
+                                                     None, _hip.ptr(i64), None, None, _hip.ptr(i64), None, None, None, 0,
+                                                     _hip.ptr(st), _hip.ptr(ws), ws_bytes, s)
     assert lib.terrace_hopb_scatter(*args(16, 2, 0, -1, ws.numel())) == _hip.EINVAL
     assert lib.terrace_hopb_scatter(*args(16, 0, 8, -1, ws.numel())) == _hip.EINVAL
     assert lib.terrace_hopb_scatter(*args(16, 2, 8, -1, 16)) == _hip.ENOSPC
