@@ -1,6 +1,7 @@
 """Benchmark of one rank's dispatch/combine path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--graph]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--no-other-configs]
+                    [--graph]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM: T-Route -> dispatch index build + Hop-A deduplicated pack -> Hop-B arrival chain ->
@@ -10,18 +11,23 @@ part of the path; its output is a fixed synthetic tensor prepared before the tim
 The all-to-all exchanges are not executed (one GPU): the rank's Hop-A send buffer is looped
 back as its arrival buffer.
 
-Prints ONE JSON line: whole-step algorithmic GB/s as `value` (each payload row counted once on the
-read side and once on the write side of every stage) and, beside it, the same step priced on the
-bytes that must cross HBM (`min_traffic`); per-stage ms / GB/s / fraction of the 8 TB/s HBM peak
-and the arrival chain's us/row in `stages`, the roofline record of
-the slowest row-moving kernel (timed alone with HIP events on the launch stream), and the CPU
-oracle timed on the host cores over a bounded sample of the same workload.
+Prints ONE JSON line.  `value` is the whole step priced on the bytes that must cross HBM (a scatter
+reads each source row once however many copies it writes; a capacity layout reads only the rows it
+keeps) over the step time; no figure in the line named `frac_hbm_peak` uses any other convention.
+The convention that counts a payload row once on the read and once on the write side of every stage
+is reported beside it as `rows_counted_twice_GBps` only.  Also in the line: per-stage ms / GB/s /
+fraction of the 8 TB/s HBM peak and the arrival chain's us/row (`stages`), the same step with Hop B
+as one pass (`onepass`), the other four workloads (`other_configs`), the roofline record of the
+slowest row-moving kernel (timed alone with HIP events on the launch stream; `traffic` from
+profiles/traffic.json when that file was measured on the sources the loaded library was built
+from), and the CPU baseline: the path as a chain of torch CPU operators on the host cores.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -31,10 +37,7 @@ for _p in (ROOT, os.path.join(ROOT, "terracemoe-simulator_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of a workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE
-# and WRITE_SIZE and scaled by the same counters' reading for the copy kernel (fetch x2.00,
-# write x1.00).  Only workloads that have been measured are listed; others report null.
-MEASURED_TRAFFIC_BYTES = {("c2", "gather_rows_sliced_kernel(regroup)"): 3.767e9}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 REFERENCE_TARGET_US_PER_ROW = 0.012     # the reference's fused-chain design target
 
 
@@ -45,11 +48,12 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="also capture the step into a HIP graph and time its replays (reported beside the eager "
                          "figure, which stays `value`)")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1 << 20,
-                    help="tokens of the workload the CPU baseline runs on (default: all of them)")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1024,
+                    help="tokens of the workload the torch-CPU chain runs on")
     return ap.parse_args()
 
 
@@ -66,126 +70,202 @@ def event_ms(fn, reps, torch):
     return start.elapsed_time(stop) / reps
 
 
-def cpu_baseline(cfg, sample_tokens):
-    """The CPU oracle timed on the host cores over `sample_tokens` tokens of the same geometry:
-    the OpenMP C restatement (oracle/terrace_oracle.c) when its library is built, else the numpy
-    one.  Passes are repeated for about eight seconds (3 to 40 of them: the hosts are shared and noisy) and
-    each stage's best time counts; algorithmic GB/s over the same stage set as the GPU figure."""
+def wall_ms(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def measured_traffic(workload, kernel, digest):
+    """HBM bytes per launch of `kernel` on `workload` from profiles/traffic.json (rocprofv3 --pmc FETCH_SIZE and
+    WRITE_SIZE, scaled by the copy kernel's reading), or None when the file was measured on other sources."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if rec.get("source_digest") != digest:
+        return None
+    return rec.get("bytes_per_launch", {}).get(f"{workload}:{kernel}")
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# CPU baseline
+# ------------------------------------------------------------------------------------------------------------------
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _torch_chain_pass(tch, torch, cfg, inp, x, ye_of):
+    """One pass of the operator chain; per-stage seconds."""
+    t = {}
+    t0 = time.perf_counter()
+    e, gates, _ = tch.t_route(inp["logits"], inp["bias"], cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups,
+                              inp["gate_affinity"])
+    t["route"] = time.perf_counter() - t0
+    gq = gates.to(cfg.gate_dtype)
+    t0 = time.perf_counter()
+    payload, mask, gate_rows, u_src, _counts, _inv = tch.k2_pack(x, e, gq, cfg.world, cfg.n_experts, cfg.rpn,
+                                                                 cfg.top_groups)
+    t["pack"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    send, gp, r_idx, s_idx, _i_send, _ordo = tch.k1_arrival(payload, mask, gate_rows, cfg.quota, cfg.epr, cfg.rpn)
+    t["arrival"] = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    perm, place, _tpe = tch.regroup(send, s_idx, cfg.slots, cfg.capacity(cfg.slots))
+    t["regroup"] = time.perf_counter() - t0
+    ye = ye_of(perm)
+    t0 = time.perf_counter()
+    tch.combine_two_level(ye, place, r_idx, gp, u_src, u_src.numel(), cfg.T)
+    t["combine"] = time.perf_counter() - t0
+    return t
+
+
+def torch_chain_baseline(cfg, sample_tokens, threads):
+    """Median-of-10 per stage (3 warm-up passes) of the torch-CPU operator chain on `sample_tokens` tokens of the
+    workload, at `threads` intra-op threads."""
+    import torch
+    from oracle import torch_chain as tch
+    from terrace import configs
+    small = cfg.scaled(min(sample_tokens, cfg.T))
+    inp = configs.make_inputs(small)
+    x = inp["x"]
+    if small.fmt == "fp8":          # the rows travel as bytes; the expert output is dequantised where the combine reads it
+        h = small.hidden
+
+        def ye_of(perm):
+            codes = perm[:, :h].contiguous().view(torch.float8_e4m3fn).float()
+            scales = perm[:, h:].contiguous().view(torch.float32).repeat_interleave(configs.FP8_BLOCK, dim=1)
+            return (codes * scales).to(torch.bfloat16)
+    else:
+        def ye_of(perm):
+            return perm
+    before = torch.get_num_threads()
+    torch.set_num_threads(threads)
+    try:
+        for _ in range(3):
+            _torch_chain_pass(tch, torch, small, inp, x, ye_of)
+        passes = [_torch_chain_pass(tch, torch, small, inp, x, ye_of) for _ in range(10)]
+    finally:
+        torch.set_num_threads(before)
+    med = {k: statistics.median(p[k] for p in passes) for k in passes[0]}
+    total = sum(med.values())
+    kept = None
+    nbytes = sum(configs.minimum_traffic_bytes(small, kept, None if small.capacity(small.slots) is None
+                                               else small.slots * small.capacity(small.slots)).values())
+    return {"threads": threads, "tokens": small.T, "GBps": round(nbytes / total / 1e9, 3),
+            "ms_per_pass": round(total * 1e3, 2), "stage_ms": {k: round(v * 1e3, 3) for k, v in med.items()},
+            "arrival_us_per_row": round(med["arrival"] * 1e6 / small.pairs, 4),
+            "repetitions": len(passes), "statistic": "median per stage"}
+
+
+def openmp_port_baseline(cfg):
+    """The OpenMP C restatement (oracle/terrace_oracle.c) over the whole workload; None when it is not built."""
     import numpy as np
     import torch
     from oracle import c_oracle as corc
     from oracle import terrace_oracle as orc
     from terrace import configs
-    use_c = corc.available()
-    small = cfg.scaled(min(sample_tokens if use_c else min(sample_tokens, 1024), cfg.T))
-    inp = configs.make_inputs(small)
+    if not corc.available():
+        return None
+    inp = configs.make_inputs(cfg)
     logits, bias = inp["logits"].numpy(), inp["bias"].numpy()
     ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].numpy()
-    if small.fmt == "f32":
+    if cfg.fmt == "f32":
         x, gcast, fmt = inp["x"].numpy(), (lambda g: g), "f32"
-    elif small.fmt == "bf16":
+    elif cfg.fmt == "bf16":
         x, gcast, fmt = inp["x"].view(torch.int16).numpy().view(np.uint16), orc.f32_to_bf16, "bf16"
     else:
         x, gcast, fmt = inp["x"].numpy(), orc.f32_to_bf16, "fp8"
-    impl = corc if use_c else orc
-    best, totals, began = None, [], time.perf_counter()
-    while len(totals) < 3 or (len(totals) < 40 and time.perf_counter() - began < 8.0):
-        t = _oracle_pass(impl, orc, np, small, logits, bias, ga, x, gcast, fmt, use_c)
-        totals.append(sum(t.values()))
-        best = t if best is None else {k: min(best[k], t[k]) for k in t}
-    t = best
-    nbytes = sum(configs.algorithmic_bytes(small).values())
-    total = sum(t.values())
-    cores = corc.threads() if use_c else 1
-    what = f"OpenMP C oracle ({cores} threads)" if use_c else "numpy oracle (1 thread)"
-    return {"value": round(nbytes / total / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{what}, whole path on {small.T} of {cfg.T} tokens of {cfg.name}, each stage's best of "
-                      f"{len(totals)} passes ({total:.3f} s: " + ", ".join(f"{k} {v:.3f}" for k, v in t.items()) +
-                      f"; whole passes took {min(totals):.3f} to {max(totals):.3f} s, median "
-                      f"{sorted(totals)[len(totals) // 2]:.3f})",
-            "arrival_us_per_row": round(t["arrival"] * 1e6 / small.pairs, 4)}
+    passes, began = [], time.perf_counter()
+    while len(passes) < 3 or (len(passes) < 12 and time.perf_counter() - began < 6.0):
+        passes.append(_openmp_pass(corc, np, cfg, logits, bias, ga, x, gcast, fmt))
+    med = {k: statistics.median(p[k] for p in passes) for k in passes[0]}
+    total = sum(med.values())
+    cap = cfg.capacity(cfg.slots)
+    nbytes = sum(configs.minimum_traffic_bytes(cfg, None, None if cap is None else cfg.slots * cap).values())
+    return {"threads": corc.threads(), "tokens": cfg.T, "GBps": round(nbytes / total / 1e9, 3),
+            "ms_per_pass": round(total * 1e3, 2), "stage_ms": {k: round(v * 1e3, 3) for k, v in med.items()},
+            "arrival_us_per_row": round(med["arrival"] * 1e6 / cfg.pairs, 4), "repetitions": len(passes),
+            "statistic": "median per stage"}
 
 
-def _oracle_pass(impl, orc, np, small, logits, bias, ga, x, gcast, fmt, use_c):
+def _openmp_pass(impl, np, cfg, logits, bias, ga, x, gcast, fmt):
     t = {}
     t0 = time.perf_counter()
-    if use_c:
-        e, gates, _ = impl.t_route(logits, bias, small.n_experts, small.n_groups, small.top_k, small.top_groups,
-                                   2, ga)
-    else:
-        e, gates, _ = impl.t_route(logits, bias, small.n_experts, small.n_groups, small.top_k, small.top_groups,
-                                   gate_affinity=ga)
+    e, gates, _ = impl.t_route(logits, bias, cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups, 2, ga)
     t["route"] = time.perf_counter() - t0
     gq = gcast(gates)
     t0 = time.perf_counter()
-    packed = impl.k2_pack(x, e, gq, small.world, small.n_experts, small.rpn, small.top_groups)
-    payload, mask, gate_rows = packed[0], packed[1], packed[2]
+    packed = impl.k2_pack(x, e, gq, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups)
     t["pack"] = time.perf_counter() - t0
     t0 = time.perf_counter()
-    arrived = impl.k1_arrival(payload, mask, gate_rows, small.quota, small.epr, small.rpn)
-    send, s_idx = arrived[0], arrived[3]
+    arrived = impl.k1_arrival(packed[0], packed[1], packed[2], cfg.quota, cfg.epr, cfg.rpn)
     t["arrival"] = time.perf_counter() - t0
     t0 = time.perf_counter()
-    cap = small.capacity(small.slots)
-    if use_c:
-        perm, place, _kept, _tpe = impl.regroup(send, s_idx, small.slots, 0, cap)
-    elif cap is None:
-        perm, order, _tpe = impl.regroup(send, s_idx, small.slots)
-        place = np.empty_like(order)
-        place[order] = np.arange(order.size)
-    else:
-        perm, place, _kept, _tpe, _kpe = impl.regroup(send, s_idx, small.slots, capacity=cap)
+    perm, place, _kept, _tpe = impl.regroup(arrived[0], arrived[3], cfg.slots, 0, cfg.capacity(cfg.slots))
     t["regroup"] = time.perf_counter() - t0
     t0 = time.perf_counter()
-    if use_c:
-        pair_tab, sort_order, pos = packed[5]["pair_table"], packed[5]["sort_order"], arrived[5]
-    else:
-        _, _, _, inverse = orc.plan_ta2a(e, small.world, small.n_experts, small.rpn, small.top_groups)
-        pair_tab, sort_order = orc.token_pair_table(e, inverse, small.quota)
-        pos = orc.arrival_positions(mask, small.epr, small.rpn)
-    where = place[pos[pair_tab]]
-    w_sorted = np.take_along_axis(gates, sort_order, 1)
-    impl.combine(perm, where, w_sorted, fmt, "f32" if fmt == "f32" else "bf16", hidden=small.hidden)
+    where = place[arrived[5][packed[5]["pair_table"]]]
+    w_sorted = np.take_along_axis(gates, packed[5]["sort_order"], 1)
+    impl.combine(perm, where, w_sorted, fmt, "f32" if fmt == "f32" else "bf16", hidden=cfg.hidden)
     t["combine"] = time.perf_counter() - t0
     return t
 
 
-def main():
-    args = parse()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build measures one GPU's share of the path; the all-to-all exchanges "
-              "between ranks are not part of it, so --gpus must be 1", file=sys.stderr)
-        sys.exit(2)
-    import torch
+def cpu_baseline(cfg, sample_tokens):
+    cores = os.cpu_count() or 1
+    one = torch_chain_baseline(cfg, sample_tokens, 1)
+    many = torch_chain_baseline(cfg, sample_tokens, cores) if cores > 1 else one
+    port = openmp_port_baseline(cfg)
+    return {"value": many["GBps"], "unit": "GB/s", "cores": many["threads"], "kind": "port",
+            "sample": f"the path as a chain of torch CPU operators (oracle/torch_chain.py: topk/gather, "
+                      f"scatter_+cumsum+searchsorted, row gathers, composite-key argsort+scatter_add_, index_add_) on "
+                      f"{many['tokens']} of {cfg.T} tokens of {cfg.name}, 3 warm-up passes then the median of 10 per "
+                      f"stage, at {many['threads']} threads; same bytes-that-must-cross-memory pricing as `value`",
+            "cpu_model": _cpu_model(), "host_cores_available": cores,
+            "torch_chain_1_thread": one, "torch_chain_all_threads": many, "openmp_c_port_whole_workload": port}
 
+
+# ------------------------------------------------------------------------------------------------------------------
+# one workload on the GPU
+# ------------------------------------------------------------------------------------------------------------------
+
+def run_workload(cfg, args, torch, detail):
+    """Times the step (two-step Hop B: the drop-in operators), the same step with Hop B as one pass, and --
+    with `detail` -- every stage and every row mover alone.  Returns a dict of figures."""
     import terrace
     import terrace.ops as tops
-    from terrace import _hip, configs
-    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
+    from terrace import configs
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, loopback_dispatch_onepass
 
-    if not torch.cuda.is_available():
-        print("bench.py: no ROCm device", file=sys.stderr)
-        sys.exit(3)
-    st = tops.status()
-    if not st.loaded:
-        print(f"bench.py: kernel library not loaded: {st.reason}", file=sys.stderr)
-        sys.exit(3)
-    cfg = configs.CONFIGS[args.config]
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-
     inp = configs.make_inputs(cfg)
     logits, bias, x = inp["logits"].to(dev), inp["bias"].to(dev), inp["x"].to(dev)
     gate_aff = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(dev)
     rcfg = terrace.TRouteConfig(cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups)
     cap = cfg.capacity(cfg.slots)
     fp8_hidden = cfg.hidden if cfg.fmt == "fp8" else None
+    geom = (cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
 
     def route():            # the gates leave the kernel in the payload dtype: no cast launch between the stages
         return terrace.t_route(logits, bias, rcfg, gate_affinity=gate_aff, gates_dtype=cfg.gate_dtype)
 
     e, gates, _ = route()
-    state = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+    state = loopback_dispatch(x, e, gates, *geom)
     # fixed synthetic expert output, one row per place of the expert-order buffer
     if cfg.fmt == "fp8":
         g = torch.Generator(device=dev).manual_seed(cfg.seed)
@@ -196,20 +276,128 @@ def main():
 
     def step():
         e_, g_, _ = route()
-        s_ = loopback_dispatch(x, e_, g_, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
+        s_ = loopback_dispatch(x, e_, g_, *geom)
         return loopback_combine(ye, s_, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def step_onepass():
+        e_, g_, _ = route()
+        s_ = loopback_dispatch_onepass(x, e_, g_, *geom)
+        return loopback_combine(ye, s_, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
 
-    # ---- optional: the same step as one HIP graph (launch overhead off the critical path) ----
-    graph_rec = None
+    y_two = step()
+    same_y = bool(torch.equal(y_two, step_onepass()))
+    del y_two
+    ms_per_step = wall_ms(step, args.steps, args.warmup, torch)
+    ms_onepass = wall_ms(step_onepass, args.steps, args.warmup, torch)
+
+    kept_pairs = int((state.place >= 0).sum()) if cap is not None else None
+    places = None if cap is None else cfg.slots * cap
+    phys = configs.minimum_traffic_bytes(cfg, kept_pairs, places)
+    conv = configs.algorithmic_bytes(cfg)
+    hopb_bytes = configs.onepass_traffic_bytes(cfg, places)
+    onepass_bytes = phys["route"] + phys["pack"] + hopb_bytes + phys["combine"]
+    reps = max(args.steps, 5)
+    quota = cfg.quota
+
+    def arrival():
+        return tops.k1_arrival_raw(state.payload, state.mask, state.gate_rows, quota, cfg.epr, cfg.rpn, 0,
+                                   want_pair_pos=True)
+
+    def pack():
+        return tops.k2_pack_raw(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, extras=True)
+
+    def combine():
+        return loopback_combine(ye, state, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+
+    def hopb():
+        return tops.hopb_scatter(state.payload, state.mask, None, quota, cfg.slots, 0, cap)
+
+    gbps = lambda nbytes, ms: nbytes / ms / 1e6
+    out = {
+        "ms_per_step": ms_per_step,
+        "GBps": gbps(sum(phys.values()), ms_per_step),
+        "rows_counted_twice_GBps": gbps(sum(conv.values()), ms_per_step),
+        "onepass": {"ms_per_step": round(ms_onepass, 4), "GBps": round(gbps(onepass_bytes, ms_onepass), 1),
+                    "frac_hbm_peak": round(gbps(onepass_bytes, ms_onepass) / HBM_PEAK_GBPS, 4),
+                    "same_output_as_two_step": same_y,
+                    "note": "Hop B as one scatter from the arrived rows to their expert-order places "
+                            "(terrace_hopb_scatter) instead of arrival chain + regroup; priced on its own bytes"},
+        "kept_pairs": kept_pairs, "places": places, "phys": phys, "conv": conv, "hopb_bytes": hopb_bytes,
+    }
+    if not detail:
+        ms_arr, ms_pack, ms_comb = event_ms(arrival, reps, torch), event_ms(pack, reps, torch), event_ms(combine, reps, torch)
+        out["arrival_us_per_row"] = ms_arr * 1e3 / cfg.pairs
+        out["pack_plus_combine_frac_hbm_peak"] = gbps(phys["pack"] + phys["combine"], ms_pack + ms_comb) / HBM_PEAK_GBPS
+        return out
+
+    # ---- per-stage timings (each stage alone, HIP events on the launch stream) ----
+    def regroup():
+        return tops.regroup(state.send_buf, state.slot_idx, cfg.slots, 0, cap)
+
+    stage_ms = {"route": event_ms(route, reps, torch), "pack": event_ms(pack, reps, torch),
+                "arrival": event_ms(arrival, reps, torch), "regroup": event_ms(regroup, reps, torch),
+                "combine": event_ms(combine, reps, torch)}
+    ms_hopb = event_ms(hopb, reps, torch)
+    # rows a stage writes: send rows, (row, slot) pairs, places of the expert-order buffer, tokens
+    rows_out = {"route": cfg.T, "pack": cfg.send_rows, "arrival": cfg.pairs,
+                "regroup": cfg.pairs if cap is None else places, "combine": cfg.T}
+    stages = {}
+    for name, ms in stage_ms.items():
+        stages[name] = {"ms": round(ms, 4), "GBps": round(gbps(phys[name], ms), 1),
+                        "frac_hbm_peak": round(gbps(phys[name], ms) / HBM_PEAK_GBPS, 4),
+                        "rows_counted_twice_GBps": round(gbps(conv[name], ms), 1),
+                        "us_per_row": round(ms * 1e3 / max(rows_out[name], 1), 6)}
+    stages["arrival"]["reference_target_us_per_row"] = REFERENCE_TARGET_US_PER_ROW
+    stages["hopb_onepass"] = {"ms": round(ms_hopb, 4), "GBps": round(gbps(hopb_bytes, ms_hopb), 1),
+                              "frac_hbm_peak": round(gbps(hopb_bytes, ms_hopb) / HBM_PEAK_GBPS, 4),
+                              "us_per_row": round(ms_hopb * 1e3 / cfg.pairs, 6),
+                              "replaces": "arrival + regroup",
+                              "two_step_ms": round(stage_ms["arrival"] + stage_ms["regroup"], 4)}
+    pc_ms = stage_ms["pack"] + stage_ms["combine"]
+    out["stages"] = stages
+    out["pack_plus_combine"] = {
+        "ms": round(pc_ms, 4), "GBps": round(gbps(phys["pack"] + phys["combine"], pc_ms), 1),
+        "frac_hbm_peak": round(gbps(phys["pack"] + phys["combine"], pc_ms) / HBM_PEAK_GBPS, 4),
+        "rows_counted_twice_GBps": round(gbps(conv["pack"] + conv["combine"], pc_ms), 1), "target_frac_hbm_peak": 0.70}
+
+    # ---- the row-moving kernels alone ----
+    row = cfg.row_bytes
+    where, w_sorted = state.extras["where"], state.extras["gate_sorted"]
+    token_rows, pair_pos2 = state.extras["token_rows"], state.pair_pos.view(cfg.send_rows, quota)
+    if cap is None:
+        _, order, _ = tops.regroup(state.send_buf, state.slot_idx, cfg.slots, 0, None)
+        gather_idx = order
+    else:
+        gather_idx = torch.full((places,), -1, dtype=torch.int64, device=dev)
+        ok = state.place >= 0
+        gather_idx[state.place[ok]] = torch.arange(cfg.pairs, device=dev)[ok]
+    place_of_pair = state.place[state.pair_pos].view(cfg.send_rows, quota).contiguous()
+    n_places = cfg.pairs if cap is None else places
+    kept = cfg.pairs if kept_pairs is None else kept_pairs
+    out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
+    # names of the kernels the library picks for this row width (whole kilobytes or not)
+    kb_rows = row % 1024 == 0
+    k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
+    k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
+    kernels = {     # name: (launch, bytes that must cross HBM per launch)
+        f"{k_scatter}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), (cfg.T + cfg.send_rows) * row),
+        f"{k_scatter}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
+                                  (cfg.send_rows + cfg.pairs) * row),
+        f"{k_scatter}(hopb_onepass)": (lambda: tops.scatter_rows(state.payload, place_of_pair, n_places),
+                                       (cfg.send_rows + kept) * row),
+        f"{k_gather}(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx), (kept + n_places) * row),
+        "combine_kernel": (lambda: tops.combine(ye, where, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
+                           kept * row + cfg.pairs * 12 + cfg.T * out_row),
+        "copy_kernel(passthrough)": (lambda: tops.passthrough(state.send_buf), 2 * state.send_buf.numel()
+                                     * state.send_buf.element_size()),
+    }
+    kern = {}
+    for name, (fn, nb) in kernels.items():
+        ms = event_ms(fn, reps, torch)
+        kern[name] = {"ms": round(ms, 4), "bytes_per_launch": nb, "GBps": round(nb / ms / 1e6, 1),
+                      "frac_hbm_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    out["kernels"] = kern
+    out["graph"] = None
     if args.graph:
         y_eager = step()
         side = torch.cuda.Stream()
@@ -232,121 +420,91 @@ def main():
         for _ in range(args.steps):
             graph.replay()
         torch.cuda.synchronize()
-        graph_rec = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / args.steps, 4),
-                     "replays_match_eager": same}
+        out["graph"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / args.steps, 4),
+                        "replays_match_eager": same}
+    return out
 
-    # ---- per-stage timings (each stage alone, HIP events on the launch stream) ----
-    nbytes = configs.algorithmic_bytes(cfg)
-    reps = max(args.steps, 5)
-    quota = cfg.quota
 
-    def pack():
-        return tops.k2_pack_raw(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, extras=True)
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU's share of the path; the all-to-all exchanges "
+              "between ranks are not part of it, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
 
-    def arrival():
-        return tops.k1_arrival_raw(state.payload, state.mask, state.gate_rows, quota, cfg.epr, cfg.rpn, 0,
-                                   want_pair_pos=True)
+    import terrace.ops as tops
+    from terrace import _hip, configs
 
-    def regroup():
-        return tops.regroup(state.send_buf, state.slot_idx, cfg.slots, 0, cap)
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm device", file=sys.stderr)
+        sys.exit(3)
+    st = tops.status()
+    if not st.loaded:
+        print(f"bench.py: kernel library not loaded: {st.reason}", file=sys.stderr)
+        sys.exit(3)
+    digest = _hip.load().terrace_version().decode().rsplit("src:", 1)[-1]
+    cfg = configs.CONFIGS[args.config]
+    torch.cuda.set_device(0)
 
-    def combine():
-        return loopback_combine(ye, state, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+    r = run_workload(cfg, args, torch, detail=True)
+    kern, stages = r["kernels"], r["stages"]
+    dominant = max((k for k in kern if not k.startswith("copy") and "onepass" not in k), key=lambda k: kern[k]["ms"])
+    # algorithmic bytes of the dominant kernel per launch: every row it moves, read once and written once
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": kern[dominant]["GBps"], "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": kern[dominant]["frac_hbm_peak"],
+                "traffic": measured_traffic(args.config, dominant, digest),
+                "traffic_source": "profiles/traffic.json (null when measured on other sources than the loaded library's)",
+                "avg_launch_ms": kern[dominant]["ms"], "algorithmic_bytes_per_launch": kern[dominant]["bytes_per_launch"]}
 
-    stage_ms = {"route": event_ms(route, reps, torch), "pack": event_ms(pack, reps, torch),
-                "arrival": event_ms(arrival, reps, torch), "regroup": event_ms(regroup, reps, torch),
-                "combine": event_ms(combine, reps, torch)}
-    kept_pairs = int((state.place >= 0).sum()) if cap is not None else None
-    min_bytes = configs.minimum_traffic_bytes(cfg, kept_pairs, None if cap is None else cfg.slots * cap)
-    stages = {}
-    # rows a stage writes: send rows, (row, slot) pairs, places of the expert-order buffer, tokens
-    rows_out = {"route": cfg.T, "pack": cfg.send_rows, "arrival": cfg.pairs,
-                "regroup": cfg.pairs if cap is None else cfg.slots * cap, "combine": cfg.T}
-    for name, ms in stage_ms.items():
-        gbps = nbytes[name] / ms / 1e6
-        min_gbps = min_bytes[name] / ms / 1e6
-        # "GBps" follows the convention that counts a payload row once on the read and once on the write side of
-        # a stage (a scatter that reads a row once for all its copies can thus exceed the peak); "min_traffic"
-        # prices the bytes that must cross HBM
-        stages[name] = {"ms": round(ms, 4), "GBps": round(gbps, 1), "frac_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
-                        "min_traffic_GBps": round(min_gbps, 1),
-                        "min_traffic_frac_hbm_peak": round(min_gbps / HBM_PEAK_GBPS, 4),
-                        "us_per_row": round(ms * 1e3 / max(rows_out[name], 1), 6)}
-    stages["arrival"]["reference_target_us_per_row"] = REFERENCE_TARGET_US_PER_ROW
-    pc_bytes = nbytes["pack"] + nbytes["combine"]
-    pc_ms = stage_ms["pack"] + stage_ms["combine"]
-
-    # ---- the row-moving kernels alone ----
-    row = cfg.row_bytes
-    where = tops.index_chain2(state.place, state.pair_pos, state.extras["pair_table"])
-    w_sorted = state.extras["gate_sorted"]
-    token_rows, pair_pos2 = state.extras["token_rows"], state.pair_pos.view(cfg.send_rows, quota)
-    if cap is None:
-        _, order, _ = tops.regroup(state.send_buf, state.slot_idx, cfg.slots, 0, None)
-        gather_idx = order
-    else:
-        gather_idx = torch.full((cfg.slots * cap,), -1, dtype=torch.int64, device=dev)
-        ok = state.place >= 0
-        gather_idx[state.place[ok]] = torch.arange(cfg.pairs, device=dev)[ok]
-    out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
-    # names of the kernels the library picks for this row width (whole kilobytes or not)
-    kb_rows = row % 1024 == 0
-    k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
-    k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
-    kernels = {
-        f"{k_scatter}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), 2 * cfg.send_rows * row),
-        f"{k_scatter}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
-                                  2 * cfg.pairs * row),
-        f"{k_gather}(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx),
-                                 2 * gather_idx.numel() * row),
-        "combine_kernel": (lambda: tops.combine(ye, where, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
-                           cfg.pairs * row + cfg.pairs * 12 + cfg.T * out_row),
-        "copy_kernel(passthrough)": (lambda: tops.passthrough(state.send_buf), 2 * state.send_buf.numel()
-                                     * state.send_buf.element_size()),
-    }
-    kern = {}
-    for name, (fn, nb) in kernels.items():
-        ms = event_ms(fn, reps, torch)
-        kern[name] = {"ms": round(ms, 4), "algorithmic_bytes": nb, "GBps": round(nb / ms / 1e6, 1)}
-    dominant = max((k for k in kern if not k.startswith("copy")), key=lambda k: kern[k]["ms"])
-    achieved = kern[dominant]["GBps"]
-    roofline = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dominant)),
-                "avg_launch_ms": kern[dominant]["ms"], "algorithmic_bytes_per_launch": kern[dominant]["algorithmic_bytes"]}
-
-    total_bytes = sum(nbytes.values())
-    value = total_bytes / ms_per_step / 1e6
+    cap = cfg.capacity(cfg.slots)
+    value = r["GBps"]
     out = {
-        "metric": "dispatch_combine_algorithmic_GBps",
+        "metric": "dispatch_combine_GBps_on_bytes_that_cross_HBM",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"f32": "f32", "bf16": "bf16", "fp8": "fp8_e4m3+f32 scales"}[cfg.fmt] + " rows, fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": cfg.name, "T": cfg.T, "E": cfg.n_experts, "n_groups": cfg.n_groups, "k": cfg.top_k,
-                   "M": cfg.top_groups, "cards_per_group": cfg.rpn, "hidden": cfg.hidden, "row_bytes": row,
+                   "M": cfg.top_groups, "cards_per_group": cfg.rpn, "hidden": cfg.hidden, "row_bytes": cfg.row_bytes,
                    "send_rows": cfg.send_rows, "pairs": cfg.pairs, "capacity": cap,
                    "exchange": "loop-back (no all-to-all on one GPU)",
                    "expert_outputs": "fixed synthetic tensor prepared before the timed region"},
         "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-        "min_traffic": {"GBps": round(sum(min_bytes.values()) / ms_per_step / 1e6, 1),
-                        "frac_hbm_peak": round(sum(min_bytes.values()) / ms_per_step / 1e6 / HBM_PEAK_GBPS, 4),
-                        "note": "bytes that must cross HBM: a scatter reads each source row once however many "
-                                "copies it writes, a capacity layout reads only the rows it keeps"},
-        "pack_plus_combine": {"GBps": round(pc_bytes / pc_ms / 1e6, 1),
-                              "frac_hbm_peak": round(pc_bytes / pc_ms / 1e6 / HBM_PEAK_GBPS, 4),
-                              "min_traffic_GBps": round((min_bytes["pack"] + min_bytes["combine"]) / pc_ms / 1e6, 1),
-                              "min_traffic_frac_hbm_peak": round((min_bytes["pack"] + min_bytes["combine"]) / pc_ms
-                                                                 / 1e6 / HBM_PEAK_GBPS, 4)},
+        "bytes_per_step": sum(r["phys"].values()),
+        "rows_counted_twice_GBps": round(r["rows_counted_twice_GBps"], 1),
+        "pricing": "value, every GBps and every frac_hbm_peak: bytes that must cross HBM (a scatter reads each source "
+                   "row once however many copies it writes; a capacity layout reads only the rows it keeps). "
+                   "rows_counted_twice_GBps: a payload row counted once on the read and once on the write side of "
+                   "every stage (can exceed the peak for a scatter; never used for a fraction)",
+        "pack_plus_combine": r["pack_plus_combine"],
         "arrival_chain_us_per_row": stages["arrival"]["us_per_row"],
+        "onepass": r["onepass"],
         "stages": stages, "kernels": kern, "roofline": roofline,
-        "library": os.path.relpath(st.lib, ROOT),
+        "library": os.path.relpath(st.lib, ROOT), "source_digest": digest,
     }
-    if graph_rec is not None:
-        out["hip_graph"] = graph_rec
+    if r["graph"] is not None:
+        out["hip_graph"] = r["graph"]
+    del r
+    torch.cuda.empty_cache()
+    if not args.no_other_configs:
+        others = {}
+        for name, c in configs.CONFIGS.items():
+            if name == args.config:
+                continue
+            o = run_workload(c, args, torch, detail=False)
+            others[name] = {"workload": c.name, "ms_per_step": round(o["ms_per_step"], 4), "GBps": round(o["GBps"], 1),
+                            "frac_hbm_peak": round(o["GBps"] / HBM_PEAK_GBPS, 4),
+                            "arrival_us_per_row": round(o["arrival_us_per_row"], 6),
+                            "pack_plus_combine_frac_hbm_peak": round(o["pack_plus_combine_frac_hbm_peak"], 4),
+                            "onepass_ms_per_step": o["onepass"]["ms_per_step"],
+                            "onepass_frac_hbm_peak": o["onepass"]["frac_hbm_peak"],
+                            "onepass_same_output": o["onepass"]["same_output_as_two_step"]}
+            del o
+            torch.cuda.empty_cache()
+        out["other_configs"] = others
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_tokens)
-        out["cpu_baseline"]["host_cores_available"] = os.cpu_count()
     print(json.dumps(out))
 
 

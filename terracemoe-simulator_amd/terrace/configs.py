@@ -166,3 +166,13 @@ def minimum_traffic_bytes(cfg: PathConfig, kept_pairs: int | None = None, places
         "regroup": alg["regroup"] - 2 * P * row + (kept + places) * row,
         "combine": alg["combine"] - P * row + kept * row,
     }
+
+
+def onepass_traffic_bytes(cfg: PathConfig, places: int | None = None) -> int:
+    """HBM bytes the one-pass Hop-B scatter cannot avoid: every arrived row read once, every row of the
+    expert-order buffer written once (kept rows and zero padding rows alike), the slot table read and the
+    place / tag planes written."""
+    S, P, row = cfg.send_rows, cfg.pairs, cfg.row_bytes
+    places = P if places is None else places
+    return (S + places) * row + P * 8 + P * (8 + 8 + 8)
+
