@@ -90,7 +90,8 @@ TERRACE_API int terrace_passthrough(const void *x, void *y, size_t nbytes, terra
  * [T,E] f32 or NULL (= affinity).  Writes expert_idx [T,k] i64, gates [T,k] f32 (bf16 / f16 with the mode flags),
  * group_idx [T,G] i64 with G = top_groups (full, group_limited), n_groups (quota_only) or
  * top_k (global_topk).  Ties go to the lowest index; gates are raw/sum(raw) with the sum
- * taken left to right in fp32.  pool = TRouteConfig.group_score_pool (1 or 2). */
+ * taken left to right in fp32.  pool = TRouteConfig.group_score_pool (>= 1): a group's score is the mean of its
+ * top-min(pool, g) scores, added from the largest down in fp32 and divided once (pool 2: an exact halving). */
 TERRACE_API int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T,
                     int n_experts, int n_groups, int top_k, int top_groups, int pool, int mode,
                     int64_t *expert_idx, void *gates, int64_t *group_idx, terrace_stream_t stream);

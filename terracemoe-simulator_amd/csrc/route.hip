@@ -334,13 +334,36 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
         int n_sel_groups = 0, per_group = 0;
         if (mode == TERRACE_ROUTE_FULL || mode == TERRACE_ROUTE_GROUP_LIMITED) {
             for (int G = lane; G < n_groups; G += kWave) {
-                float a1 = kNegInf, a2 = kNegInf;
-                for (int x = 0; x < g; ++x) {
-                    const float v = s[G * g + x];
-                    a2 = fmaxf(fminf(a1, v), a2);
-                    a1 = fmaxf(a1, v);
+                const int p = pool < g ? pool : g;                     // mean of the top-min(pool, g)
+                if (p <= 2) {
+                    float a1 = kNegInf, a2 = kNegInf;
+                    for (int x = 0; x < g; ++x) {
+                        const float v = s[G * g + x];
+                        a2 = fmaxf(fminf(a1, v), a2);
+                        a1 = fmaxf(a1, v);
+                    }
+                    gsc[G] = p == 2 ? __fmul_rn(__fadd_rn(a1, a2), 0.5f) : a1;
+                } else {
+                    // the p largest, one after the other in (value desc, index asc) order, added from the
+                    // largest down and divided once: fl(fl(..fl(v1 + v2).. + vp) / p)
+                    float acc = 0.0f, pv = kPosInf;
+                    int pi = -1;
+                    for (int i = 0; i < p; ++i) {
+                        float cv = kNegInf;
+                        int ci = 0x7FFFFFFF;
+                        for (int x = 0; x < g; ++x) {
+                            const float v = s[G * g + x];
+                            if (after(v, x, pv, pi) && ahead(v, x, cv, ci)) {
+                                cv = v;
+                                ci = x;
+                            }
+                        }
+                        acc = i == 0 ? cv : __fadd_rn(acc, cv);
+                        pv = cv;
+                        pi = ci;
+                    }
+                    gsc[G] = __fdiv_rn(acc, (float)p);
                 }
-                gsc[G] = (pool >= 2 && g >= 2) ? __fmul_rn(__fadd_rn(a1, a2), 0.5f) : a1;
             }
             __builtin_amdgcn_wave_barrier();
             float pv = kPosInf;
@@ -444,7 +467,7 @@ static bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
 int run_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int E, int n_groups,
                 int k, int M, int pool, int mode, int64_t *expert_idx, void *gates, int gate_dtype,
                 int64_t *group_idx, int force_generic, hipStream_t s) {
-    if (T < 0 || E <= 0 || n_groups <= 0 || k <= 0 || M <= 0 || pool < 1 || pool > 2 || mode < 0 || mode > 3 ||
+    if (T < 0 || E <= 0 || n_groups <= 0 || k <= 0 || M <= 0 || pool < 1 || mode < 0 || mode > 3 ||
         (gate_dtype != TERRACE_F32 && gate_dtype != TERRACE_BF16 && gate_dtype != TERRACE_F16))
         return TERRACE_EINVAL;
     if (E % n_groups || k % M || k > E || E > 2048 || M > n_groups) return TERRACE_EINVAL;
@@ -459,7 +482,8 @@ int run_t_route(const float *affinity, const float *bias, const float *gate_affi
     // groups of fewer than 4 experts, larger ones rows too long for 64 lanes of 4.  VPL must divide g
     // into a power-of-two number of lanes and leave the token k lanes for its outputs.
     const bool aligned = (((uintptr_t)affinity) & 15) == 0 && (!gate_affinity || (((uintptr_t)gate_affinity) & 15) == 0);
-    if (!force_generic && mode == TERRACE_ROUTE_FULL) {
+    // the register-resident form keeps a group's top two only; a wider pool takes the LDS-staged kernel
+    if (!force_generic && mode == TERRACE_ROUTE_FULL && (pool <= 2 || g <= 2)) {
         static const int kVplOrder[] = {4, 2, 1, 8, 16};
         for (int vpl : kVplOrder) {
             if (g % vpl || !is_pow2(g / vpl)) continue;

@@ -997,6 +997,26 @@ def _register_torch_ops():
     lib.impl("passthrough", lambda x: torch.empty_like(x), "Meta")
     lib.impl("k1_arrival", _k1_meta, "Meta")
     lib.impl("k2_pack", _k2_meta, "Meta")
+
+    # A call through torch.ops on tensors that require grad must not drop the gradient silently: the two float
+    # outputs of each operator hang on the same adjoints as the functional entry points.
+    def _below_autograd(op, *args):
+        with torch._C._AutoDispatchBelowAutograd():
+            return op(*args)
+
+    def _k1_autograd(rx, rslot, rgate, quota, epr, rpn, my_local):
+        if not rx.is_cuda:
+            return _below_autograd(torch.ops.terrace.k1_arrival, rx, rslot, rgate, quota, epr, rpn, my_local)
+        return TerraceK1ArrivalFn.apply(rx, rslot, rgate, quota, epr, rpn, my_local)
+
+    def _k2_autograd(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+        if not hidden.is_cuda:
+            return _below_autograd(torch.ops.terrace.k2_pack, hidden, expert_idx, gates, world, n_experts, rpn,
+                                   groups_m)
+        return TerraceK2PackFn.apply(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+
+    lib.impl("k1_arrival", _k1_autograd, "Autograd")
+    lib.impl("k2_pack", _k2_autograd, "Autograd")
     _TORCH_LIB = lib
 
 
@@ -1103,15 +1123,73 @@ def k1_arrival_segment(rx, rslot, rgate, quota: int, epr: int, rpn: int, my_loca
     return send_buf, gate_pairs, r_idx, slot_idx, i_send
 
 
+class TerraceK2PackFn(torch.autograd.Function):
+    """Forward = the send-side kernels; backward = the adjoints of the two differentiable outputs
+    (terrace/ops/k2_ref.py:77-81 of the reference: ``payload``, a deduplicated gather of ``hidden``, and
+    ``gate_rows``, a permutation gather of ``gates``, carry gradients), also as kernels: a token sums the
+    gradients of its M send rows in ascending row order, a gate takes the gradient of the one cell it was
+    copied to."""
+
+    @staticmethod
+    def forward(ctx, hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
+        (payload, mask, gate_rows, u_src, node_counts), ex = k2_pack_raw(
+            hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+        _guard_k2(ex["status"], expert_idx, world, rpn, groups_m)
+        ctx.save_for_backward(ex["token_rows"], ex["pair_table"], ex["sort_order"])
+        ctx.k2_dtypes = (hidden.dtype, gates.dtype)
+        ctx.mark_non_differentiable(mask, u_src, node_counts)
+        return payload, mask, gate_rows, u_src, node_counts
+
+    @staticmethod
+    def backward(ctx, g_payload, _g_mask, g_gate_rows, _g_src, _g_counts):
+        token_rows, pair_table, sort_order = ctx.saved_tensors
+        hidden_dtype, gates_dtype = ctx.k2_dtypes
+        d_hidden = d_gates = None
+        if ctx.needs_input_grad[0] and g_payload is not None:
+            d_hidden = combine(g_payload.contiguous(), token_rows, None, out_dtype=hidden_dtype)
+        if ctx.needs_input_grad[2] and g_gate_rows is not None:
+            T, k = pair_table.shape
+            by_rank = gather_rows(g_gate_rows.contiguous().to(gates_dtype).reshape(-1, 1), pair_table.reshape(-1))
+            d_gates = torch.zeros((T, k), dtype=gates_dtype, device=pair_table.device)
+            rows = torch.arange(T, device=pair_table.device, dtype=torch.int64).unsqueeze(1).expand(T, k)
+            scatter_elems(by_rank, rows, sort_order, d_gates)
+        return d_hidden, None, d_gates, None, None, None, None
+
+
+def _guard_k2(status, expert_idx, world, rpn, groups_m):
+    """The plan's guard (first call per shape and every 256th, one read-back when it fires) applied to the
+    status words of a send-side call: an id out of range, a fan-out other than M or a node off the quota
+    raise ValueError as in the reference (terrace/ta2a.py:161-204, terrace/ops/k2_ref.py:108)."""
+    from .. import ta2a as _plan            # deferred: ta2a imports this module
+    T, k = expert_idx.shape
+    _plan._guard(status, T, k, world // rpn, groups_m)
+
+
 def k2_pack(hidden, expert_idx, gates, world: int, n_experts: int, rpn: int, groups_m: int):
-    """Send-side fused chain: (payload, mask, gate_rows, u_src, node_counts)."""
+    """Send-side fused chain: (payload, mask, gate_rows, u_src, node_counts).  ``payload`` and ``gate_rows``
+    carry gradients to ``hidden`` and ``gates``; a malformed routing raises ValueError on the guard's cadence."""
     _require()
-    return k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+    if torch.is_grad_enabled() and (hidden.requires_grad or gates.requires_grad):
+        return TerraceK2PackFn.apply(hidden, expert_idx, gates, world, n_experts, rpn, groups_m)
+    out, ex = k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True)
+    _guard_k2(ex["status"], expert_idx, world, rpn, groups_m)
+    return out
+
+
+def k1_arrival_ref(rx, rslot, rgate, quota: int, epr: int, rpn: int, my_local: int = 0):
+    """The name under which the reference keeps the executable specification of K1
+    (terrace/ops/__init__.py:255-300 there: the composed torch chain).  This build has one implementation of
+    that specification, the kernels, so the name resolves to them: same arguments, same five outputs, same
+    gradients as :func:`k1_arrival`."""
+    if rslot.dim() == 2 and rslot.shape[1] != quota:
+        raise AssertionError(f"rslot dim 1 {rslot.shape[1]} != quota {quota} (quota wire-format contract)")
+    return k1_arrival(rx, rslot, rgate, quota, epr, rpn, my_local)
 
 
 __all__ = [
-    "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn",
-    "custom_ops_enabled", "k1_arrival", "k1_arrival_segment", "k2_pack", "passthrough", "reset", "status",
+    "OpsLoadError", "OpsState", "TerracePassthroughFn", "TerraceK1ArrivalFn", "TerraceK2PackFn",
+    "custom_ops_enabled", "k1_arrival", "k1_arrival_ref", "k1_arrival_segment", "k2_pack", "passthrough", "reset",
+    "status",
     "regroup", "combine", "gather_rows", "scatter_rows", "index_chain", "index_chain2", "hist", "argsort_small", "hopa_send_splits",
     "plan_general", "build_mask", "scatter_elems", "expand_mask", "arrival_pairs", "routing_map_topk", "segment_table", "pair_places",
     "wire_words", "k2_pack_wire", "k1_arrival_wire", "regroup_wire", "hopb_scatter", "hopb_scatter_move",

@@ -64,8 +64,8 @@ def t_route(affinity: torch.Tensor, bias: torch.Tensor, cfg: TRouteConfig, mode:
                          f"got {cfg.top_k // cfg.n_groups} experts/group")
     if mode == "quota_only" and cfg.top_k % cfg.n_groups:
         raise ValueError(f"quota_only needs top_k ({cfg.top_k}) divisible by n_groups ({cfg.n_groups})")
-    if cfg.group_score_pool not in (1, 2):
-        raise ValueError("this build implements group_score_pool 1 and 2")
+    if cfg.group_score_pool < 1:
+        raise ValueError(f"group_score_pool must be at least 1, got {cfg.group_score_pool}")
     _ops._require()
     _hip.need_device(affinity, bias, gate_affinity)
     if affinity.dim() != 2 or affinity.shape[1] != cfg.n_experts or bias.numel() != cfg.n_experts:

@@ -118,6 +118,26 @@ def test_route_ties_and_pool(generic):
     assert to_np(e)[0].tolist() == [0, 1, 8, 9, 16, 17, 24, 25]
 
 
+@pytest.mark.parametrize("mode", ["full", "group_limited"])
+@pytest.mark.parametrize("pool", [3, 4, 5, 8, 100])
+def test_route_group_score_pool_beyond_two(mode, pool):
+    """mean of the top-min(pool, g) scores of a group (terrace/routing.py:24,88), any pool: bit-exact against the
+    oracle's largest-first fp32 sum, ties and all-equal tokens included."""
+    import terrace
+    announce("route pool", mode, pool)
+    g = torch.Generator().manual_seed(pool)
+    for (T, E, Ng, k, M) in [(300, 64, 8, 8, 4), (130, 256, 8, 8, 4), (65, 24, 3, 6, 3), (40, 16, 8, 2, 2),
+                             (50, 96, 4, 8, 2)]:
+        aff = torch.rand(T, E, generator=g)
+        aff[1] = 0.5
+        aff[2, ::3] = 0.25
+        bias = torch.randn(E, generator=g) * 0.05
+        cfg = terrace.TRouteConfig(E, Ng, k, M, group_score_pool=pool)
+        e, gt, grp = terrace.t_route(aff.to(DEV), bias.to(DEV), cfg, mode=mode)
+        oe, og, ogrp = orc.t_route(aff.numpy(), bias.numpy(), E, Ng, k, M, pool=pool, mode=mode)
+        same(e, oe, "expert_idx"), same(grp, ogrp, "group_idx"), same(gt, og, "gates")
+
+
 @pytest.mark.parametrize("mode", ["group_limited", "quota_only", "global_topk"])
 def test_route_other_modes(mode):
     import terrace
@@ -796,3 +816,80 @@ def test_row_movers_at_every_base_alignment(row_bytes):
                     want[pos[r, f]] = src.cpu()[r]
         assert torch.equal(got, want), (off_src, off_dst)
         assert bool((dst_buf[:off_dst] == 0xCD).all()) and bool((dst_buf[off_dst + n_dst * row_bytes:] == 0xCD).all())
+
+
+# ------------------------------------------------------------------------------- K2 gradients, reference names
+
+@pytest.mark.parametrize("entry", ["functional", "torch_ops", "k2_pack_ref"])
+def test_k2_pack_backward_is_the_adjoint(literals, entry):
+    """payload = hidden[u_src] and gate_rows (a permutation gather of gates) carry gradients
+    (terrace/ops/k2_ref.py:77-81): both against float64 autograd over the oracle's index planes."""
+    import terrace.ops as tops
+    from terrace import ta2a
+    from terrace.ops.k2_ref import k2_pack_ref
+    for world, rpn, E, T, k, M in literals["k2_geometries"]["rows"] + [[64, 8, 256, 700, 8, 4]]:
+        announce("k2 backward", entry, (world, rpn, E, T, k, M))
+        ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+        q = k // M
+        e = equal_quota_routing(T, k, E, world // rpn, M, 31)
+        g = torch.Generator().manual_seed(T + k)
+        x, gates = torch.randn(T, 12, generator=g), torch.rand(T, k, generator=g)
+        Gp, Gg = torch.randn(T * M, 12, generator=g), torch.randn(T * M, q, generator=g)
+        xd, gd = x.to(DEV).requires_grad_(), gates.to(DEV).requires_grad_()
+        fn = {"functional": tops.k2_pack, "torch_ops": torch.ops.terrace.k2_pack, "k2_pack_ref": k2_pack_ref}[entry]
+        payload, mask, gate_rows, u_src, counts = fn(xd, torch.from_numpy(e).to(DEV), gd, world, E, rpn, M)
+        assert payload.requires_grad and gate_rows.requires_grad and not mask.requires_grad
+        o_payload, o_mask, o_gate_rows, o_src, o_counts = orc.k2_pack(x.numpy(), e, gates.numpy(), world, E, rpn, M)
+        same(payload, o_payload, "payload"), same(mask, o_mask, "mask"), same(gate_rows, o_gate_rows, "gate_rows")
+        same(u_src, o_src, "u_src"), same(counts, o_counts, "node_counts")
+        ((payload * Gp.to(DEV)).sum() + (gate_rows * Gg.to(DEV)).sum()).backward()
+        _, _, _, inverse = orc.plan_ta2a(e, world, E, rpn, M)
+        pair_tab, sort_order = orc.token_pair_table(e, inverse, q)
+        x64, g64 = x.double().requires_grad_(), gates.double().requires_grad_()
+        pay64 = x64[torch.from_numpy(o_src)]
+        # cell (row, i) of gate_rows holds gates[t, sort_order[t, s]] for the (t, s) whose pair id is row*q + i
+        flat = torch.zeros(T * k, dtype=torch.float64)
+        flat = flat.index_add(0, torch.from_numpy(pair_tab.reshape(-1)),
+                              g64.gather(1, torch.from_numpy(sort_order)).reshape(-1))
+        ((pay64 * Gp.double()).sum() + (flat.view(T * M, q) * Gg.double()).sum()).backward()
+        for name, got, want in (("hidden.grad", xd.grad, x64.grad), ("gates.grad", gd.grad, g64.grad)):
+            assert got is not None, f"{name} missing"
+            err = (got.cpu().double() - want).abs().max().item()
+            assert err <= 1e-5 * max(want.abs().max().item(), 1.0), f"{name} differs by {err}"
+
+
+def test_public_k2_pack_raises_on_a_malformed_routing_and_ref_names_resolve():
+    import terrace.ops as tops
+    from terrace import ta2a
+    from terrace.ops.k2_ref import k2_pack_ref
+    announce("k2 guard, reference names")
+    x = torch.randn(6, 16, device=DEV)
+    gts = torch.rand(6, 4, device=DEV)
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    with pytest.raises(ValueError, match="out of range"):
+        tops.k2_pack(x, torch.tensor([[0, 2, 4, 99]] * 6, device=DEV), gts, 4, 8, 2, 2)
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    with pytest.raises(ValueError, match="quota"):
+        tops.k2_pack(x, torch.tensor([[0, 2, 3, 5]] * 6, device=DEV), gts, 4, 8, 2, 2)
+    with pytest.raises(ValueError, match="out of range"):          # the reference function checks ids on every call
+        k2_pack_ref(x, torch.tensor([[0, 2, 4, 99]] * 6, device=DEV), gts, 4, 8, 2, 2)
+    with pytest.raises(ValueError, match="chain bound"):
+        k2_pack_ref(torch.randn(4, 8, device=DEV), torch.zeros(4, 2, dtype=torch.int64, device=DEV),
+                    torch.rand(4, 2, device=DEV), 8, 1024, 8, 1)
+    with pytest.raises(RuntimeError, match="dtype"):
+        k2_pack_ref(x.to(torch.bfloat16), torch.tensor([[0, 1, 4, 5]] * 6, device=DEV), gts, 4, 8, 2, 2)
+    # a repeated id inside a well-formed count pattern: every plane is defined and in range
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    e = torch.tensor([[0, 0, 4, 6], [1, 3, 5, 7]], device=DEV)
+    (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x[:2], e, gts[:2], 4, 8, 2, 2, extras=True)
+    assert ex["status"].tolist()[0] == 0                     # two per node on two nodes: the census cannot see it
+    assert sorted(ex["pair_table"][0].tolist()) == [0, 1, 4, 5] and ex["sort_order"][0].tolist() == [0, 1, 2, 3]
+    assert mask.tolist() == [[0, 0], [1, 3], [0, 2], [1, 3]] and ex["gate_sorted"][0].tolist() == gts[0].tolist()
+    assert gate_rows[0].tolist() == gts[0, :2].tolist() and gate_rows[2].tolist() == gts[0, 2:].tolist()
+    # k1_arrival_ref is the arrival operator under the reference's name
+    rslot = torch.from_numpy(arrival_plane(40, 2, 2, 8, 3)).to(DEV)
+    rx, rg = torch.randn(40, 8, device=DEV), torch.rand(40, 2, device=DEV)
+    for a, b in zip(tops.k1_arrival_ref(rx, rslot, rg, 2, 2, 8), tops.k1_arrival(rx, rslot, rg, 2, 2, 8)):
+        assert torch.equal(a, b)
+    with pytest.raises(AssertionError):
+        tops.k1_arrival_ref(rx, rslot, rg, 3, 2, 8)
