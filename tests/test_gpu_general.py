@@ -209,17 +209,18 @@ SEAM = [(4, 2, 8, 8, 4, 2, 6), (32, 8, 64, 48, 4, 2, 32), (32, 8, 96, 32, 8, 4, 
         (64, 8, 256, 1500, 8, 4, 128), (64, 8, 128, 33, 6, 3, 8)]
 
 
-@pytest.mark.parametrize("world,rpn,E,T,k,M,H", SEAM)
+# every geometry in the default container mode; the other two modes on the small geometries
+SEAM_CASES = [(geom, mode) for geom in SEAM for mode in ("small", "full", "off") if mode == "small" or geom[3] <= 100]
+
+
+@pytest.mark.parametrize("geom,mode", SEAM_CASES)
 @pytest.mark.parametrize("fmt", ["f32", "bf16"])
 @pytest.mark.parametrize("branch", ["quota", "general"])
-@pytest.mark.parametrize("mode", ["small", "full", "off"])
-def test_seam_halves_loopback(world, rpn, E, T, k, M, H, fmt, branch, mode, monkeypatch):
+def test_seam_halves_loopback(geom, fmt, branch, mode, monkeypatch):
     from terrace import ta2a, ta2a_pack
     from terrace.ta2a_dispatch import ta2a_permute, ta2a_unpermute
-    if (E // world) * rpn > 63 and branch == "general":
-        pytest.skip("bitmask branch needs <= 63 slots per node")
-    if mode != "small" and T > 100:
-        pytest.skip("container modes are covered on the small geometries")
+    world, rpn, E, T, k, M, H = geom
+    assert (E // world) * rpn <= 63, "every seam geometry fits the bitmask branch"
     announce("seam", (world, rpn, E, T, k, M, H), fmt, branch, mode)
     monkeypatch.setenv("TERRACE_TA2A_PACK", mode)
     ta2a_pack.reset()
@@ -380,3 +381,96 @@ def test_seam_refuses_process_groups_and_mismatched_probs():
                      groups_m=2)
     with pytest.raises(RuntimeError, match="dtypes match"):
         ta2a_permute(x.bfloat16(), torch.rand(4, 8, device=DEV), rm, world=4, rank=0, rpn=2, n_experts=8, groups_m=2)
+
+
+# ------------------------------------------------------------------------------- the overlap seam
+
+@pytest.mark.parametrize("world,rpn,E,T,k,M,H", [(4, 2, 8, 8, 4, 2, 6), (32, 8, 64, 48, 4, 2, 32), (64, 8, 256, 300, 8, 4, 64)])
+@pytest.mark.parametrize("branch", ["quota", "general"])
+@pytest.mark.parametrize("pack_mode", ["small", "off"])
+def test_overlap_seam_seats_and_hand_replayed_backward(world, rpn, E, T, k, M, H, branch, pack_mode, monkeypatch):
+    """The overlap halves append 7 + 3 save_tensors entries at the positions the vendor layer's hand-written
+    backward unpacks (terrace/ta2a_dispatch.py:519-535 of the reference), give the forward values of the plain
+    halves, and -- replayed segment by segment the way that backward does it -- the plain halves' gradients."""
+    from terrace import ta2a, ta2a_pack
+    from terrace.ta2a_dispatch import (ta2a_permute, ta2a_permute_overlap, ta2a_unpermute, ta2a_unpermute_overlap)
+    if (E // world) * rpn > 63 and branch == "general":
+        pytest.skip("bitmask branch needs <= 63 slots per node")
+    announce("overlap seam", (world, rpn, E, T, k, M, H), branch, pack_mode)
+    monkeypatch.setenv("TERRACE_TA2A_PACK", pack_mode)
+    ta2a_pack.reset()
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    slots = (E // world) * rpn
+    gm = M if branch == "quota" else None
+    e = equal_quota_routing(T, k, E, world // rpn, M, 91, sort_rows=True)
+    g = torch.Generator().manual_seed(T + H)
+    x, probs, G = torch.randn(T, H, generator=g), torch.rand(T, E, generator=g), torch.randn(T, H, generator=g)
+    rm = torch.zeros(T, E, dtype=torch.bool)
+    rm[torch.arange(T)[:, None], torch.from_numpy(e)] = True
+    geom = dict(world=world, rank=0, rpn=rpn, n_experts=E, groups_m=gm)
+    # ---- the plain halves: values and gradients to match
+    xp, pp = x.to(DEV).requires_grad_(), probs.to(DEV).requires_grad_()
+    permuted0, tpe0, pprobs0, st0 = ta2a_permute(xp, pp, rm.to(DEV), **geom)
+    scale = ((torch.repeat_interleave(torch.arange(slots, device=DEV), tpe0) + 1).float() / slots)[:, None]
+    y0 = ta2a_unpermute(permuted0 * scale * pprobs0[:, None], st0, xp)
+    (y0 * G.to(DEV)).sum().backward()
+    # ---- the overlap halves
+    xd, pd = x.to(DEV).requires_grad_(), probs.to(DEV).requires_grad_()
+    save, calls = [], []
+    permuted, tpe, pprobs, shared, st = ta2a_permute_overlap(
+        xd, pd, rm.to(DEV), save_tensors=save, run_shared_experts=lambda: calls.append(len(save)) or "shared", **geom)
+    assert shared == "shared" and calls == [2], "the shared-expert callback runs once, after Hop A is launched"
+    assert len(save) == 7 and save[2] is None
+    assert save[4] is permuted and save[6] is pprobs
+    assert save[3].is_leaf and save[3].requires_grad and save[5].is_leaf and save[5].requires_grad
+    assert save[0].requires_grad and save[1].requires_grad and not save[0].is_leaf and not save[1].is_leaf
+    assert save[0].shape == save[3].shape and save[1].shape == save[5].shape
+    assert torch.equal(permuted.detach(), permuted0.detach()) and torch.equal(pprobs.detach(), pprobs0.detach())
+    assert torch.equal(tpe, tpe0) and torch.equal(save[3].detach(), save[0].detach())
+    # the expert layer is a segment of its own, on detached leaves
+    p_in, pp_in = permuted.detach().requires_grad_(), pprobs.detach().requires_grad_()
+    eo = p_in * scale * pp_in[:, None]
+    y = ta2a_unpermute_overlap(eo.detach(), st, save, out_shape=(T, H))
+    assert len(save) == 10 and save[7].is_leaf and save[9].is_leaf and not save[8].is_leaf
+    assert torch.equal(y.detach(), y0.detach())
+    # ---- the backward, replayed by fixed position
+    y.backward(G.to(DEV))
+    save[8].backward(save[9].grad)                 # Hop A's reverse is loop-back: the leaf's gradient is the row's
+    eo.backward(save[7].grad)
+    save[4].backward(p_in.grad)
+    save[6].backward(pp_in.grad)
+    save[0].backward(save[3].grad)
+    save[1].backward(save[5].grad)
+    for name, got, want in (("hidden.grad", xd.grad, xp.grad), ("probs.grad", pd.grad, pp.grad)):
+        assert got is not None, f"{name} is missing"
+        err = (got - want).abs().max().item()
+        assert err <= 1e-5 * max(want.abs().max().item(), 1.0), f"{name} differs by {err}"
+    ta2a_pack.reset()
+
+
+def test_overlap_seam_switches(monkeypatch):
+    from terrace import ta2a_dispatch as td
+    monkeypatch.delenv("TERRACE_TA2A", raising=False)
+    assert not td.ta2a_enabled(128, 8)
+    monkeypatch.setenv("TERRACE_TA2A", "1")
+    assert td.ta2a_enabled(128, 8) and td.ta2a_enabled(16, 8) and not td.ta2a_enabled(8, 8)
+    td.reset_shared_overlap()
+    monkeypatch.setenv("TERRACE_SHARED_OVERLAP", "0")
+    assert not td.shared_overlap_enabled()
+    td.reset_shared_overlap()
+    monkeypatch.delenv("TERRACE_SHARED_OVERLAP")
+    assert td.shared_overlap_enabled()
+    # with the switch off the callback runs after every dispatch exchange: all seven seats are filled by then
+    from terrace import ta2a
+    ta2a._VERIFIED.clear(), ta2a._VERIFY_COUNT.clear()
+    monkeypatch.setenv("TERRACE_SHARED_OVERLAP", "0")
+    td.reset_shared_overlap()
+    e = equal_quota_routing(8, 4, 8, 2, 2, 5, sort_rows=True)
+    rm = torch.zeros(8, 8, dtype=torch.bool)
+    rm[torch.arange(8)[:, None], torch.from_numpy(e)] = True
+    save, calls = [], []
+    td.ta2a_permute_overlap(torch.randn(8, 6, device=DEV), torch.rand(8, 8, device=DEV), rm.to(DEV), world=4, rank=0,
+                            rpn=2, n_experts=8, groups_m=2, save_tensors=save,
+                            run_shared_experts=lambda: calls.append(len(save)))
+    assert calls == [7]
+    td.reset_shared_overlap()

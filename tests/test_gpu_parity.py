@@ -764,7 +764,7 @@ def test_alias_tripwire_fires_on_a_view():
     from terrace import ta2a_pack as pk
     buf = torch.zeros(4, 8, dtype=torch.int64, device=DEV)
     view = buf[:, :2]
-    with pytest.raises(RuntimeError, match="shared storage"):
+    with pytest.raises(RuntimeError, match="shares storage"):
         pk.assert_not_aliased(buf, view)
     pk.assert_not_aliased(buf, view.clone())
     pk.assert_not_aliased(buf, torch.zeros(0, dtype=torch.int64, device=DEV), None)
