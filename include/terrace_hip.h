@@ -310,10 +310,10 @@ TERRACE_API int terrace_regroup_wire(const void *node_rx, const int64_t *my_meta
 /* ---- the general (data-dependent fan-out) branch and the seam's entry helper ---- */
 
 /* plan_ta2a without groups_m (terrace/ta2a.py:70-275, general branch): one send row per occupied
- * (node, token) pair in (node asc, token asc) order, for n_nodes <= 64.  u_src / u_node must hold
+ * (node, token) pair in (node asc, token asc) order, for any n_nodes up to 2048.  u_src / u_node must hold
  * T*min(k, n_nodes) entries; the number actually written is sum(counts), which the caller reads
  * back (the reference pays the same synchronisation at terrace/ta2a.py:148). */
-TERRACE_API size_t terrace_plan_general_workspace(int64_t T, int n_nodes);
+TERRACE_API size_t terrace_plan_general_workspace(int64_t T, int k, int n_nodes);
 TERRACE_API int terrace_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn,
                                      int64_t *u_src, int64_t *u_node, int64_t *counts, int64_t *inverse,
                                      int32_t *status, void *workspace, size_t workspace_bytes,

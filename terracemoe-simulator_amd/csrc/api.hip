@@ -59,7 +59,7 @@ int run_k2_pack(const void *hidden, const int64_t *expert_idx, const void *gates
 int run_pack_quota_wire(const int64_t *expert_idx, const void *gates, const int64_t *inverse, int64_t T, int k,
                         int gate_bytes, int64_t n_rows, int slots, int quota, int64_t *slot_tab, void *gate_tab,
                         int32_t *status, hipStream_t s);
-size_t plan_general_workspace(int64_t T, int n_nodes);
+size_t plan_general_workspace(int64_t T, int k, int n_nodes);
 int run_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn, int64_t *u_src,
                      int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status, void *ws, size_t ws_bytes,
                      hipStream_t s);
@@ -339,7 +339,9 @@ int terrace_unpack_planes(const void *packed, int64_t row_bytes, int64_t n_rows,
     return launch_unpack_planes(packed, row_bytes, n_rows, a, a_bytes, b, b_bytes, c, c_bytes, (hipStream_t)stream);
 }
 
-size_t terrace_plan_general_workspace(int64_t T, int n_nodes) { return plan_general_workspace(T, n_nodes); }
+size_t terrace_plan_general_workspace(int64_t T, int k, int n_nodes) {
+    return plan_general_workspace(T, k, n_nodes);
+}
 
 int terrace_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int n_experts, int rpn,
                          int64_t *u_src, int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status,

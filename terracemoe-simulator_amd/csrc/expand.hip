@@ -82,7 +82,15 @@ __global__ __launch_bounds__(kBlock) void plan_place_kernel(const int64_t *__res
     }
 }
 
-size_t plan_general_workspace(int64_t T, int n_nodes) {
+size_t plan_wide_workspace(int64_t T, int k, int n_nodes);
+int run_plan_wide(const int64_t *expert_idx, int64_t T, int k, int slots, int n_nodes, int n_experts, int64_t *u_src,
+                  int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status, void *ws, size_t ws_bytes,
+                  hipStream_t s);
+
+// Up to 64 nodes a token's node set is one mask word and a lane handles a token; beyond, the (token, column)
+// item sort of sort.hip takes over.
+size_t plan_general_workspace(int64_t T, int k, int n_nodes) {
+    if (n_nodes > 64) return plan_wide_workspace(T, k, n_nodes);
     Units u{T, 1, (int)((T + 63) / 64 > 0 ? (T + 63) / 64 : 1), n_nodes};
     return units_table_bytes(u);
 }
@@ -93,7 +101,11 @@ int run_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int
     if (T < 0 || k <= 0 || world <= 0 || rpn <= 0 || n_experts <= 0 || world % rpn || n_experts % world || !counts)
         return TERRACE_EINVAL;
     const int n_nodes = world / rpn, slots = (n_experts / world) * rpn;
-    if (n_nodes > 64 || T * (int64_t)k >= (int64_t)1 << 31) return TERRACE_EINVAL;
+    if (T * (int64_t)k >= (int64_t)1 << 31) return TERRACE_EINVAL;
+    if (T > 0 && (!expert_idx || !u_src || !u_node || !inverse)) return TERRACE_EINVAL;
+    if (n_nodes > 64)
+        return run_plan_wide(expert_idx, T, k, slots, n_nodes, n_experts, u_src, u_node, counts, inverse, status, ws,
+                             ws_bytes, s);
     Units u{T, 1, (int)((T + 63) / 64 > 0 ? (T + 63) / 64 : 1), n_nodes};
     if (!ws || ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     int32_t *table = (int32_t *)ws;

@@ -203,6 +203,65 @@ struct KeyRun {              // item = t*M + m  ->  node of the m-th run of toke
     }
 };
 
+// An emitter that loads nothing of its own.
+struct NoPre {};
+
+// General plan with more nodes than one mask word holds: item = (token, column); an item counts only when it is the
+// first column of its token on its node, so each occupied (token, node) pair is one item, keyed by the node.
+// Items enumerate token-major, hence pairs of one node come out in ascending token order
+// (terrace/ta2a.py:205-253: the (node ascending, token ascending) rows of the general branch).
+struct KeyFirstOnNode {
+    const int64_t *expert_idx;
+    int k, slots, n_nodes, n_experts;
+    __device__ __forceinline__ int64_t fetch(int64_t item) const { return expert_idx[item]; }
+    // -1: not an item (a later column on a node the token already touches, or an id out of range)
+    __device__ __forceinline__ int bucket(int64_t item, int64_t e, bool *bad) const {
+        if (e < 0 || e >= n_experts) {
+            *bad = true;
+            return -1;
+        }
+        const int node = (int)(e / slots);
+        const int64_t t = item / k;
+        const int j = (int)(item - t * k);
+        const int64_t *row = expert_idx + t * k;
+        for (int i = 0; i < j; ++i) {
+            const int64_t o = row[i];
+            if (o >= 0 && o < n_experts && (int)(o / slots) == node) return -1;
+        }
+        return node;
+    }
+};
+
+struct EmitPlanWide {
+    const int64_t *expert_idx;
+    int k, slots, n_experts;
+    int64_t *u_src, *u_node, *inverse;
+    static constexpr bool kTallies = false;
+    typedef NoPre Pre;
+    __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
+    __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, int64_t, Pre, const int32_t *,
+                                              int *) const {
+        const int64_t t = item / k;
+        const int j = (int)(item - t * k);
+        u_src[row] = t;
+        u_node[row] = node;
+        const int64_t *ids = expert_idx + t * k;
+        for (int i = j; i < k; ++i) {                  // every column of the token on this node rides this row
+            const int64_t o = ids[i];
+            if (o >= 0 && o < n_experts && (int)(o / slots) == node) inverse[t * k + i] = row;
+        }
+        return 0;
+    }
+};
+
+__global__ __launch_bounds__(kBlock) void mark_bad_ids_kernel(const int64_t *__restrict__ expert_idx, int64_t n,
+                                                              int n_experts, int64_t *__restrict__ inverse) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const int64_t e = expert_idx[i];
+    if (e < 0 || e >= n_experts) inverse[i] = -1;
+}
+
 // Lanes of the wave that hold the same key as this one (valid lanes only): one ballot per key bit
 // instead of one pass per distinct key.
 __device__ __forceinline__ uint64_t same_key_lanes(int key, bool valid, int key_bits) {
@@ -537,8 +596,6 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
 // ---------------------------------------------------------------------------------------------
 // An emitter's fetch(item) loads what it needs beyond the key (issued with the key loads); its call
 // operator gets the key's fetched value and that Pre back and only computes and stores.
-struct NoPre {};
-
 struct EmitOrder {           // plain stable argsort: order[dest] = item
     int64_t *order;
     static constexpr bool kTallies = false;
@@ -1042,6 +1099,27 @@ int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *or
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyAffine key{keyp, 0, 1, n_buckets};
     return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, hist, nullptr, nullptr, status, true, s);
+}
+
+// ---- general plan beyond 64 nodes ----------------------------------------------------------------
+size_t plan_wide_workspace(int64_t T, int k, int n_nodes) {
+    if (T <= 0 || k <= 0 || n_nodes <= 0 || n_nodes > kMaxBuckets) return 256;
+    return units_table_bytes(make_units(T * k, n_nodes));
+}
+
+int run_plan_wide(const int64_t *expert_idx, int64_t T, int k, int slots, int n_nodes, int n_experts, int64_t *u_src,
+                  int64_t *u_node, int64_t *counts, int64_t *inverse, int32_t *status, void *ws, size_t ws_bytes,
+                  hipStream_t s) {
+    if (n_nodes > kMaxBuckets) return TERRACE_EINVAL;
+    if (T == 0) return empty_outputs(counts, nullptr, nullptr, n_nodes, status, s);
+    const Units u = make_units(T * k, n_nodes);
+    if (!ws || ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
+    KeyFirstOnNode key{expert_idx, k, slots, n_nodes, n_experts};
+    EmitPlanWide emit{expert_idx, k, slots, n_experts, u_src, u_node, inverse};
+    int rc = run_sort(key, emit, u, (int32_t *)ws, counts, nullptr, nullptr, status, true, s);
+    if (rc != TERRACE_OK) return rc;
+    mark_bad_ids_kernel<<<(int)((T * k + kBlock - 1) / kBlock), kBlock, 0, s>>>(expert_idx, T * k, n_experts, inverse);
+    return check_launch();
 }
 
 // ---- Hop-B arrival ----------------------------------------------------------------------------

@@ -67,7 +67,7 @@ SIGNATURES = {
     "terrace_k2_pack_move": (_I, [_P, _L, _L, _I, _I, _I, _P, _P, _Z, _P]),
     "terrace_k1_arrival_move": (_I, [_P, _L, _L, _I, _I, _P, _P, _Z, _P]),
     "terrace_regroup_move": (_I, [_P, _L, _L, _I, _L, _P, _P, _Z, _P]),
-    "terrace_plan_general_workspace": (_Z, [_L, _I]),
+    "terrace_plan_general_workspace": (_Z, [_L, _I, _I]),
     "terrace_plan_general": (_I, [_P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_build_mask": (_I, [_P, _P, _L, _I, _L, _P, _P, _P]),
     "terrace_scatter_elems": (_I, [_P, _I, _P, _P, _I, _L, _L, _I, _P, _P]),

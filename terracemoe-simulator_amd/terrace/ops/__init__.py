@@ -748,15 +748,13 @@ def plan_general(expert_idx, world, n_experts, rpn):
     dev = expert_idx.device
     T, k = expert_idx.shape
     n_nodes = world // rpn
-    if n_nodes > 64:
-        raise ValueError(f"plan_ta2a: the general plan handles at most 64 destination nodes, got {n_nodes}")
     cap = T * min(k, n_nodes)
     u_src = torch.empty((cap,), dtype=torch.int64, device=dev)
     u_node = torch.empty((cap,), dtype=torch.int64, device=dev)
     inverse = torch.empty((T * k,), dtype=torch.int64, device=dev)
     counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
     st = _hip.new_status(dev)
-    ws = _hip.workspace(_hip.query("terrace_plan_general_workspace", T, n_nodes), dev)
+    ws = _hip.workspace(_hip.query("terrace_plan_general_workspace", T, k, n_nodes), dev)
     _hip.call("terrace_plan_general", _hip.ptr(expert_idx), T, k, world, n_experts, rpn, _hip.ptr(u_src),
               _hip.ptr(u_node), _hip.ptr(counts), _hip.ptr(inverse), _hip.ptr(st), _hip.ptr(ws), ws.numel(),
               _hip.stream(dev))

@@ -28,7 +28,11 @@ def _free_routing(T, k, E, seed):
 
 
 GEOMS = [(4, 2, 8, 9, 3), (32, 8, 64, 40, 4), (16, 8, 32, 17, 5), (64, 8, 128, 333, 6), (8, 4, 8, 1, 2),
-         (64, 8, 256, 3000, 8), (512, 8, 512, 700, 12)]
+         (64, 8, 256, 3000, 8), (512, 8, 512, 700, 12),
+         # more than 64 destination nodes (the reference's general plan has no node bound, terrace/ta2a.py:205-253):
+         # 80, 128 and 300 nodes, several experts of a token on one node, a single token, many units
+         (640, 8, 1280, 500, 8), (1024, 8, 1024, 257, 12), (600, 2, 2400, 90, 16), (160, 2, 160, 1, 4),
+         (1040, 8, 4160, 20000, 6)]
 
 
 @pytest.mark.parametrize("world,rpn,E,T,k", GEOMS)
@@ -74,6 +78,11 @@ def test_general_plan_errors_and_empty():
                         2, 2, 128, 2)
     u_src, u_node, counts, inverse = ta2a.plan_ta2a(torch.zeros((0, 4), dtype=torch.int64, device=DEV), 4, 8, 2)
     assert u_src.numel() == 0 and inverse.numel() == 0 and counts.tolist() == [0, 0]
+    # the same on the wide-node form
+    with pytest.raises(ValueError, match="out of range"):
+        ta2a.plan_ta2a(torch.tensor([[0, 2, 999]] * 5, device=DEV), 400, 800, 4)
+    u_src, u_node, counts, inverse = ta2a.plan_ta2a(torch.zeros((0, 4), dtype=torch.int64, device=DEV), 400, 800, 4)
+    assert u_src.numel() == 0 and inverse.numel() == 0 and counts.tolist() == [0] * 100
 
 
 @pytest.mark.parametrize("slots", [1, 5, 16, 24, 25, 40, 63])
