@@ -25,6 +25,7 @@ from), and the CPU baseline: the path as a chain of torch CPU operators on the h
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import statistics
@@ -71,14 +72,23 @@ def event_ms(fn, reps, torch):
 
 
 def wall_ms(fn, steps, warmup, torch):
+    """W untimed steps, then exactly K timed ones between two device synchronisations.  The interpreter's cyclic
+    garbage collector is held off for the timed region, as ``timeit`` does: a full collection pass stalls the host
+    for tens of milliseconds, which is this process's bookkeeping and not a cost of the path."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) * 1e3 / steps
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 def measured_traffic(workload, kernel, digest):

@@ -97,7 +97,9 @@ TERRACE_API int terrace_t_route(const float *affinity, const float *bias, const 
                     int64_t *expert_idx, void *gates, int64_t *group_idx, terrace_stream_t stream);
 
 /* expert_load (terrace/routing.py:112-113) and fixed_hist (terrace/ta2a_fwd.py:299-321):
- * out[b] = #{i : idx[i] == b}; out is int64 [n_buckets] or, with as_float != 0, float32. */
+ * out[b] = #{i : idx[i] == b}; out is int64 [n_buckets] or, with as_float != 0, float32.  An index outside
+ * [0, n_buckets) is counted nowhere and sets TERRACE_FAULT_ID_RANGE in the status block (the reference's bincount
+ * would grow its result and its scatter_add_ would fail on the spot; a kernel can do neither). */
 TERRACE_API size_t terrace_hist_workspace(int64_t n, int n_buckets);
 TERRACE_API int terrace_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_float, int32_t *status,
                  void *workspace, size_t workspace_bytes, terrace_stream_t stream);
@@ -240,7 +242,9 @@ TERRACE_API int terrace_index_chain2(const int64_t *outer, int64_t n_outer, cons
  * accumulated in fp32 as acc = fl(acc + fl(w*x)) for j = 0..fan-1, rounded once to out_dtype.
  * src rows are src_dtype (F32, BF16, F16 or FP8_E4M3_B128 with `hidden` elements per row),
  * weights [n_out,fan] are w_dtype (F32, BF16, F16) or NULL (all ones), idx is [n_out,fan] i64,
- * out is [n_out,hidden] of out_dtype (F32, BF16 or F16). */
+ * out is [n_out,hidden] of out_dtype (F32, BF16 or F16).  The weights plane must be 4-byte aligned; a 16-bit
+ * weight is read as the aligned 32-bit word that holds it, so when n_out*fan is odd the last read covers the two
+ * bytes after the plane (the same aligned word: never another page, never used). */
 TERRACE_API int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
                     int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
                     terrace_stream_t stream);

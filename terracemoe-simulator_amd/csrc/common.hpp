@@ -29,9 +29,8 @@ __device__ __forceinline__ int read_lane(int v, int src_lane) {
     return __builtin_amdgcn_readlane(v, src_lane);
 }
 
-// Butterfly exchange with lane ^ mask.  Distances 1 and 2 use DPP quad permutes, 4 and 8 the
-// DPP row mirrors (valid whenever the lanes below that distance already agree or the
-// reduction is symmetric -- see each call site), 16 a ds_swizzle, 32 a ds_bpermute.
+// Butterfly exchange with lane ^ mask.  Distances 1 and 2 use DPP quad permutes, 4, 8 and 16 a
+// ds_swizzle in bit mode (and-mask 0x1F, xor-mask the distance), 32 a ds_bpermute.
 template <int MASK>
 __device__ __forceinline__ int xchg_xor_i(int v) {
     if constexpr (MASK == 1) {

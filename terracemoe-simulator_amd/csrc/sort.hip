@@ -83,6 +83,9 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
     // r*width + i is then at plane[r*pitch + i]
     int width = 1;
     int64_t pitch = 1;
+    // a value outside [sub, sub + n_buckets*div): false = contained in bucket 0 (a sort must place every item),
+    // true = not an item at all (a histogram must not count it); reported as TERRACE_FAULT_ID_RANGE either way
+    bool drop_bad = false;
     // fetch() is one unconditional load (the kernels issue every chunk's fetch before any key is
     // used, so the loads overlap); bucket() turns the fetched value into the key
     __device__ __forceinline__ int64_t fetch(int64_t item) const {
@@ -94,7 +97,7 @@ struct KeyAffine {           // bucket = (plane[item] - sub) / div
         const int64_t v = fetched - sub;
         const bool out = v < 0 || v >= (int64_t)n_buckets * div;
         if (out) *bad = true;
-        return out ? 0 : (int)((uint32_t)v / (uint32_t)div);
+        return out ? (drop_bad ? -1 : 0) : (int)((uint32_t)v / (uint32_t)div);
     }
 };
 
@@ -1085,7 +1088,7 @@ int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_flo
     if (!idx || !ws) return TERRACE_EINVAL;
     const Units u = make_units(n, n_buckets);
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
-    KeyAffine key{idx, 0, 1, n_buckets};
+    KeyAffine key{idx, 0, 1, n_buckets, 1, 1, true};
     // the rank pass runs only to report out-of-range ids
     return run_sort(key, EmitNothing{}, u, (int32_t *)ws, h, hf, nullptr, status, status != nullptr, s);
 }

@@ -93,7 +93,9 @@ def t_route(affinity: torch.Tensor, bias: torch.Tensor, cfg: TRouteConfig, mode:
 
 
 def expert_load(expert_idx: torch.Tensor, n_experts: int) -> torch.Tensor:
-    """Per-expert pick counts as float32 (``bincount(...).float()`` in the reference)."""
+    """Per-expert pick counts as float32 (``bincount(...).float()`` in the reference).  An id outside
+    ``[0, n_experts)`` is counted nowhere; the status words that report it are not read back here (no host sync on
+    this path): use ``terrace.ops.hist`` to get them."""
     out, _ = _ops.hist(expert_idx, n_experts, as_float=True)
     return out
 

@@ -11,16 +11,17 @@ the balanced size) and every expert slot of the node treated as local.
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass
 
 import torch
 
-from . import _hip
+from . import _hip, _planes
 from . import ops as _ops
 
 
 def fixed_hist(idx: torch.Tensor, n_buckets: int) -> torch.Tensor:
-    """Fixed-length int64 histogram (``bincount(idx, minlength=n_buckets)`` without the sync)."""
+    """Fixed-length int64 histogram (``bincount(idx, minlength=n_buckets)`` without the sync).  An index outside
+    ``[0, n_buckets)`` is counted nowhere (the reference's ``scatter_add_`` would fail on it); ``terrace.ops.hist``
+    also returns the status words that report it."""
     out, _ = _ops.hist(idx, n_buckets)
     return out
 
@@ -102,43 +103,18 @@ def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: i
     return payload, mask, gate_rows, u_src, node_counts, inverse, u_node
 
 
-@dataclass
-class LoopbackState:
-    """What the combine needs from the dispatch, and what a caller may want to inspect."""
-    payload: torch.Tensor
-    mask: torch.Tensor
-    gate_rows: torch.Tensor
-    u_src: torch.Tensor
-    node_counts: torch.Tensor
-    extras: dict
-    send_buf: torch.Tensor
-    gate_pairs: torch.Tensor
-    r_idx: torch.Tensor
-    slot_idx: torch.Tensor
-    i_send: torch.Tensor
-    pair_pos: torch.Tensor
-    permuted: torch.Tensor
-    tokens_per_expert: torch.Tensor
-    place: torch.Tensor            # [P] where each arrival row sits in the expert-order buffer, -1 = dropped
-    kept: torch.Tensor | None
-    capacity: int | None
+class LoopbackState(_planes.LazyFields):
+    """What the combine needs from the dispatch, and what a caller may want to inspect: ``payload``, ``mask``,
+    ``gate_rows``, ``u_src``, ``node_counts``, ``extras`` (dict), ``send_buf``, ``gate_pairs``, ``r_idx``,
+    ``slot_idx``, ``i_send``, ``pair_pos``, ``permuted``, ``tokens_per_expert``, ``place`` ([P]: where each arrival row
+    sits in the expert-order buffer, -1 = dropped), ``kept`` (None when drop-less) and ``capacity``.  The small planes
+    live in one allocation and become tensors when first read."""
 
 
-@dataclass
-class OnePassState:
-    """Dispatch state when Hop B ran as one pass (:func:`loopback_dispatch_onepass`): no arrival-order send
-    buffer exists, so ``place`` is indexed by Hop-A pair ``row*quota + i`` directly."""
-    payload: torch.Tensor
-    mask: torch.Tensor
-    gate_rows: torch.Tensor
-    u_src: torch.Tensor
-    node_counts: torch.Tensor
-    extras: dict
-    permuted: torch.Tensor
-    tokens_per_expert: torch.Tensor
-    place: torch.Tensor            # [P] by pair; -1 = dropped
-    kept: torch.Tensor | None
-    capacity: int | None
+class OnePassState(_planes.LazyFields):
+    """Dispatch state when Hop B ran as one pass (:func:`loopback_dispatch_onepass`): ``payload``, ``mask``,
+    ``gate_rows``, ``u_src``, ``node_counts``, ``extras``, ``permuted``, ``tokens_per_expert``, ``place``, ``kept``,
+    ``capacity``.  No arrival-order send buffer exists, so ``place`` is indexed by Hop-A pair ``row*quota + i``."""
 
 
 _INDEX_STREAMS: dict = {}
@@ -185,23 +161,7 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
     if overlap is None:
         overlap = os.environ.get("TERRACE_OVERLAP", "0") == "1"
     if not overlap or x.shape[0] == 0:
-        # the combine's [T, k] place table is filled on the way: every Hop-A pair carries the entry it answers
-        # (pair_src) through the arrival reorder, and the regroup writes the pair's place there
-        (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
-            x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True, combine_table=True)
-        carried = []
-        send_buf, gate_pairs, r_idx, slot_idx, i_send, pair_pos = _ops.k1_arrival_raw(
-            payload, mask, gate_rows, quota, epr, rpn, 0, want_pair_pos=True, tags=extras["pair_src"],
-            tags_out=carried)
-        if capacity is None:
-            permuted, order, tpe, place = _regroup_with_place(send_buf, slot_idx, slots, tags=carried[0],
-                                                              table=extras["where"])
-            kept = None
-        else:
-            permuted, place, kept, tpe, _kpe = _ops.regroup(send_buf, slot_idx, slots, 0, capacity,
-                                                            tags=carried[0], table=extras["where"])
-        return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
-                             slot_idx, i_send, pair_pos, permuted, tpe, place, kept, capacity)
+        return _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity, onepass=False)
 
     _ops._check_k2(x, expert_idx, gates, world, n_experts, rpn, groups_m)
     dev = x.device
@@ -230,8 +190,10 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
     permuted = _ops.regroup_move(send_buf, rg["workspace"], slots, capacity)
     rows.wait_event(chained)            # joins the index stream: nothing of it is in flight on return
     extras["where"] = where
-    return LoopbackState(payload, mask, gate_rows, u_src, node_counts, extras, send_buf, gate_pairs, r_idx,
-                         slot_idx, i_send, pair_pos, permuted, rg["tokens_per_expert"], place, rg["kept"], capacity)
+    return LoopbackState(None, (), payload=payload, mask=mask, gate_rows=gate_rows, u_src=u_src, node_counts=node_counts,
+                         extras=extras, send_buf=send_buf, gate_pairs=gate_pairs, r_idx=r_idx, slot_idx=slot_idx,
+                         i_send=i_send, pair_pos=pair_pos, permuted=permuted,
+                         tokens_per_expert=rg["tokens_per_expert"], place=place, kept=rg["kept"], capacity=capacity)
 
 
 def loopback_dispatch_onepass(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8, groups_m: int = 1,
@@ -240,15 +202,86 @@ def loopback_dispatch_onepass(x, expert_idx, gates, world: int, n_experts: int, 
     straight to the expert-order (capacity-padded) place of each of its pairs (``ops.hopb_scatter``).  Same
     ``permuted`` / ``tokens_per_expert`` as :func:`loopback_dispatch` and ``place == its place[its pair_pos]``;
     the arrival-order planes (send_buf, r_idx, slot_idx, i_send) are never formed."""
-    epr = n_experts // world
-    slots = epr * rpn
-    quota = expert_idx.shape[1] // groups_m
-    (payload, mask, gate_rows, u_src, node_counts), extras = _ops.k2_pack_raw(
-        x, expert_idx, gates, world, n_experts, rpn, groups_m, extras=True, combine_table=True)
-    hb = _ops.hopb_scatter(payload, mask, None, quota, slots, 0, capacity, tags=extras["pair_src"],
-                           table=extras["where"])
-    return OnePassState(payload, mask, gate_rows, u_src, node_counts, extras, hb["permuted"], hb["tokens_per_expert"],
-                        hb["place"], hb["kept"], capacity)
+    return _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity, onepass=True)
+
+
+_DISPATCH_LAYOUTS: dict = {}
+
+
+def _dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass):
+    """The slab arrangement of a dispatch's small planes (cached per geometry).  Names: state fields as they are,
+    ``x.<key>`` the entries of ``extras``, ``_<name>`` scratch nobody reads."""
+    key = (T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass)
+    lay = _DISPATCH_LAYOUTS.get(key)
+    if lay is not None:
+        return lay
+    S, P, quota = T * groups_m, T * k, k // groups_m
+    cap = -1 if capacity is None else int(capacity)
+    i64, i32, u8 = torch.int64, torch.int32, torch.uint8
+    planes = [("mask", (S, quota), i64), ("gate_rows", (S, quota), gdt), ("u_src", (S,), i64),
+              ("node_counts", (n_nodes,), i64), ("tokens_per_expert", (slots,), i64), ("place", (P,), i64),
+              ("kept", (P,) if capacity is not None else None, torch.bool),
+              ("x.u_node", (S,), i64), ("x.inverse", (P,), i64), ("x.node_offsets", (n_nodes,), i64),
+              ("x.pair_table", (T, k), i64), ("x.sort_order", (T, k), i64), ("x.token_rows", (T, groups_m), i64),
+              ("x.gate_sorted", (T, k), gdt), ("x.pair_src", (P,), i64), ("x.where", (T, k), i64),
+              ("x.status", (4,), i32), ("_kept_per_expert", (slots,), i64),
+              ("_ws_k2", (_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m),), u8)]
+    if onepass:
+        planes += [("_status_b", (4,), i32),
+                   ("_ws_b", (_hip.query("terrace_hopb_scatter_workspace", S, quota, slots),), u8)]
+    else:
+        planes += [("gate_pairs", (P,), gdt), ("r_idx", (P,), i64), ("slot_idx", (P,), i64), ("i_send", (rpn,), i64),
+                   ("pair_pos", (P,), i64), ("_carried", (P,), i64), ("_status_a", (4,), i32), ("_status_r", (4,), i32),
+                   ("_order", (P,) if capacity is None else None, i64),
+                   ("_ws_a", (_hip.query("terrace_k1_arrival_workspace", S, quota, rpn),), u8),
+                   ("_ws_r", (_hip.query("terrace_regroup_workspace", P, slots, cap),), u8)]
+    if len(_DISPATCH_LAYOUTS) > 64:
+        _DISPATCH_LAYOUTS.clear()
+    lay = _DISPATCH_LAYOUTS[key] = _planes.Layout(planes)
+    return lay
+
+
+def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity, onepass):
+    """Stages 2-4 through the C ABI with every small plane in one allocation (three library calls, or two with
+    Hop B as one pass).  The combine's [T, k] place table is filled on the way: every Hop-A pair carries the entry
+    it answers (pair_src) through the sorts, and the last one writes the pair's place there."""
+    _ops._require()
+    _hip.need_device(x, expert_idx, gates)
+    _ops._check_k2(x, expert_idx, gates, world, n_experts, rpn, groups_m)
+    x, expert_idx, gates = x.contiguous(), expert_idx.contiguous(), gates.contiguous()
+    dev = x.device
+    T, k = expert_idx.shape
+    H = x.shape[1]
+    epr, n_nodes = n_experts // world, world // rpn
+    slots, quota = epr * rpn, k // groups_m
+    S, P = T * groups_m, T * k
+    cap = -1 if capacity is None else int(capacity)
+    places = P if capacity is None else slots * cap
+    row_bytes, gb = H * x.element_size(), gates.element_size()
+    slab = _planes.Slab(_dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gates.dtype, onepass), dev)
+    payload = torch.empty((S, H), dtype=x.dtype, device=dev)
+    permuted = torch.empty((places, H), dtype=x.dtype, device=dev)
+    ptr, at, stream = _hip.ptr, slab.ptr, _hip.stream(dev)
+    _hip.call("terrace_k2_pack", ptr(x), ptr(expert_idx), ptr(gates), T, row_bytes, gb, k, world, n_experts, rpn,
+              groups_m, ptr(payload), at("mask"), at("gate_rows"), at("u_src"), at("node_counts"), at("x.u_node"),
+              at("x.inverse"), at("x.node_offsets"), at("x.pair_table"), at("x.sort_order"), at("x.token_rows"),
+              at("x.gate_sorted"), at("x.pair_src"), at("x.where"), at("x.status"), at("_ws_k2"), slab.nbytes("_ws_k2"),
+              stream)
+    extras = _planes.LazyDict(slab, "x.")
+    if onepass:
+        _hip.call("terrace_hopb_scatter", ptr(payload), at("mask"), None, S, row_bytes, gb, quota, 0, slots, cap,
+                  ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"), at("_kept_per_expert"),
+                  at("x.pair_src"), at("x.where"), P, at("_status_b"), at("_ws_b"), slab.nbytes("_ws_b"), stream)
+        return OnePassState(slab, ("kept",), payload=payload, permuted=permuted, extras=extras, capacity=capacity)
+    send_buf = torch.empty((P, H), dtype=x.dtype, device=dev)
+    _hip.call("terrace_k1_arrival", ptr(payload), at("mask"), at("gate_rows"), S, row_bytes, gb, quota, epr, rpn, 0,
+              ptr(send_buf), at("gate_pairs"), at("r_idx"), at("slot_idx"), at("i_send"), at("pair_pos"),
+              at("x.pair_src"), at("_carried"), at("_status_a"), at("_ws_a"), slab.nbytes("_ws_a"), stream)
+    _hip.call("terrace_regroup", ptr(send_buf), at("slot_idx"), None, P, row_bytes, gb, slots, 0, cap, ptr(permuted),
+              None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"), at("_kept_per_expert"),
+              at("_carried"), at("x.where"), P, at("_status_r"), at("_ws_r"), slab.nbytes("_ws_r"), stream)
+    return LoopbackState(slab, ("kept",), payload=payload, send_buf=send_buf, permuted=permuted, extras=extras,
+                         capacity=capacity)
 
 
 def _regroup_with_place(node_rx, my_slot, epr, my_local: int = 0, my_gate=None, tags=None, table=None):

@@ -247,6 +247,19 @@ def test_expert_load_and_hist_and_argsort():
         same(_stable_argsort_small(kd, nb), orc.stable_argsort_small(key, nb), "argsort")
     e = rng.integers(0, 64, (4096, 8)).astype(np.int64)
     same(terrace.expert_load(torch.from_numpy(e).to(DEV), 64), orc.expert_load(e, 64), "expert_load")
+    # an index outside the range is counted nowhere and reported, in the direct and in the scan-launch form
+    import terrace.ops as tops
+    from terrace import _hip
+    for n, nb in [(5000, 16), (40000, 1500)]:
+        key = rng.integers(0, nb, n).astype(np.int64)
+        bad = key.copy()
+        bad[[3, n // 2, n - 1]] = [-1, nb, 1 << 40]
+        out, st = tops.hist(torch.from_numpy(bad).to(DEV), nb)
+        want = np.bincount(np.delete(key, [3, n // 2, n - 1]), minlength=nb)
+        same(out, want.astype(np.int64), "hist with bad ids")
+        assert st.tolist()[0] & _hip.FAULT_ID_RANGE
+        _, st = tops.hist(torch.from_numpy(key).to(DEV), nb)
+        assert st.tolist()[0] == 0
 
 
 # ------------------------------------------------------------------------------- plan + pack
