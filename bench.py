@@ -58,17 +58,25 @@ def parse():
     return ap.parse_args()
 
 
-def event_ms(fn, reps, torch):
-    """Average milliseconds of fn() over reps launches, HIP events on the current stream."""
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+EVENT_BATCHES = 5
+
+
+def event_ms(fn, reps, torch, batches=EVENT_BATCHES):
+    """Milliseconds per launch of fn(): the median over `batches` batches of the average over `reps` back-to-back
+    launches, each batch between two HIP events on the current stream (a median so that one disturbed batch
+    does not move the figure)."""
     fn()
     torch.cuda.synchronize()
-    start.record()
-    for _ in range(reps):
-        fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / reps
+    per_batch = []
+    for _ in range(batches):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        stop.synchronize()
+        per_batch.append(start.elapsed_time(stop) / reps)
+    return statistics.median(per_batch)
 
 
 def wall_ms(fn, steps, warmup, torch):
@@ -491,6 +499,8 @@ def main():
         "arrival_chain_us_per_row": stages["arrival"]["us_per_row"],
         "onepass": r["onepass"],
         "stages": stages, "kernels": kern, "roofline": roofline,
+        "stage_and_kernel_timing": f"each alone on the launch stream between HIP events: median of {EVENT_BATCHES} "
+                                   f"batches of {max(args.steps, 5)} back-to-back launches",
         "library": os.path.relpath(st.lib, ROOT), "source_digest": digest,
     }
     if r["graph"] is not None:

@@ -88,6 +88,41 @@ def test_random_geometries_every_plane_matches_oracle(index):
     _check_every_plane(cfg)
 
 
+def _large_geometries(n, seed):
+    """Seeded geometries with many tokens and narrow rows: every choice the sorts make of their unit size and of
+    the way a workgroup finds its base (table re-derived per workgroup, or a scan launch) is met, at sizes the
+    oracle still finishes in a second."""
+    from terrace import configs
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        n_groups = int(rng.choice([1, 2, 4, 8, 16, 32, 64]))
+        rpn = int(rng.choice([1, 2, 4, 8]))
+        g = rpn * int(rng.integers(1, 9))
+        E = n_groups * g
+        M = int(rng.integers(1, min(n_groups, 6) + 1))
+        q = int(rng.integers(1, min(g, 6) + 1))
+        if E > 2048 or M * q > 24 or g > 63:
+            continue
+        fmt = str(rng.choice(["f32", "bf16", "fp8"]))
+        hidden = 128 * int(rng.integers(1, 3)) if fmt == "fp8" else int(rng.choice([8, 24, 64, 200, 128]))
+        T = int(rng.choice([1023, 1025, 4097, 9000, 16384, 30000, 65537, 100000]))
+        if T * M * q * hidden > 2e9:
+            continue
+        out.append(configs.PathConfig(
+            f"large{len(out)}", T, E, n_groups, M * q, M, rpn, hidden, fmt,
+            bias=str(rng.choice(["none", "normal", "zipf"])), softmax_gates=bool(rng.integers(0, 2)),
+            capacity_factor=[None, 0.5, 1.25][int(rng.integers(0, 3))], seed=int(rng.integers(1, 1 << 30))))
+    return out
+
+
+@pytest.mark.parametrize("index", range(10))
+def test_large_random_geometries_every_plane_matches_oracle(index):
+    cfg = _large_geometries(10, 20261126)[index]
+    announce("large random", cfg)
+    _check_every_plane(cfg)
+
+
 def _check_every_plane(cfg):
     from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, twolevel_combine
     from terrace import configs
