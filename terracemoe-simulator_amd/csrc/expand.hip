@@ -112,7 +112,9 @@ int run_plan_general(const int64_t *expert_idx, int64_t T, int k, int world, int
     const int blocks = (u.n_units + kWavesPerBlock - 1) / kWavesPerBlock;
     if (T > 0 && (!expert_idx || !u_src || !u_node || !inverse)) return TERRACE_EINVAL;
     plan_count_kernel<<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, u.n_units, table);
-    launch_scan(u, table, counts, nullptr, nullptr, status, s);
+    TableOut out;
+    out.hist_i64 = counts;
+    launch_scan(u, table, out, status, s);
     plan_place_kernel<<<blocks, kBlock, 0, s>>>(expert_idx, T, k, slots, n_nodes, n_experts, u.n_units, table, u_src,
                                                 u_node, inverse, status);
     return check_launch();
@@ -240,7 +242,9 @@ int run_expand_count(const int64_t *rmask, int64_t R, int slots, int64_t *n_pair
     }
     if (!rmask) return TERRACE_EINVAL;
     expand_count_kernel<<<(unsigned)((R + kBlock - 1) / kBlock), kBlock, 0, s>>>(rmask, R, slots, cnt);
-    launch_scan(u, cnt, n_pairs, nullptr, nullptr, nullptr, s);
+    TableOut pairs_out;
+    pairs_out.hist_i64 = n_pairs;
+    launch_scan(u, cnt, pairs_out, nullptr, s);
     return check_launch();
 }
 

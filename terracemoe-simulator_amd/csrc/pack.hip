@@ -192,8 +192,10 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     if (threadIdx.x < n_nodes) tab = table[(int64_t)threadIdx.x * u.n_units + unit];
     // ---- cursors of this unit: start[n] + earlier workgroups (+ s_tab: earlier units of the count workgroup) ----
     const int me = unit / u.wpb;
-    direct_block_base(u, table, me, unit == 0, (lds_i32 *)s_tot, (lds_i32 *)s_base, (lds_i32 *)s_start, node_counts,
-                      nullptr, node_offsets);
+    TableOut out;
+    out.hist_i64 = node_counts;
+    out.offsets_i64 = node_offsets;
+    direct_block_base(u, table, me, unit == 0, (lds_i32 *)s_tot, (lds_i32 *)s_base, (lds_i32 *)s_start, out);
     // ---- the token's ids, shared inside the group; ranks by (id, column) ----
     TokenView<LPT> tv;
     tv.build(v, has_col, col, tok_lane, slots, n_experts, M, quota);

@@ -349,11 +349,8 @@ __device__ __forceinline__ i32x4 load4_guarded(const int32_t *t, int64_t i, int6
     return v;
 }
 
-__global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table,
-                                                            int64_t *__restrict__ hist_i64,
-                                                            float *__restrict__ hist_f32,
-                                                            int64_t *__restrict__ offsets_i64,
-                                                            int32_t *__restrict__ status) {
+__global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__restrict__ table, TableOut out,
+        int32_t *__restrict__ status) {
     constexpr int kWaves = kScanThreads / kWave;
     __shared__ int32_t wave_tot[kWaves];
     __shared__ int32_t grand_total;
@@ -403,9 +400,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__
         start[b] = s0;
         if (b == u.n_buckets) break;
         const int32_t s1 = b + 1 < u.n_buckets ? table[(int64_t)(b + 1) * u.n_units] : grand_total;
-        if (hist_i64) hist_i64[b] = s1 - s0;
-        if (hist_f32) hist_f32[b] = (float)(s1 - s0);
-        if (offsets_i64) offsets_i64[b] = s0;
+        out.put(b, s1 - s0, s0);
     }
 }
 
@@ -415,11 +410,8 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(Units u, int32_t *__
 // all loads issued at once, and scans it there: one memory round trip in, one out.
 constexpr int kScanRegVecs = 16;                 // 16 x 256 entries per wave
 
-__global__ __launch_bounds__(kScanThreads) void scan_registers_kernel(Units u, int32_t *__restrict__ table,
-                                                                      int64_t *__restrict__ hist_i64,
-                                                                      float *__restrict__ hist_f32,
-                                                                      int64_t *__restrict__ offsets_i64,
-                                                                      int32_t *__restrict__ status) {
+__global__ __launch_bounds__(kScanThreads) void scan_registers_kernel(Units u, int32_t *__restrict__ table, TableOut out,
+        int32_t *__restrict__ status) {
     constexpr int kWaves = kScanThreads / kWave;
     __shared__ int32_t wave_tot[kWaves];
     __shared__ int32_t grand_total;
@@ -481,19 +473,16 @@ __global__ __launch_bounds__(kScanThreads) void scan_registers_kernel(Units u, i
         start[b] = s0;
         if (b == u.n_buckets) break;
         const int32_t s1 = b + 1 < u.n_buckets ? table[(int64_t)(b + 1) * u.n_units] : grand_total;
-        if (hist_i64) hist_i64[b] = s1 - s0;
-        if (hist_f32) hist_f32[b] = (float)(s1 - s0);
-        if (offsets_i64) offsets_i64[b] = s0;
+        out.put(b, s1 - s0, s0);
     }
 }
 
-void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
-                 int32_t *status, hipStream_t s) {
+void launch_scan(const Units &u, int32_t *table, const TableOut &out, int32_t *status, hipStream_t s) {
     const int64_t n = (int64_t)u.n_units * u.n_buckets;
     if (n <= (int64_t)kScanThreads * kScanRegVecs * 4)
-        scan_registers_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
+        scan_registers_kernel<<<1, kScanThreads, 0, s>>>(u, table, out, status);
     else
-        scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, hist_i64, hist_f32, offsets_i64, status);
+        scan_kernel<<<1, kScanThreads, 0, s>>>(u, table, out, status);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -501,10 +490,7 @@ void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_
 // ---------------------------------------------------------------------------------------------
 template <typename KeyFn, typename EmitFn, int CH>
 __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitFn emit, Units u,
-                                                             int32_t *__restrict__ table,
-                                                             int64_t *__restrict__ hist_i64,
-                                                             float *__restrict__ hist_f32,
-                                                             int64_t *__restrict__ offsets_i64,
+                                                             int32_t *__restrict__ table, TableOut out,
                                                              int32_t *__restrict__ status) {
     extern __shared__ int32_t lds[];
     const int lane = lane_id();
@@ -539,8 +525,7 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
         }
         lds_i32 *shared = (lds_i32 *)lds + u.wpb * u.n_buckets;          // tot, base, start
         lds_i32 *base = shared + u.n_buckets, *lstart = base + u.n_buckets;
-        direct_block_base(u, table, (int)blockIdx.x, blockIdx.x == 0, shared, base, lstart, hist_i64, hist_f32,
-                          offsets_i64);
+        direct_block_base(u, table, (int)blockIdx.x, blockIdx.x == 0, shared, base, lstart, out);
         if (!active) return;
 #pragma unroll
         for (int i = 0; i < kTabRegs; ++i) {
@@ -1047,8 +1032,8 @@ static size_t lds_rank(const Units &u) {
 }
 
 template <typename KeyFn, typename EmitFn>
-static int run_sort(const KeyFn &key, const EmitFn &emit, Units u, int32_t *table, int64_t *hist,
-                    float *hist_f, int64_t *offsets, int32_t *status, bool do_rank, hipStream_t s) {
+static int run_sort(const KeyFn &key, const EmitFn &emit, Units u, int32_t *table, const TableOut &out,
+                    int32_t *status, bool do_rank, hipStream_t s) {
     if (!do_rank && u.direct) {          // the histogram alone: the scan launch writes it, so take that path
         u.direct = 0;                    // (the table region of a direct layout is large enough for it)
         u.wpb = 4;
@@ -1059,11 +1044,11 @@ static int run_sort(const KeyFn &key, const EmitFn &emit, Units u, int32_t *tabl
     if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, threads, lc, s>>>(key, u, table, status);
     else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, threads, lc, s>>>(key, u, table, status);
     else count_kernel<KeyFn, 16><<<blocks, threads, lc, s>>>(key, u, table, status);
-    if (!u.direct) launch_scan(u, table, hist, hist_f, offsets, status, s);
+    if (!u.direct) launch_scan(u, table, out, status, s);
     if (do_rank) {
-        if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
-        else if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
-        else rank_kernel<KeyFn, EmitFn, 16><<<blocks, threads, lr, s>>>(key, emit, u, table, hist, hist_f, offsets, status);
+        if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, threads, lr, s>>>(key, emit, u, table, out, status);
+        else if (u.chunks == 4) rank_kernel<KeyFn, EmitFn, 4><<<blocks, threads, lr, s>>>(key, emit, u, table, out, status);
+        else rank_kernel<KeyFn, EmitFn, 16><<<blocks, threads, lr, s>>>(key, emit, u, table, out, status);
     }
     return check_launch();
 }
@@ -1090,7 +1075,10 @@ int run_hist(const int64_t *idx, int64_t n, int n_buckets, void *out, int as_flo
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyAffine key{idx, 0, 1, n_buckets, 1, 1, true};
     // the rank pass runs only to report out-of-range ids
-    return run_sort(key, EmitNothing{}, u, (int32_t *)ws, h, hf, nullptr, status, status != nullptr, s);
+    TableOut planes;
+    planes.hist_i64 = h;
+    planes.hist_f32 = hf;
+    return run_sort(key, EmitNothing{}, u, (int32_t *)ws, planes, status, status != nullptr, s);
 }
 
 int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *order, int64_t *hist, int32_t *status,
@@ -1101,7 +1089,9 @@ int run_argsort_small(const int64_t *keyp, int64_t n, int n_buckets, int64_t *or
     const Units u = make_units(n, n_buckets);
     if (ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyAffine key{keyp, 0, 1, n_buckets};
-    return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, hist, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = hist;
+    return run_sort(key, EmitOrder{order}, u, (int32_t *)ws, out, status, true, s);
 }
 
 // ---- general plan beyond 64 nodes ----------------------------------------------------------------
@@ -1119,7 +1109,9 @@ int run_plan_wide(const int64_t *expert_idx, int64_t T, int k, int slots, int n_
     if (!ws || ws_bytes < units_table_bytes(u)) return TERRACE_ENOSPC;
     KeyFirstOnNode key{expert_idx, k, slots, n_nodes, n_experts};
     EmitPlanWide emit{expert_idx, k, slots, n_experts, u_src, u_node, inverse};
-    int rc = run_sort(key, emit, u, (int32_t *)ws, counts, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = counts;
+    int rc = run_sort(key, emit, u, (int32_t *)ws, out, status, true, s);
     if (rc != TERRACE_OK) return rc;
     mark_bad_ids_kernel<<<(int)((T * k + kBlock - 1) / kBlock), kBlock, 0, s>>>(expert_idx, T * k, n_experts, inverse);
     return check_launch();
@@ -1153,7 +1145,9 @@ int run_k1_arrival(const void *rx, const int64_t *rslot, const void *rgate, int6
     KeyAffine key{rslot, 0, epr, rpn, quota, slot_pitch};
     EmitArrival emit{rslot, rgate, gate_bytes, quota, slot_pitch, gate_pitch, gate_pairs, r_idx, slot_idx, pair_pos,
                      pos32, meta, tags_out ? tags_in : nullptr, tags_in ? tags_out : nullptr};
-    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = i_send;
+    int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_scatter_rows<int32_t>(rx, send_buf, pos32, R, quota, row_bytes, P, s);
 }
@@ -1181,7 +1175,9 @@ int run_arrival_pairs(const void *rx, const int64_t *r_in, const int64_t *slot_i
     int32_t *src32 = (int32_t *)((char *)ws + table_bytes);
     KeyAffine key{slot_in, 0, epr, rpn};
     EmitPairs emit{r_in, slot_in, rgate, gate_bytes, gate_width, R, gate_pairs, r_idx, slot_idx, ordo, src32};
-    int rc = run_sort(key, emit, u, table, i_send, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = i_send;
+    int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK || !rx) return rc;
     return launch_gather_rows<int32_t>(rx, send_buf, src32, P, row_bytes, R, s);
 }
@@ -1253,18 +1249,16 @@ int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, in
     EmitHopB emit{rgate, gate_bytes, quota, (int64_t)quota, capacity, place, kept, pair_of_place,
                   rgate ? permuted_gate : nullptr, pos32, tagged ? tags_in : nullptr,
                   tagged ? place_by_tag : nullptr, n_tags};
-    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = tokens_per_expert;
+    if (capacity < 0) out.kept_i64 = kept_per_expert;          // nothing is dropped: the sort's own publication
+    int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *start = table + units_start_at(u);
     if (capacity >= 0) {
         // padding planes now; the padding rows with the row mover (they may be moved later, by the _move call)
         rc = launch_zero_pad(start, n_local, capacity, rx ? permuted : nullptr, rx ? row_bytes : 0,
                              rgate ? permuted_gate : nullptr, gate_bytes, pair_of_place, kept_per_expert, s);
-        if (rc != TERRACE_OK) return rc;
-    } else if (kept_per_expert) {
-        capacity_index_kernel<<<(n_local + kBlock - 1) / kBlock, kBlock, 0, s>>>(nullptr, start, n_local, INT64_MAX, 0,
-                                                                                nullptr, kept_per_expert);
-        rc = check_launch();
         if (rc != TERRACE_OK) return rc;
     }
     if (!rx) return rc;
@@ -1336,7 +1330,10 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     const bool tagged = tags_in && place_by_tag && n_tags > 0;
     EmitRegroup emit{capacity, order, dest, kept, order32, tagged ? tags_in : nullptr,
                      tagged ? place_by_tag : nullptr, n_tags};
-    int rc = run_sort(key, emit, u, table, tokens_per_expert, nullptr, nullptr, status, true, s);
+    TableOut out;
+    out.hist_i64 = tokens_per_expert;
+    if (capacity < 0) out.kept_i64 = kept_per_expert;          // nothing is dropped: the sort's own publication
+    int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK) return rc;
     const int32_t *src_of_place = order32;
     const int32_t *start = table + units_start_at(u);
@@ -1345,9 +1342,6 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
         capacity_index_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(order32, start, epr, capacity,
                                                                                  places, gidx, kept_per_expert);
         src_of_place = gidx;
-    } else if (kept_per_expert) {
-        capacity_index_kernel<<<(epr + kBlock - 1) / kBlock, kBlock, 0, s>>>(order32, start, epr, INT64_MAX, 0,
-                                                                            nullptr, kept_per_expert);
     }
     if (my_gate && places > 0) {
         const int grid = (int)((places + kBlock - 1) / kBlock);
@@ -1402,7 +1396,10 @@ static int run_k2_t(const void *hidden, const int64_t *expert_idx, const void *g
     EmitPack<KMAX> emit{expert_idx, gates, gate_bytes, k, groups_m, quota, slots, n_experts,
                         mask, u_src, u_node, inverse, pair_table, sort_order, token_rows, gate_rows, gate_sorted,
                         pos32, pair_src, combine_table, mask_pitch, gate_pitch, gate_pad};
-    int rc = run_sort(key, emit, u, table, node_counts, nullptr, node_offsets, status, true, s);
+    TableOut out;
+    out.hist_i64 = node_counts;
+    out.offsets_i64 = node_offsets;
+    int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK || !hidden) return rc;
     return launch_scatter_rows<int32_t>(hidden, payload, pos32, T, groups_m, row_bytes, T * groups_m, s);
 }

@@ -43,11 +43,26 @@ __host__ __device__ inline int64_t units_census_at(const Units &u) {
     return units_blocktot_at(u) + (int64_t)u.n_buckets * u.n_blocks;
 }
 
+// What the one workgroup of a sort that holds every bucket's total and offset publishes for the caller, each
+// plane optional: the histogram as int64 and / or float32, the exclusive offsets, and min(count, capacity).
+struct TableOut {
+    int64_t *hist_i64 = nullptr;
+    float *hist_f32 = nullptr;
+    int64_t *offsets_i64 = nullptr;
+    int64_t *kept_i64 = nullptr;
+    int64_t capacity = INT64_MAX;
+    __device__ __forceinline__ void put(int b, int32_t count, int32_t offset) const {
+        if (hist_i64) hist_i64[b] = count;
+        if (hist_f32) hist_f32[b] = (float)count;
+        if (offsets_i64) offsets_i64[b] = offset;
+        if (kept_i64) kept_i64[b] = count < capacity ? count : capacity;
+    }
+};
+
 // Scan path: exclusive prefix over the bucket-major count table table[b * n_units + unit], in place; also
 // start[b] (n_buckets + 1 int32 right after the table), the optional histogram / offsets planes
 // and a zeroed status block.
-void launch_scan(const Units &u, int32_t *table, int64_t *hist_i64, float *hist_f32, int64_t *offsets_i64,
-                 int32_t *status, hipStream_t s);
+void launch_scan(const Units &u, int32_t *table, const TableOut &out, int32_t *status, hipStream_t s);
 
 constexpr int kSortBlockMax = 1024;      // 16 waves: the widest count / rank workgroup
 
@@ -56,12 +71,10 @@ constexpr int kSortBlockMax = 1024;      // 16 waves: the widest count / rank wo
 //   start[b]  first place of bucket b (n_buckets + 1 entries, the last one the item total),
 //   base[b]   first place of the items of bucket b that count workgroup `me` holds,
 // using tot[n_buckets] as scratch; with `publish` it also writes start[] after the table and fills the caller's
-// histogram / offsets planes (exactly one workgroup of a launch does).  A unit's cursor is then
+// planes (`out`) (exactly one workgroup of a launch does).  A unit's cursor is then
 // base[b] + table[b * n_units + unit].
 __device__ __forceinline__ void direct_block_base(const Units &u, int32_t *__restrict__ table, int me, bool publish,
-                                                  lds_i32 *tot, lds_i32 *base, lds_i32 *start,
-                                                  int64_t *__restrict__ hist_i64, float *__restrict__ hist_f32,
-                                                  int64_t *__restrict__ offsets_i64) {
+                                                  lds_i32 *tot, lds_i32 *base, lds_i32 *start, const TableOut &out) {
     const int lane = lane_id(), w = wave_in_block(), nw = (int)(blockDim.x >> 6);
     const int32_t *blocktot = table + units_blocktot_at(u);
     for (int b = w; b < u.n_buckets; b += nw) {            // one wave per bucket: no two waves share a word
@@ -103,10 +116,7 @@ __device__ __forceinline__ void direct_block_base(const Units &u, int32_t *__res
             const int32_t s0 = start[b];
             start_out[b] = s0;
             if (b == u.n_buckets) break;
-            const int32_t c = tot[b];
-            if (hist_i64) hist_i64[b] = c;
-            if (hist_f32) hist_f32[b] = (float)c;
-            if (offsets_i64) offsets_i64[b] = s0;
+            out.put(b, tot[b], s0);
         }
     }
 }
