@@ -767,13 +767,26 @@ struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
     const int64_t *tags_in;  // [P] a caller's tag per row: place_by_tag[tags_in[p]] = place of row p (-1 dropped)
     int64_t *place_by_tag;
     int64_t n_tags;
+    const void *gate_in;     // drop-less layout only: the row's gate goes to its place from here; with a capacity
+    void *gate_out;          // the padded plane is gathered per place afterwards (its padding places are zeros)
+    int gate_bytes;
+    int64_t gate_pitch;
     static constexpr bool kTallies = false;
-    struct Pre { int64_t tag; };
-    __device__ __forceinline__ Pre fetch(int64_t p) const { return Pre{tags_in ? tags_in[p] : -1}; }
+    struct Pre { int64_t tag; uint32_t gate; };
+    __device__ __forceinline__ Pre fetch(int64_t p) const {
+        Pre pre{tags_in ? tags_in[p] : -1, 0u};
+        if (gate_in) pre.gate = gate_bytes == 4 ? ((const uint32_t *)gate_in)[p * gate_pitch]
+                                                : (uint32_t)((const uint16_t *)gate_in)[p * gate_pitch];
+        return pre;
+    }
     __device__ __forceinline__ int operator()(int64_t p, int key, int32_t dest, int64_t, Pre pre,
                                               const int32_t *start, int *) const {
         order32[dest] = (int32_t)p;
         if (order) order[dest] = p;
+        if (gate_in) {
+            if (gate_bytes == 4) ((uint32_t *)gate_out)[dest] = pre.gate;
+            else ((uint16_t *)gate_out)[dest] = (uint16_t)pre.gate;
+        }
         int64_t d = dest;
         bool keep = true;
         if (capacity >= 0) {
@@ -1328,8 +1341,10 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     int32_t *gidx = (int32_t *)((char *)order32 + align_up((size_t)P * sizeof(int32_t), 256));
     KeyAffine key{my_slot, (int64_t)my_local * epr, 1, epr, 1, slot_pitch};
     const bool tagged = tags_in && place_by_tag && n_tags > 0;
+    const bool gate_in_sort = my_gate && capacity < 0;
     EmitRegroup emit{capacity, order, dest, kept, order32, tagged ? tags_in : nullptr,
-                     tagged ? place_by_tag : nullptr, n_tags};
+                     tagged ? place_by_tag : nullptr, n_tags, gate_in_sort ? my_gate : nullptr,
+                     gate_in_sort ? permuted_gate : nullptr, gate_bytes, gate_pitch};
     TableOut out;
     out.hist_i64 = tokens_per_expert;
     if (capacity < 0) out.kept_i64 = kept_per_expert;          // nothing is dropped: the sort's own publication
@@ -1343,7 +1358,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
                                                                                  places, gidx, kept_per_expert);
         src_of_place = gidx;
     }
-    if (my_gate && places > 0) {
+    if (my_gate && places > 0 && !gate_in_sort) {
         const int grid = (int)((places + kBlock - 1) / kBlock);
         if (gate_bytes == 4)
             gather_elems_kernel<uint32_t><<<grid, kBlock, 0, s>>>((const uint32_t *)my_gate, src_of_place, places, gate_pitch, (uint32_t *)permuted_gate);
