@@ -205,3 +205,22 @@ def test_pack_mode_switch(monkeypatch):
     assert pk.pack_mode() == "off"
     lay = pk.HopALayout(2048, 3, 3, False, torch.bfloat16)
     assert lay.words == 516 and pk.HopASmallLayout(3, 3, False, torch.bfloat16).words == 4
+
+
+def test_traffic_file_is_what_bench_reads():
+    """profiles/traffic.json: a source digest and positive byte counts keyed "<config>:<kernel>"; bench.py hands
+    the roofline's `traffic` out of it only when the digest is the loaded library's, and None otherwise."""
+    import json
+    import bench
+    with open(bench.TRAFFIC_FILE) as f:
+        rec = json.load(f)
+    assert isinstance(rec["source_digest"], str) and len(rec["source_digest"]) == 16
+    per_launch = rec["bytes_per_launch"]
+    assert "c2:gather_rows_sliced_kernel(regroup)" in per_launch
+    for key, nbytes in per_launch.items():
+        config, kernel = key.split(":", 1)
+        assert config in ("c1", "c2", "c3", "c4", "c5") and kernel and isinstance(nbytes, int) and nbytes > 0
+    key = "c2:gather_rows_sliced_kernel(regroup)"
+    assert bench.measured_traffic("c2", "gather_rows_sliced_kernel(regroup)", rec["source_digest"]) == per_launch[key]
+    assert bench.measured_traffic("c2", "gather_rows_sliced_kernel(regroup)", "0" * 16) is None
+    assert bench.measured_traffic("c2", "no_such_kernel", rec["source_digest"]) is None
