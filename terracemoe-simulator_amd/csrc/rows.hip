@@ -327,8 +327,8 @@ __device__ __forceinline__ void store_chunk(void *out_row, int64_t first_elem, c
 // the weights -- is fetched first through addresses the compiler can prove uniform (scalar loads; 16-bit
 // weights are read as the aligned dword that holds them).  The batch's row loads are then issued back to
 // back with nothing between them that waits on memory, and only the accumulation that follows consumes
-// them in order.  Dead entries (idx < 0) load row 0 and are zeroed with selects: no branch splits the
-// batch.
+// them in order.  A dead entry (idx outside [0, n_src)) touches no memory: its load sits behind a branch that
+// is uniform over the wave (the ids are), which costs nothing measurable against a select around a dummy load.
 constexpr int kWNone = -1;
 
 template <int WD>
@@ -362,16 +362,19 @@ __device__ __forceinline__ void combine_batch(float *acc, const uint8_t *__restr
     float sc[B];
 #pragma unroll
     for (int jj = 0; jj < B; ++jj) {
-        const uint8_t *s = src + (row_in(from[jj], n_src) ? from[jj] : 0) * src_row_bytes;
-        raw[jj] = ld_stream((const u32x4 *)s + c);
-        if constexpr (SRC == TERRACE_FP8_E4M3_B128) sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
-        else sc[jj] = 1.0f;
+        raw[jj] = zero_of<u32x4>();
+        sc[jj] = SRC == TERRACE_FP8_E4M3_B128 ? 0.0f : 1.0f;
+        if (row_in(from[jj], n_src)) {                       // wave-uniform: a dead entry touches no memory at all
+            const uint8_t *s = src + from[jj] * src_row_bytes;
+            raw[jj] = ld_stream((const u32x4 *)s + c);
+            if constexpr (SRC == TERRACE_FP8_E4M3_B128) sc[jj] = *(const float *)(s + hidden + 4 * (c * N / 128));
+        }
     }
 #pragma unroll
     for (int jj = 0; jj < B; ++jj) {
         const bool live = row_in(from[jj], n_src);
-        const u32x4 r = live ? raw[jj] : zero_of<u32x4>();
-        const float scale = live ? sc[jj] : 0.0f, weight = live ? wj[jj] : 0.0f;
+        const u32x4 r = raw[jj];
+        const float scale = sc[jj], weight = live ? wj[jj] : 0.0f;
         float f[N];
         decode_chunk<SRC>(r, f);
 #pragma unroll
@@ -735,7 +738,7 @@ int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t 
     if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
     if (n_out * ((hidden + 1023) / 1024 + 1) > kMaxGridRows) return TERRACE_EINVAL;
     const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
-    if (n_src <= 0) {           // no source rows: every entry is dead and every sum empty (the kernels read row 0)
+    if (n_src <= 0) {           // no source rows: every entry is dead and every sum empty; no kernel needs to look
         zero_bytes_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)out, n_out * orb);
         return check_launch();
     }
