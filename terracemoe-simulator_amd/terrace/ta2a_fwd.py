@@ -190,6 +190,7 @@ def loopback_dispatch(x, expert_idx, gates, world: int, n_experts: int, rpn: int
     permuted = _ops.regroup_move(send_buf, rg["workspace"], slots, capacity)
     rows.wait_event(chained)            # joins the index stream: nothing of it is in flight on return
     extras["where"] = where
+    extras["kept_per_expert"] = rg["kept_per_expert"]
     return LoopbackState(None, (), payload=payload, mask=mask, gate_rows=gate_rows, u_src=u_src, node_counts=node_counts,
                          extras=extras, send_buf=send_buf, gate_pairs=gate_pairs, r_idx=r_idx, slot_idx=slot_idx,
                          i_send=i_send, pair_pos=pair_pos, permuted=permuted,
@@ -224,7 +225,7 @@ def _dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass
               ("x.u_node", (S,), i64), ("x.inverse", (P,), i64), ("x.node_offsets", (n_nodes,), i64),
               ("x.pair_table", (T, k), i64), ("x.sort_order", (T, k), i64), ("x.token_rows", (T, groups_m), i64),
               ("x.gate_sorted", (T, k), gdt), ("x.pair_src", (P,), i64), ("x.where", (T, k), i64),
-              ("x.status", (4,), i32), ("_kept_per_expert", (slots,), i64),
+              ("x.status", (4,), i32), ("x.kept_per_expert", (slots,), i64),
               ("_ws_k2", (_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m),), u8)]
     if onepass:
         planes += [("_status_b", (4,), i32),
@@ -270,7 +271,7 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
     extras = _planes.LazyDict(slab, "x.")
     if onepass:
         _hip.call("terrace_hopb_scatter", ptr(payload), at("mask"), None, S, row_bytes, gb, quota, 0, slots, cap,
-                  ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"), at("_kept_per_expert"),
+                  ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"), at("x.kept_per_expert"),
                   at("x.pair_src"), at("x.where"), P, at("_status_b"), at("_ws_b"), slab.nbytes("_ws_b"), stream)
         return OnePassState(slab, ("kept",), payload=payload, permuted=permuted, extras=extras, capacity=capacity)
     send_buf = torch.empty((P, H), dtype=x.dtype, device=dev)
@@ -278,7 +279,7 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
               ptr(send_buf), at("gate_pairs"), at("r_idx"), at("slot_idx"), at("i_send"), at("pair_pos"),
               at("x.pair_src"), at("_carried"), at("_status_a"), at("_ws_a"), slab.nbytes("_ws_a"), stream)
     _hip.call("terrace_regroup", ptr(send_buf), at("slot_idx"), None, P, row_bytes, gb, slots, 0, cap, ptr(permuted),
-              None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"), at("_kept_per_expert"),
+              None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"), at("x.kept_per_expert"),
               at("_carried"), at("x.where"), P, at("_status_r"), at("_ws_r"), slab.nbytes("_ws_r"), stream)
     return LoopbackState(slab, ("kept",), payload=payload, send_buf=send_buf, permuted=permuted, extras=extras,
                          capacity=capacity)

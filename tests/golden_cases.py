@@ -79,4 +79,13 @@ def oracle_planes(name) -> dict:
     w_sorted = np.take_along_axis(g_pay, sort_order, 1)
     wf = orc.decode_rows(w_sorted, "f32" if c["fmt"] == "f32" else "bf16")
     out["y"] = orc.combine(perm, where, wf, c["fmt"], "f32" if c["fmt"] == "f32" else "bf16", hidden=c["H"])
+    # the tables the stages hand on: each pair's arrival position, the [T, k] entry behind each Hop-A pair, the
+    # combine's place table, and the one-pass Hop B's place of each pair in arrival order
+    pair_src = np.full(pair_tab.size, -1, dtype=np.int64)
+    live = pair_tab.reshape(-1) >= 0
+    pair_src[pair_tab.reshape(-1)[live]] = np.nonzero(live)[0]
+    one = orc.hopb_local_scatter(payload, mask, gate_rows, q, slots, 0, c["capacity"])
+    assert np.array_equal(one[0], perm)
+    out.update(pair_pos=pos, pair_src=pair_src, where=where.astype(np.int64), onepass_place=one[1],
+               kept_per_expert=one[4])
     return out

@@ -489,6 +489,12 @@ def test_kernels_reproduce_the_committed_fixture(name):
                tokens_per_expert=st.tokens_per_expert, y=y)
     if c["capacity"] is not None:
         got["kept"] = st.kept
+    from terrace.ta2a_fwd import loopback_dispatch_onepass
+    one = loopback_dispatch_onepass(x.to(DEV), e, g_pay.to(DEV), c["world"], c["E"], c["rpn"], c["M"], c["capacity"])
+    assert torch.equal(one.permuted, st.permuted)
+    got.update(pair_pos=st.pair_pos, pair_src=st.extras["pair_src"], where=st.extras["where"], onepass_place=one.place,
+               kept_per_expert=one.extras["kept_per_expert"])
+    assert torch.equal(st.extras["kept_per_expert"], one.extras["kept_per_expert"])
     assert sorted(got) == sorted(want)
     wrong = [k for k, v in got.items() if gc.digest(to_np(v)) != want[k]]
     assert not wrong, f"{name}: {wrong} differ from the committed fixture"
