@@ -240,6 +240,7 @@ struct EmitPlanWide {
     int k, slots, n_experts;
     int64_t *u_src, *u_node, *inverse;
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     typedef NoPre Pre;
     __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
     __device__ __forceinline__ int operator()(int64_t item, int node, int32_t row, int64_t, Pre, const int32_t *,
@@ -566,6 +567,7 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
         const int64_t item = first + (int64_t)c * kWave + lane;
         if (keys[c] >= 0) fault |= emit(item, keys[c], dests[c], fetched[c], pre[c], start, tally);
     }
+    if constexpr (EmitFn::kFills) emit.fill(unit, u.n_units, lane, start);
     if (!status) return;
     if (fault) atomicOr(&status[0], fault);
     if (EmitFn::kTallies) {
@@ -587,6 +589,7 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
 struct EmitOrder {           // plain stable argsort: order[dest] = item
     int64_t *order;
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     typedef NoPre Pre;
     __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
     __device__ __forceinline__ int operator()(int64_t item, int, int32_t dest, int64_t, Pre, const int32_t *,
@@ -598,6 +601,7 @@ struct EmitOrder {           // plain stable argsort: order[dest] = item
 
 struct EmitNothing {
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     typedef NoPre Pre;
     __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
     __device__ __forceinline__ int operator()(int64_t, int, int32_t, int64_t, Pre, const int32_t *, int *) const {
@@ -617,6 +621,7 @@ struct EmitArrival {         // terrace/ops/__init__.py:287-299
     const int64_t *tags_in;  // [P] a caller's tag per pair, carried to the pair's place: tags_out[dest] = tags_in[p]
     int64_t *tags_out;
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     struct Pre { uint32_t gbits; int64_t tag; };
     __device__ __forceinline__ Pre fetch(int64_t p) const {
         Pre pre{0u, -1};
@@ -662,6 +667,7 @@ struct EmitHopB {            // arrival + expert-order regroup in one placement 
     int64_t *place_by_tag;
     int64_t n_tags;
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     struct Pre { uint32_t gbits; int64_t tag; };
     __device__ __forceinline__ Pre fetch(int64_t p) const {
         Pre pre{0u, -1};
@@ -739,6 +745,7 @@ struct EmitPairs {           // terrace/ta2a_fwd.py:605-628, general branch: pai
     int64_t *r_idx, *slot_idx, *ordo;
     int32_t *src32;          // source row of each output place (-1: row id out of range)
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = false;
     struct Pre { int64_t r; };
     __device__ __forceinline__ Pre fetch(int64_t p) const { return Pre{r_in[p]}; }
     __device__ __forceinline__ int operator()(int64_t p, int, int32_t dest, int64_t sl, Pre pre, const int32_t *,
@@ -771,7 +778,23 @@ struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
     void *gate_out;          // the padded plane is gathered per place afterwards (its padding places are zeros)
     int gate_bytes;
     int64_t gate_pitch;
+    int32_t *gidx;           // capacity layout only: the source row of every place, -1 for a padding place
+    int epr;
     static constexpr bool kTallies = false;
+    static constexpr bool kFills = true;
+    // The padding places of the capacity layout, shared out over the launch's units: place d = x*capacity + r is
+    // padding when r is past expert x's count (the kept places are written by the rows that take them).
+    __device__ __forceinline__ void fill(int unit, int n_units, int lane, const int32_t *start) const {
+        if (capacity < 0 || !gidx) return;
+        const int64_t places = (int64_t)epr * capacity;
+        const int64_t per = (places + n_units - 1) / n_units;
+        const int64_t lo = (int64_t)unit * per, hi = lo + per < places ? lo + per : places;
+        for (int64_t d = lo + lane; d < hi; d += kWave) {
+            const uint32_t x = (uint32_t)d / (uint32_t)capacity;          // places < 2^31
+            const int64_t r = d - (int64_t)x * capacity;
+            if (r >= start[x + 1] - start[x]) gidx[d] = -1;
+        }
+    }
     struct Pre { int64_t tag; uint32_t gate; };
     __device__ __forceinline__ Pre fetch(int64_t p) const {
         Pre pre{tags_in ? tags_in[p] : -1, 0u};
@@ -796,6 +819,7 @@ struct EmitRegroup {         // terrace/ta2a_fwd.py:641-646 (+ capacity cut)
         }
         if (dest_out) dest_out[p] = d;
         if (kept) kept[p] = keep ? 1 : 0;
+        if (capacity >= 0 && gidx && keep) gidx[d] = (int32_t)p;
         if (place_by_tag && (uint64_t)pre.tag < (uint64_t)n_tags) place_by_tag[pre.tag] = d;
         return 0;
     }
@@ -816,6 +840,7 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
     // status word 1 receives the number of occupied (token, node) pairs, word 2 the number of
     // those holding other than k/M experts: the two quantities terrace/ta2a.py:170-204 checks.
     static constexpr bool kTallies = true;
+    static constexpr bool kFills = false;
     typedef NoPre Pre;
     __device__ __forceinline__ Pre fetch(int64_t) const { return Pre{}; }
     // rank m*quota + i of token t and cell i of its send row `row`: no pair, zero slot, zero gate
@@ -938,25 +963,6 @@ struct EmitPack {            // terrace/ta2a.py:246-253 + terrace/ta2a_fwd.py:23
         return fault;
     }
 };
-
-// Per-place source row for the capacity layout: gidx[x*C + r] = order[start[x] + r] or -1
-// (places = epr*C; with places = 0 only kept_per_expert = min(count, capacity) is written).
-__global__ __launch_bounds__(kBlock) void capacity_index_kernel(const int32_t *__restrict__ order32,
-                                                                const int32_t *__restrict__ start, int epr,
-                                                                int64_t capacity, int64_t places,
-                                                                int32_t *__restrict__ gidx,
-                                                                int64_t *__restrict__ kept_per_expert) {
-    const int64_t d = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (d < epr && kept_per_expert) {
-        const int64_t c = start[d + 1] - start[d];
-        kept_per_expert[d] = c < capacity ? c : capacity;
-    }
-    if (d >= places) return;
-    const int x = (int)(d / capacity);
-    const int64_t r = d - x * capacity;
-    const int64_t c = start[x + 1] - start[x];
-    gidx[d] = r < c ? order32[start[x] + r] : -1;
-}
 
 __global__ __launch_bounds__(kBlock) void fill_zero_kernel(uint8_t *__restrict__ p, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) p[i] = 0;
@@ -1344,20 +1350,15 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     const bool gate_in_sort = my_gate && capacity < 0;
     EmitRegroup emit{capacity, order, dest, kept, order32, tagged ? tags_in : nullptr,
                      tagged ? place_by_tag : nullptr, n_tags, gate_in_sort ? my_gate : nullptr,
-                     gate_in_sort ? permuted_gate : nullptr, gate_bytes, gate_pitch};
+                     gate_in_sort ? permuted_gate : nullptr, gate_bytes, gate_pitch, capacity >= 0 ? gidx : nullptr,
+                     epr};
     TableOut out;
     out.hist_i64 = tokens_per_expert;
-    if (capacity < 0) out.kept_i64 = kept_per_expert;          // nothing is dropped: the sort's own publication
+    out.kept_i64 = kept_per_expert;                            // min(count, capacity): the sort's own publication
+    if (capacity >= 0) out.capacity = capacity;
     int rc = run_sort(key, emit, u, table, out, status, true, s);
     if (rc != TERRACE_OK) return rc;
-    const int32_t *src_of_place = order32;
-    const int32_t *start = table + units_start_at(u);
-    if (capacity >= 0) {
-        const int64_t n = places > epr ? places : epr;
-        capacity_index_kernel<<<(int)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(order32, start, epr, capacity,
-                                                                                 places, gidx, kept_per_expert);
-        src_of_place = gidx;
-    }
+    const int32_t *src_of_place = capacity >= 0 ? gidx : order32;    // the rank kernel filled gidx, padding included
     if (my_gate && places > 0 && !gate_in_sort) {
         const int grid = (int)((places + kBlock - 1) / kBlock);
         if (gate_bytes == 4)
