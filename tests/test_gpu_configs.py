@@ -210,15 +210,20 @@ def _check_every_plane(cfg):
     # ---- the stated tolerance against float64
     src64 = orc.decode_rows(ye_rows, fmt_in, cfg.hidden).astype(np.float64)
     ref = np.zeros((cfg.T, cfg.hidden))
+    mag = np.zeros((cfg.T, cfg.hidden))
     for j in range(cfg.top_k):
         ok = where[:, j] >= 0
-        ref += np.where(ok[:, None], src64[np.where(ok, where[:, j], 0)] * wf[:, j:j + 1].astype(np.float64), 0.0)
+        term = np.where(ok[:, None], src64[np.where(ok, where[:, j], 0)] * wf[:, j:j + 1].astype(np.float64), 0.0)
+        ref += term
+        mag += np.abs(term)
     err = np.abs(orc.decode_rows(to_np(got), out_fmt) - ref).max() / (np.abs(ref).max() + 1e-30)
     assert err <= TOL[cfg.fmt], err
     # ---- the reference's two-level shape agrees with the fused one to the same tolerance
     if cfg.fmt != "fp8":
         two = twolevel_combine(ye, st, out_dtype=cfg.out_dtype)
-        err2 = np.abs(orc.decode_rows(to_np(two), out_fmt) - ref).max() / (np.abs(ref).max() + 1e-30)
+        # that shape rounds every partial sum to the payload dtype, so its error follows the magnitudes added, not
+        # their sum: raw-affinity gates can be negative and cancel
+        err2 = np.abs(orc.decode_rows(to_np(two), out_fmt) - ref).max() / (mag.max() + 1e-30)
         assert err2 <= 2 * TOL[cfg.fmt], err2
 
 
