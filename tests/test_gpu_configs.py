@@ -230,8 +230,25 @@ def _check_every_plane(cfg):
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
 def test_full_size_index_planes_and_round_trip(name):
     from terrace import configs
+    _full_size_check(configs.CONFIGS[name])
+
+
+@pytest.mark.parametrize("fmt,tokens", [("bf16", 49152), ("fp8", 81920)])
+def test_buffers_beyond_four_gigabytes(fmt, tokens):
+    """Three (five, for the one-byte rows) times the tokens of the DeepSeek-V3-shaped slice: the arrival and
+    expert-order buffers are 5.6 GB (4.8 GB) each, so every row offset past the first 4 GB needs more than 32 bits,
+    in every mover -- the kilobyte-sliced ones and the ones for other widths -- and in the combine."""
+    from terrace import configs
+    cfg = configs.PathConfig("beyond_4gb_" + fmt, tokens, 256, 8, 8, 4, 8, 7168, fmt, bias="normal", softmax_gates=True,
+                             seed=20261127)
+    assert cfg.pairs * cfg.row_bytes > 4.5 * (1 << 30)
+    _full_size_check(cfg)
+    torch.cuda.empty_cache()
+
+
+def _full_size_check(cfg):
+    from terrace import configs
     from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, loopback_dispatch_onepass
-    cfg = configs.CONFIGS[name]
     announce("full", cfg.name, cfg.T)
     inp = configs.make_inputs(cfg)
     e, g32, oe, og = _route(cfg, inp)
