@@ -32,7 +32,9 @@ GEOMS = [(4, 2, 8, 9, 3), (32, 8, 64, 40, 4), (16, 8, 32, 17, 5), (64, 8, 128, 3
          # more than 64 destination nodes (the reference's general plan has no node bound, terrace/ta2a.py:205-253):
          # 80, 128 and 300 nodes, several experts of a token on one node, a single token, many units
          (640, 8, 1280, 500, 8), (1024, 8, 1024, 257, 12), (600, 2, 2400, 90, 16), (160, 2, 160, 1, 4),
-         (1040, 8, 4160, 20000, 6)]
+         (1040, 8, 4160, 20000, 6),
+         # the widest table the sorts take: 2048 nodes
+         (2048, 1, 2048, 700, 8)]
 
 
 @pytest.mark.parametrize("world,rpn,E,T,k", GEOMS)
