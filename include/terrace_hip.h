@@ -404,9 +404,15 @@ TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, 
  * rpn) > terrace_static_scratch_bytes(); about 900 thousand pairs) are refused with TERRACE_E2BIG.  The call
  * allocates and frees nothing.  Unlike the rest of the library it is not reentrant: all calls on one GPU use
  * that GPU's one array, so two of them must not overlap (same stream, or ordered by events).  The device the
- * stream belongs to must be current. */
+ * stream belongs to must be current.
+ *
+ * The first call on a device looks the array's device address up (hipGetSymbolAddress, a runtime call that takes
+ * a lock and may load the code object).  That must not happen under stream capture: call terrace_static_init()
+ * once per device beforehand, with that device current (it does only the look-up, launches nothing and is
+ * idempotent), or make one eager call first.  Every later call on that device is kernel launches only. */
 #define TERRACE_STATIC_SCRATCH_BYTES (4u << 20)
 TERRACE_API size_t terrace_static_scratch_bytes(void);
+TERRACE_API int terrace_static_init(void);
 TERRACE_API int terrace_k1_arrival_static(const void *rx, const int64_t *rslot, const void *rgate, int64_t R,
                                           int64_t row_bytes, int gate_bytes, int quota, int epr, int rpn,
                                           int my_local, void *send_buf, void *gate_pairs, int64_t *r_idx,

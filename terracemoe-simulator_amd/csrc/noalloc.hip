@@ -10,6 +10,10 @@
 // ever handed to a kernel.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU race.
 // Nothing in it has to start at zero -- the count kernel writes every table entry and the rank kernel every
 // position before either is read -- so a call never depends on what the last one left behind.
+//
+// The look-up is a runtime call that may load the code object, so it must not happen while a stream is being
+// captured: terrace_static_init() does it for the current device ahead of time (the first
+// terrace_k1_arrival_static call on a device does the same when nobody called it).
 #include <atomic>
 #include <mutex>
 
@@ -58,6 +62,11 @@ void *scratch_of_current_device(int *rc) {
 extern "C" {
 
 size_t terrace_static_scratch_bytes(void) { return (size_t)TERRACE_STATIC_SCRATCH_BYTES; }
+
+int terrace_static_init(void) {
+    int rc = TERRACE_OK;
+    return scratch_of_current_device(&rc) ? TERRACE_OK : rc;
+}
 
 int terrace_k1_arrival_static(const void *rx, const int64_t *rslot, const void *rgate, int64_t R, int64_t row_bytes,
                               int gate_bytes, int quota, int epr, int rpn, int my_local, void *send_buf,

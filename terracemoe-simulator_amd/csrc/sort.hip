@@ -709,7 +709,7 @@ struct EmitHopB {            // arrival + expert-order regroup in one placement 
 constexpr int kPadRows = 16;
 template <typename V>
 __global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restrict__ start, int epr, int64_t capacity,
-                                                          int chunks, V *__restrict__ rows, int64_t row_vecs,
+                                                          int chunks, int pad_rows, V *__restrict__ rows, int64_t row_vecs,
                                                           void *__restrict__ gate_plane, int gate_bytes,
                                                           int64_t *__restrict__ pair_of_place,
                                                           int64_t *__restrict__ kept_per_expert) {
@@ -717,7 +717,7 @@ __global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restr
     const int64_t count = start[x + 1] - start[x];
     const int64_t used = count < capacity ? count : capacity;
     if (c == 0 && threadIdx.x == 0 && kept_per_expert) kept_per_expert[x] = used;
-    int64_t lo = (int64_t)c * kPadRows, hi = lo + kPadRows;
+    int64_t lo = (int64_t)c * pad_rows, hi = lo + pad_rows;
     if (lo < used) lo = used;
     if (hi > capacity) hi = capacity;
     if (lo >= hi) return;
@@ -1216,21 +1216,24 @@ static int launch_zero_pad(const int32_t *start, int epr, int64_t capacity, void
                            void *gate_plane, int gate_bytes, int64_t *pair_of_place, int64_t *kept_per_expert,
                            hipStream_t s) {
     if (epr <= 0) return TERRACE_OK;
-    const int chunks = capacity > 0 ? (int)((capacity + kPadRows - 1) / kPadRows) : 1;
+    // kPadRows places per workgroup; more where that many workgroups would pass what one launch can hold
+    // (blocks * kBlock has to stay below 2^32)
+    int pad_rows = kPadRows;
+    while ((int64_t)epr * ((capacity + pad_rows - 1) / pad_rows) > (int64_t)1 << 22) pad_rows *= 2;
+    const int chunks = capacity > 0 ? (int)((capacity + pad_rows - 1) / pad_rows) : 1;
     const int64_t blocks = (int64_t)epr * chunks;
-    if (blocks >= (int64_t)1 << 31) return TERRACE_EINVAL;
     if (!rows || row_bytes == 0) {
-        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, nullptr, 0,
+        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows, nullptr, 0,
                                                                     gate_plane, gate_bytes, pair_of_place,
                                                                     kept_per_expert);
     } else if ((((uintptr_t)rows | (uintptr_t)row_bytes) & 15) == 0) {
-        zero_pad_kernel<pad_u32x4><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, (pad_u32x4 *)rows,
-                                                                      row_bytes / 16, gate_plane, gate_bytes,
-                                                                      pair_of_place, kept_per_expert);
+        zero_pad_kernel<pad_u32x4><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows,
+                                                                      (pad_u32x4 *)rows, row_bytes / 16, gate_plane,
+                                                                      gate_bytes, pair_of_place, kept_per_expert);
     } else {
-        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, (uint8_t *)rows,
-                                                                    row_bytes, gate_plane, gate_bytes, pair_of_place,
-                                                                    kept_per_expert);
+        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows,
+                                                                    (uint8_t *)rows, row_bytes, gate_plane, gate_bytes,
+                                                                    pair_of_place, kept_per_expert);
     }
     return check_launch();
 }

@@ -84,6 +84,7 @@ SIGNATURES = {
     "terrace_routing_map_topk": (_I, [_P, _P, _I, _L, _I, _I, _P, _P, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
     "terrace_static_scratch_bytes": (_Z, []),
+    "terrace_static_init": (_I, []),
     "terrace_k1_arrival_static": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I,
                                        _P, _P, _P, _P, _P, _P, _P, _P]),
 }

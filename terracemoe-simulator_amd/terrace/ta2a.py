@@ -36,11 +36,16 @@ def _raise_from_status(status: torch.Tensor, T: int, k: int, groups_m: int):
             f"only for equal-quota routings (t_route mode='full'/'quota_only'), leave it None otherwise.")
 
 
-def _guard(status, T, k, n_nodes, groups_m):
-    key = (T, k, n_nodes, groups_m)
+def _guard_due(key) -> bool:
+    """Counts one call of shape ``key`` and says whether the guard reads the status words back on it."""
     cnt = _VERIFY_COUNT.get(key, 0)
     _VERIFY_COUNT[key] = cnt + 1
-    if key not in _VERIFIED or cnt % 256 == 0:
+    return key not in _VERIFIED or cnt % 256 == 0
+
+
+def _guard(status, T, k, n_nodes, groups_m):
+    key = (T, k, n_nodes, groups_m)
+    if _guard_due(key):
         _raise_from_status(status, T, k, groups_m)
         _VERIFIED.add(key)
 

@@ -269,10 +269,18 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
               at("x.gate_sorted"), at("x.pair_src"), at("x.where"), at("x.status"), at("_ws_k2"), slab.nbytes("_ws_k2"),
               stream)
     extras = _planes.LazyDict(slab, "x.")
+    # the plan's guard (terrace/ta2a.py:161-204 of the reference): the status words are read back on the first
+    # dispatch of a shape and on every 256th, after the last launch below so the read-back waits for nothing extra
+    from . import ta2a as _plan
+    guard_key = (T, k, n_nodes, groups_m)
+    guard = _plan._guard_due(guard_key)
     if onepass:
         _hip.call("terrace_hopb_scatter", ptr(payload), at("mask"), None, S, row_bytes, gb, quota, 0, slots, cap,
                   ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"), at("x.kept_per_expert"),
                   at("x.pair_src"), at("x.where"), P, at("_status_b"), at("_ws_b"), slab.nbytes("_ws_b"), stream)
+        if guard:
+            _plan._raise_from_status(extras["status"], T, k, groups_m)
+            _plan._VERIFIED.add(guard_key)
         return OnePassState(slab, ("kept",), payload=payload, permuted=permuted, extras=extras, capacity=capacity)
     send_buf = torch.empty((P, H), dtype=x.dtype, device=dev)
     _hip.call("terrace_k1_arrival", ptr(payload), at("mask"), at("gate_rows"), S, row_bytes, gb, quota, epr, rpn, 0,
@@ -281,6 +289,9 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
     _hip.call("terrace_regroup", ptr(send_buf), at("slot_idx"), None, P, row_bytes, gb, slots, 0, cap, ptr(permuted),
               None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"), at("x.kept_per_expert"),
               at("_carried"), at("x.where"), P, at("_status_r"), at("_ws_r"), slab.nbytes("_ws_r"), stream)
+    if guard:
+        _plan._raise_from_status(extras["status"], T, k, groups_m)
+        _plan._VERIFIED.add(guard_key)
     return LoopbackState(slab, ("kept",), payload=payload, send_buf=send_buf, permuted=permuted, extras=extras,
                          capacity=capacity)
 

@@ -415,7 +415,10 @@ def test_malformed_routing_is_contained_and_counted():
         e = torch.tensor(rows, device=DEV)
         x = torch.randn(6, 16, device=DEV)
         gts = torch.rand(6, 4, device=DEV)
-        (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e, gts, 4, 8, 2, 2, extras=True)
+        (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e, gts, 4, 8, 2, 2, extras=True,
+                                                                         combine_table=True)
+        assert ((ex["pair_src"] >= -1) & (ex["pair_src"] < 24)).all()
+        assert (ex["where"] == -1).all(), "the pre-set combine table of a malformed token must read -1"
         fault, occ, offq, _ = ex["status"].tolist()
         assert fault != 0 and occ == occupied and offq == off_quota, (name, fault, occ, offq)
         assert int(counts.sum()) <= 12 and (counts >= 0).all()
@@ -453,6 +456,64 @@ def test_malformed_routing_is_contained_and_counted():
         clean[1:6] = False
         rows_of_clean = ex["token_rows"].cpu()[clean]
         assert torch.equal(payload.cpu()[rows_of_clean.reshape(-1)], x.cpu()[clean].repeat_interleave(M, 0))
+
+
+def _poison_next_allocation(nbytes):
+    """Leaves a freed block of ``nbytes`` full of 0x5A bytes at the head of torch's cache, so that the next
+    allocation of that size starts from garbage that reads as huge positive ids."""
+    junk = torch.full((nbytes,), 0x5A, dtype=torch.uint8, device=DEV)
+    torch.cuda.synchronize()
+    del junk
+
+
+@pytest.mark.parametrize("onepass", [False, True])
+def test_malformed_routing_through_the_whole_dispatch(onepass):
+    """The loop-back dispatch on a slab that arrives full of garbage, with tokens that break every invariant: the
+    combine's place table, filled through the tag chain, must name a valid place or -1 for every entry, pair_src
+    must stay inside [-1, T*k), and the combine over it must be finite -- on the lane-per-token send side (k <= 16,
+    <= 64 nodes) and on the item kernels (k = 24; 80 nodes)."""
+    from terrace import ta2a_fwd
+    announce("dispatch malformed", onepass)
+    for world, rpn, E, T, k, M in [(4, 2, 8, 70, 4, 2), (64, 8, 256, 300, 8, 4), (8, 2, 64, 40, 24, 4),
+                                   (160, 2, 160, 50, 4, 2)]:
+        n_nodes, slots, q = world // rpn, (E // world) * rpn, k // M
+        g = torch.Generator().manual_seed(T)
+        e = torch.from_numpy(equal_quota_routing(T, k, E, n_nodes, M, 5, False)).clone()
+        e[1, 0] = E + 7                          # outside [0, E)
+        e[2, 1] = -3
+        e[3, :] = e[3, 0]                        # one expert k times
+        e[5] = torch.randint(0, E, (k,), generator=g)     # no quota structure at all
+        e[7, :q + 1] = e[7, 0] // slots * slots + torch.arange(q + 1) % slots   # q + 1 experts on one node
+        x = torch.randn(T, 32, generator=g).to(DEV)
+        gts = torch.rand(T, k, generator=g).to(DEV)
+        lay = ta2a_fwd._dispatch_layout(T, k, M, n_nodes, rpn, slots, None, gts.dtype, onepass)
+        dispatch = ta2a_fwd.loopback_dispatch_onepass if onepass else ta2a_fwd.loopback_dispatch
+        # the first dispatch of a shape reads the guard's census back and raises on such a routing; later ones
+        # (up to the 256th) run unchecked, which is the case that has to be contained
+        from terrace import ta2a
+        ta2a._VERIFIED.discard((T, k, n_nodes, M)), ta2a._VERIFY_COUNT.pop((T, k, n_nodes, M), None)
+        with pytest.raises(ValueError):
+            dispatch(x, e.to(DEV), gts, world, E, rpn, M)
+        ta2a._VERIFIED.add((T, k, n_nodes, M))
+        _poison_next_allocation(max(lay.total, 256))
+        st = dispatch(x, e.to(DEV), gts, world, E, rpn, M)
+        torch.cuda.synchronize()
+        P = T * k
+        pair_src, where = st.extras["pair_src"], st.extras["where"]
+        assert bool(((pair_src >= -1) & (pair_src < P)).all()), "pair_src out of range"
+        assert bool(((where >= -1) & (where < st.permuted.shape[0])).all()), "combine table out of range"
+        assert st.extras["status"].tolist()[0] != 0
+        # a live entry names the place of the very pair that answers it
+        live = where.reshape(-1) >= 0
+        assert int(live.sum()) >= (T - 6) * k
+        y = ta2a_fwd.loopback_combine(st.permuted, st)
+        assert bool(torch.isfinite(y).all())
+        # the clean tokens combine to what the oracle's table gives on the clean part alone
+        clean = torch.ones(T, dtype=torch.bool)
+        clean[[1, 2, 3, 5, 7]] = False
+        assert bool((where.cpu()[clean] >= 0).all())
+        rows = st.permuted[where[clean.to(DEV)].reshape(-1)].view(-1, k, 32)
+        assert torch.equal(rows, x[clean.to(DEV)][:, None, :].expand(-1, k, -1)), "a clean token's places hold other rows"
 
 
 def test_hopa_send_splits_literal(literals):
