@@ -1,7 +1,7 @@
 """Benchmark of one rank's dispatch/combine path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--no-other-configs]
-                    [--graph]
+                    [--no-seam] [--graph]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM: T-Route -> dispatch index build + Hop-A deduplicated pack -> Hop-B arrival chain ->
@@ -51,6 +51,7 @@ def parse():
     ap.add_argument("--config", default="c2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
+    ap.add_argument("--no-seam", action="store_true", help="skip the ta2a_permute / ta2a_unpermute timings")
     ap.add_argument("--graph", action="store_true",
                     help="also capture the step into a HIP graph and time its replays (reported beside the eager "
                          "figure, which stays `value`)")
@@ -273,6 +274,131 @@ def cpu_baseline(cfg, sample_tokens):
 
 
 # ------------------------------------------------------------------------------------------------------------------
+# stream ceilings, the seam halves, a step inside a HIP graph
+# ------------------------------------------------------------------------------------------------------------------
+
+def stream_ceilings(torch, reps):
+    """What the part sustains, in this run, for the traffic mixes the row movers are made of: the library's own
+    stream probes (terrace_stream_probe) at the c2 sizes -- a 1.88 GB read-only stream, a 0.94 GB write-only one,
+    the 8:1 streaming sum (1.88 GB read, 0.23 GB written) and a 1.88 + 1.88 GB copy in one-wave workgroups --
+    beside terrace_passthrough's 256-lane copy."""
+    import terrace.ops as tops
+    dev = torch.device("cuda:0")
+    big = 1879048192                       # bytes of c2's arrival buffer
+    src = torch.zeros(big, dtype=torch.uint8, device=dev)
+    dst = torch.empty(big, dtype=torch.uint8, device=dev)
+    out = {}
+    cases = {"read_only": ("read", src, dst, big), "write_only": ("write", None, dst[: big // 2], big // 2),
+             "sum_8_to_1": ("sum8", src, dst[: big // 8], big + big // 8), "copy_one_wave": ("copy", src, dst, 2 * big)}
+    for name, (kind, x, y, nbytes) in cases.items():
+        ms = event_ms(lambda: tops.stream_probe(kind, x, y), reps, torch)
+        out[name] = {"ms": round(ms, 4), "bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    ms = event_ms(lambda: tops.passthrough(src), reps, torch)
+    out["copy_passthrough"] = {"ms": round(ms, 4), "bytes": 2 * big, "GBps": round(2 * big / ms / 1e6, 1),
+                               "frac_hbm_peak": round(2 * big / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    out["note"] = ("terrace_stream_probe kernels timed like the movers (HIP events, median of batches); a mover's "
+                   "floor on this part is its read bytes at the read_only rate plus its written bytes at the "
+                   "write_only rate")
+    return out
+
+
+def predicted_floor_ms(ceil, read_bytes, written_bytes):
+    """Milliseconds a kernel's bytes cost at the run's own read-only and write-only stream rates."""
+    return read_bytes / (ceil["read_only"]["GBps"] * 1e6) + written_bytes / (ceil["write_only"]["GBps"] * 1e6)
+
+
+def count_launches(fn, torch):
+    """Kernel launches one call of fn() makes, from torch's profiler (None when it is unavailable, e.g. under
+    another profiler)."""
+    try:
+        from torch.profiler import ProfilerActivity, profile
+        fn()
+        torch.cuda.synchronize()
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            fn()
+            torch.cuda.synchronize()
+        n = 0
+        for ev in prof.events():
+            if ev.device_type is not None and "cuda" in str(ev.device_type).lower() and "memcpy" not in ev.name.lower() \
+                    and "memset" not in ev.name.lower():
+                n += 1
+        return n or None
+    except Exception:
+        return None
+
+
+def seam_block(cfg, args, torch, raw_step_ms, e, gates, x):
+    """The Megatron-shaped surface (terrace/ta2a_dispatch.py of the reference: ta2a_permute -> experts ->
+    ta2a_unpermute) at this workload's shape: ms per permute + unpermute pair, launches and host synchronisations
+    per pair, and the ratio to the raw loop-back step (route excluded there as here)."""
+    import terrace.ta2a_dispatch as seam
+    from terrace import ta2a_pack
+    dev = x.device
+    T, E = cfg.T, cfg.n_experts
+    routing_map = torch.zeros((T, E), dtype=torch.bool, device=dev)
+    routing_map.scatter_(1, e, True)
+    probs = torch.zeros((T, E), dtype=x.dtype, device=dev)
+    probs.scatter_(1, e, gates.to(x.dtype))
+    kw = dict(world=cfg.world, rank=0, rpn=cfg.rpn, n_experts=E)
+    ta2a_pack.reset()
+
+    def plain(groups_m):
+        def run():
+            permuted, _tpe, _pp, st = seam.ta2a_permute(x, probs, routing_map, groups_m=groups_m, **kw)
+            return seam.ta2a_unpermute(permuted, st, x)
+        return run
+
+    def overlap():
+        saved = []
+        permuted, _tpe, _pp, _sh, st = seam.ta2a_permute_overlap(x, probs, routing_map, groups_m=cfg.top_groups,
+                                                                save_tensors=saved, **kw)
+        return seam.ta2a_unpermute_overlap(permuted.detach(), st, saved)
+
+    legs = {"quota_branch_small_containers": (plain(cfg.top_groups), 1),
+            "general_branch": (plain(None), 2),
+            "overlap_seam_quota_branch": (overlap, 1)}
+    out = {"container_mode": ta2a_pack.pack_mode(), "raw_dispatch_plus_combine_ms": round(raw_step_ms, 4),
+           "note": "wall time per ta2a_permute + ta2a_unpermute pair (expert output = the permuted rows), host "
+                   "synchronisations included; the raw figure is loopback_dispatch + the fused combine on the same "
+                   "rows.  The seam's combine is the reference's two levels (a send row sums its pairs, a token its "
+                   "rows): it writes and re-reads the [T*M, H] plane the fused combine never forms"}
+    with torch.no_grad():
+        for name, (fn, syncs) in legs.items():
+            ms = wall_ms(fn, max(args.steps // 2, 5), 2, torch)
+            out[name] = {"ms_per_call": round(ms, 4), "ratio_to_raw": round(ms / raw_step_ms, 3),
+                         "kernel_launches": count_launches(fn, torch), "host_syncs": syncs}
+    return out
+
+
+def graph_replay_ms(step, args, torch):
+    """The step captured once into a HIP graph: ms per replay, and whether replays interleaved with eager steps
+    reproduce the eager result every time."""
+    y_eager = step()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_graph = step()
+    same = True
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        same = same and bool(torch.equal(y_graph, y_eager))
+        step()
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / args.steps, 4), "replays_match_eager": same}
+
+
+# ------------------------------------------------------------------------------------------------------------------
 # one workload on the GPU
 # ------------------------------------------------------------------------------------------------------------------
 
@@ -360,6 +486,8 @@ def run_workload(cfg, args, torch, detail):
         ms_arr, ms_pack, ms_comb = event_ms(arrival, reps, torch), event_ms(pack, reps, torch), event_ms(combine, reps, torch)
         out["arrival_us_per_row"] = ms_arr * 1e3 / cfg.pairs
         out["pack_plus_combine_frac_hbm_peak"] = gbps(phys["pack"] + phys["combine"], ms_pack + ms_comb) / HBM_PEAK_GBPS
+        # a step this short is bound by the host's launches: its HIP-graph replay says what the kernels alone take
+        out["graph"] = graph_replay_ms(step, args, torch) if (args.graph or ms_per_step < 0.3) else None
         return out
 
     # ---- per-stage timings (each stage alone, HIP events on the launch stream) ----
@@ -429,31 +557,40 @@ def run_workload(cfg, args, torch, detail):
         kern[name] = {"ms": round(ms, 4), "bytes_per_launch": nb, "GBps": round(nb / ms / 1e6, 1),
                       "frac_hbm_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     out["kernels"] = kern
-    out["graph"] = None
-    if args.graph:
-        y_eager = step()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                step()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            y_graph = step()
-        same = True
-        for _ in range(3):                 # replays interleaved with eager work must all reproduce the eager result
-            graph.replay()
-            torch.cuda.synchronize()
-            same = same and bool(torch.equal(y_graph, y_eager))
-            step()
-            torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        out["graph"] = {"ms_per_step": round((time.perf_counter() - t0) * 1e3 / args.steps, 4),
-                        "replays_match_eager": same}
+    out["graph"] = graph_replay_ms(step, args, torch) if args.graph else None
+    # ---- each stage timed INSIDE the step: events between the stage calls of K whole steps, so that no stage sees
+    # inputs a previous launch of itself left in a cache (alone, back to back, the pack re-reads the same 235 MB)
+    names = ("route", "pack", "arrival", "regroup", "combine")
+    marks = []
+    for it in range(reps + 2):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+        ev[0].record()
+        e_, g_, _ = route()
+        ev[1].record()
+        (pl_, mk_, gr_, _us, _nc), ex_ = tops.k2_pack_raw(x, e_, g_, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups,
+                                                          extras=True, combine_table=True)
+        ev[2].record()
+        tg_ = []
+        sb_, _gp, _ri, si_, _is, _pp = tops.k1_arrival_raw(pl_, mk_, gr_, quota, cfg.epr, cfg.rpn, 0, want_pair_pos=True,
+                                                           tags=ex_["pair_src"], tags_out=tg_)
+        ev[3].record()
+        tops.regroup(sb_, si_, cfg.slots, 0, cap, tags=tg_[0], table=ex_["where"])
+        ev[4].record()
+        tops.combine(ye, ex_["where"], ex_["gate_sorted"], out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+        ev[5].record()
+        if it >= 2:
+            marks.append(ev)
+    torch.cuda.synchronize()
+    in_step = {n: statistics.median(m[i].elapsed_time(m[i + 1]) for m in marks) for i, n in enumerate(names)}
+    pc_in = in_step["pack"] + in_step["combine"]
+    out["in_step"] = {"stage_ms": {n: round(v, 4) for n, v in in_step.items()},
+                      "stage_frac_hbm_peak": {n: round(gbps(phys[n], v) / HBM_PEAK_GBPS, 4) for n, v in in_step.items()},
+                      "pack_plus_combine_ms": round(pc_in, 4),
+                      "pack_plus_combine_frac_hbm_peak": round(gbps(phys["pack"] + phys["combine"], pc_in) / HBM_PEAK_GBPS, 4),
+                      "note": "median over the timed steps of the time between HIP events recorded around each stage "
+                              "call inside whole steps (stage operators called one by one, same kernels)"}
+    out["raw_dispatch_plus_combine_ms"] = sum(v for n, v in in_step.items() if n != "route")
+    out["tensors"] = (e, gates, x)
     return out
 
 
@@ -481,6 +618,26 @@ def main():
 
     r = run_workload(cfg, args, torch, detail=True)
     kern, stages = r["kernels"], r["stages"]
+    seam = None
+    if not args.no_seam and cfg.fmt != "fp8":          # the seam's probs plane has the payload's float dtype
+        seam = seam_block(cfg, args, torch, r["raw_dispatch_plus_combine_ms"], *r["tensors"])
+    del r["tensors"]
+    torch.cuda.empty_cache()
+    ceilings = stream_ceilings(torch, max(args.steps, 5))
+    torch.cuda.empty_cache()
+    # every mover beside what its bytes cost at this run's own read-only and write-only stream rates
+    row, S, P, T = cfg.row_bytes, cfg.send_rows, cfg.pairs, cfg.T
+    kept = P if r["kept_pairs"] is None else r["kept_pairs"]
+    n_places = P if r["places"] is None else r["places"]
+    out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
+    rw = {"(pack)": (T * row, S * row), "(arrival)": (S * row, P * row), "(hopb_onepass)": (S * row, kept * row),
+          "(regroup)": (kept * row, n_places * row), "combine_kernel": (kept * row + P * 12, T * out_row)}
+    for name, v in kern.items():
+        for tag, (rd, wr) in rw.items():
+            if name.endswith(tag):
+                floor = predicted_floor_ms(ceilings, rd, wr)
+                v["floor_ms_at_stream_rates"] = round(floor, 4)
+                v["ms_over_floor"] = round(v["ms"] / floor, 3)
     dominant = max((k for k in kern if not k.startswith("copy") and "onepass" not in k), key=lambda k: kern[k]["ms"])
     # algorithmic bytes of the dominant kernel per launch: every row it moves, read once and written once
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": kern[dominant]["GBps"], "peak": HBM_PEAK_GBPS,
@@ -512,7 +669,8 @@ def main():
         "pack_plus_combine": r["pack_plus_combine"],
         "arrival_chain_us_per_row": stages["arrival"]["us_per_row"],
         "onepass": r["onepass"],
-        "stages": stages, "kernels": kern, "roofline": roofline,
+        "stages": stages, "in_step": r["in_step"], "kernels": kern, "ceilings": ceilings, "seam": seam,
+        "roofline": roofline,
         "stage_and_kernel_timing": f"each alone on the launch stream between HIP events: median of {EVENT_BATCHES} "
                                    f"batches of {max(args.steps, 5)} back-to-back launches",
         "library": os.path.relpath(st.lib, ROOT), "source_digest": digest,
@@ -534,6 +692,8 @@ def main():
                             "onepass_ms_per_step": o["onepass"]["ms_per_step"],
                             "onepass_frac_hbm_peak": o["onepass"]["frac_hbm_peak"],
                             "onepass_same_output": o["onepass"]["same_output_as_two_step"]}
+            if o.get("graph") is not None:
+                others[name]["hip_graph"] = o["graph"]
             del o
             torch.cuda.empty_cache()
         out["other_configs"] = others

@@ -86,6 +86,21 @@ TERRACE_API const char *terrace_strerror(int status);
  * terrace/ops/ascendc/op_kernel/terrace_passthrough.cpp:119). */
 TERRACE_API int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t stream);
 
+/* Stream probes beside terrace_passthrough: what the part sustains for the traffic mixes the row movers are made
+ * of, in the movers' own launch shape (one-wave workgroups, 16 bytes per lane, streaming loads and stores).  The
+ * benchmark times them in the run that times the movers, so every "this mover sits at its bytes' stream rate"
+ * statement can be checked from one record.  No counterpart in the reference beyond its passthrough toolchain
+ * probe (terrace/ops/ascendc/op_kernel/terrace_passthrough.cpp:119).
+ *   TERRACE_PROBE_READ   reads nbytes from x, writes nothing (y is only named by a store that never happens when x
+ *                        holds zeros)
+ *   TERRACE_PROBE_WRITE  writes nbytes to y
+ *   TERRACE_PROBE_SUM8   y = the fp32-accumulated sum of eight contiguous bf16 streams of nbytes each starting at x
+ *                        (reads 8 * nbytes): the combine's read:write mix and arithmetic with no row ids
+ *   TERRACE_PROBE_COPY   y = x, one wave per kilobyte
+ * nbytes must be a multiple of 8192 and both pointers 16-byte aligned, else TERRACE_EINVAL. */
+enum terrace_probe { TERRACE_PROBE_READ = 0, TERRACE_PROBE_WRITE = 1, TERRACE_PROBE_SUM8 = 2, TERRACE_PROBE_COPY = 3 };
+TERRACE_API int terrace_stream_probe(int kind, const void *x, void *y, size_t nbytes, terrace_stream_t stream);
+
 /* T-Route (terrace/routing.py:45-96).  affinity [T,E] f32, bias [E] f32, gate_affinity
  * [T,E] f32 or NULL (= affinity).  Writes expert_idx [T,k] i64, gates [T,k] f32 (bf16 / f16 with the mode flags),
  * group_idx [T,G] i64 with G = top_groups (full, group_limited), n_groups (quota_only) or
@@ -393,6 +408,57 @@ TERRACE_API int terrace_routing_map_topk(const void *routing_map, const void *pr
  * except send[n*rpn + my_local] = node_counts[n]. */
 TERRACE_API int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local,
                              int64_t *send, terrace_stream_t stream);
+
+/* ---- the whole dispatch in one call ----
+ * terrace_k2_pack, then terrace_k1_arrival and terrace_regroup on the rank's own send buffers (the exchanges of
+ * terrace/ta2a_fwd.py:471-646 looped back: every slot of the node counts as local, my_local = 0), or -- `onepass`
+ * -- terrace_hopb_scatter in place of those two.  Same kernels, same planes bit for bit; what it saves is host
+ * time: one call, one workspace, and the small planes addressed as offsets into ONE caller buffer, so a binding
+ * computes the table of offsets once per geometry and passes two pointers per step.
+ *   plane_offsets[TERRACE_DP_PLANES]: byte offset of each plane from `planes`, or -1 for a plane the caller does
+ *   not want.  Required: MASK, U_SRC, NODE_COUNTS, PLACE, TOKENS_PER_EXPERT, STATUS, STATUS_HOPB, GATE_ROWS when
+ *   gates is given, and in the two-step form GATE_PAIRS, R_IDX, SLOT_IDX, I_SEND, STATUS_REGROUP.  WHERE (the
+ *   combine's [T, k] place table, filled through the pairs' tags) needs PAIR_SRC.  Shapes and dtypes are those of
+ *   the same-named arguments of the three stage entry points; the three STATUS planes are 4 int32 each (pack;
+ *   arrival or one-pass Hop B; regroup).
+ *   capacity < 0: drop-less.  send_buf is not used with `onepass`.
+ *   workspace: terrace_dispatch_workspace(...) bytes (it also holds the tags carried between the two sorts). */
+enum terrace_dispatch_plane {
+    TERRACE_DP_MASK = 0,
+    TERRACE_DP_GATE_ROWS,
+    TERRACE_DP_U_SRC,
+    TERRACE_DP_NODE_COUNTS,
+    TERRACE_DP_U_NODE,
+    TERRACE_DP_INVERSE,
+    TERRACE_DP_NODE_OFFSETS,
+    TERRACE_DP_PAIR_TABLE,
+    TERRACE_DP_SORT_ORDER,
+    TERRACE_DP_TOKEN_ROWS,
+    TERRACE_DP_GATE_SORTED,
+    TERRACE_DP_PAIR_SRC,
+    TERRACE_DP_WHERE,
+    TERRACE_DP_STATUS,
+    TERRACE_DP_GATE_PAIRS,
+    TERRACE_DP_R_IDX,
+    TERRACE_DP_SLOT_IDX,
+    TERRACE_DP_I_SEND,
+    TERRACE_DP_PAIR_POS,
+    TERRACE_DP_STATUS_HOPB,
+    TERRACE_DP_ORDER,
+    TERRACE_DP_PLACE,
+    TERRACE_DP_KEPT,
+    TERRACE_DP_TOKENS_PER_EXPERT,
+    TERRACE_DP_KEPT_PER_EXPERT,
+    TERRACE_DP_STATUS_REGROUP,
+    TERRACE_DP_PLANES
+};
+TERRACE_API size_t terrace_dispatch_workspace(int64_t T, int k, int world, int n_experts, int rpn, int groups_m,
+                                              int64_t capacity, int onepass);
+TERRACE_API int terrace_dispatch(const void *x, const int64_t *expert_idx, const void *gates, int64_t T,
+                                 int64_t row_bytes, int gate_bytes, int k, int world, int n_experts, int rpn,
+                                 int groups_m, int64_t capacity, int onepass, void *payload, void *send_buf,
+                                 void *permuted, void *planes, const int64_t *plane_offsets, void *workspace,
+                                 size_t workspace_bytes, terrace_stream_t stream);
 
 /* ---- the entry point that brings its own scratch memory ----
  * No counterpart in the reference.  It is for callers that cannot allocate device memory at all -- code under

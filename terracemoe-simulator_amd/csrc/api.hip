@@ -3,6 +3,7 @@
 
 namespace terrace {
 int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
+int launch_stream_probe(int kind, const void *x, void *y, size_t nbytes, hipStream_t s);
 int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
                    int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
 int launch_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n, int64_t *out,
@@ -122,6 +123,10 @@ const char *terrace_strerror(int status) {
 int terrace_passthrough(const void *x, void *y, size_t nbytes, terrace_stream_t stream) {
     if (nbytes && (!x || !y)) return TERRACE_EINVAL;
     return launch_copy(x, y, nbytes, (hipStream_t)stream);
+}
+
+int terrace_stream_probe(int kind, const void *x, void *y, size_t nbytes, terrace_stream_t stream) {
+    return launch_stream_probe(kind, x, y, nbytes, (hipStream_t)stream);
 }
 
 int terrace_t_route(const float *affinity, const float *bias, const float *gate_affinity, int64_t T, int n_experts,
@@ -412,6 +417,95 @@ int terrace_routing_map_count(const void *routing_map, int64_t T, int n_experts,
 int terrace_routing_map_topk(const void *routing_map, const void *probs, int elem_bytes, int64_t T, int n_experts,
                              int k, int64_t *expert_idx, void *gates, terrace_stream_t stream) {
     return run_map_topk(routing_map, probs, elem_bytes, T, n_experts, k, expert_idx, gates, (hipStream_t)stream);
+}
+
+// ---- the whole dispatch in one call ----
+namespace {
+struct DispatchGeometry {
+    int64_t S, P;
+    int n_nodes, epr, slots, quota;
+    size_t ws_k2, ws_a, ws_r, ws_b, carried;
+};
+
+bool dispatch_geometry(int64_t T, int k, int world, int n_experts, int rpn, int groups_m, int64_t capacity,
+                       DispatchGeometry *g) {
+    if (T < 0 || k <= 0 || world <= 0 || rpn <= 0 || groups_m <= 0 || n_experts <= 0 || world % rpn ||
+        n_experts % world || k % groups_m)
+        return false;
+    if (T > (((int64_t)1 << 31) - 1) / k) return false;
+    g->S = T * groups_m;
+    g->P = T * k;
+    g->n_nodes = world / rpn;
+    g->epr = n_experts / world;
+    g->slots = g->epr * rpn;
+    g->quota = k / groups_m;
+    g->ws_k2 = align_up(k2_workspace(T, k, g->n_nodes, groups_m), 256);
+    g->ws_a = align_up(k1_workspace(g->S, g->quota, rpn), 256);
+    g->ws_r = align_up(regroup_workspace(g->P, g->slots, capacity), 256);
+    g->ws_b = align_up(hopb_workspace(g->S, g->quota, g->slots), 256);
+    g->carried = align_up((size_t)g->P * sizeof(int64_t), 256);
+    return true;
+}
+}  // namespace
+
+size_t terrace_dispatch_workspace(int64_t T, int k, int world, int n_experts, int rpn, int groups_m, int64_t capacity,
+                                  int onepass) {
+    DispatchGeometry g;
+    if (!dispatch_geometry(T, k, world, n_experts, rpn, groups_m, capacity, &g)) return 256;
+    return onepass ? g.ws_k2 + g.ws_b : g.ws_k2 + g.ws_a + g.ws_r + g.carried;
+}
+
+int terrace_dispatch(const void *x, const int64_t *expert_idx, const void *gates, int64_t T, int64_t row_bytes,
+                     int gate_bytes, int k, int world, int n_experts, int rpn, int groups_m, int64_t capacity,
+                     int onepass, void *payload, void *send_buf, void *permuted, void *planes,
+                     const int64_t *plane_offsets, void *workspace, size_t workspace_bytes, terrace_stream_t stream) {
+    DispatchGeometry g;
+    if (!dispatch_geometry(T, k, world, n_experts, rpn, groups_m, capacity, &g) || !plane_offsets) return TERRACE_EINVAL;
+    if (workspace_bytes < terrace_dispatch_workspace(T, k, world, n_experts, rpn, groups_m, capacity, onepass))
+        return TERRACE_ENOSPC;
+    if (!workspace || !planes) return TERRACE_EINVAL;
+    auto at = [&](int which) -> void * {
+        const int64_t off = plane_offsets[which];
+        return off < 0 ? nullptr : (void *)((char *)planes + off);
+    };
+    int32_t *status = (int32_t *)at(TERRACE_DP_STATUS), *status_b = (int32_t *)at(TERRACE_DP_STATUS_HOPB);
+    int32_t *status_r = (int32_t *)at(TERRACE_DP_STATUS_REGROUP);
+    int64_t *pair_src = (int64_t *)at(TERRACE_DP_PAIR_SRC), *where = (int64_t *)at(TERRACE_DP_WHERE);
+    if (!status || !status_b || (!onepass && !status_r) || !at(TERRACE_DP_PLACE) || !at(TERRACE_DP_TOKENS_PER_EXPERT) || (where && !pair_src))
+        return TERRACE_EINVAL;
+    if (!onepass && (!at(TERRACE_DP_GATE_PAIRS) || !at(TERRACE_DP_R_IDX) || !at(TERRACE_DP_SLOT_IDX) ||
+                     !at(TERRACE_DP_I_SEND)))
+        return TERRACE_EINVAL;
+    char *ws = (char *)workspace;
+    hipStream_t s = (hipStream_t)stream;
+    int rc = run_k2_pack(x, expert_idx, gates, T, row_bytes, gate_bytes, k, world, n_experts, rpn, groups_m, payload,
+                         (int64_t *)at(TERRACE_DP_MASK), at(TERRACE_DP_GATE_ROWS), (int64_t *)at(TERRACE_DP_U_SRC),
+                         (int64_t *)at(TERRACE_DP_NODE_COUNTS), (int64_t *)at(TERRACE_DP_U_NODE),
+                         (int64_t *)at(TERRACE_DP_INVERSE), (int64_t *)at(TERRACE_DP_NODE_OFFSETS),
+                         (int64_t *)at(TERRACE_DP_PAIR_TABLE), (int64_t *)at(TERRACE_DP_SORT_ORDER),
+                         (int64_t *)at(TERRACE_DP_TOKEN_ROWS), at(TERRACE_DP_GATE_SORTED), pair_src, where, status,
+                         ws, g.ws_k2, 0, 0, 0, s);
+    if (rc != TERRACE_OK) return rc;
+    const int64_t n_tags = where ? g.P : 0;
+    if (onepass)
+        return run_hopb_scatter(payload, (const int64_t *)at(TERRACE_DP_MASK), nullptr, g.S, row_bytes, gate_bytes,
+                                g.quota, 0, g.slots, capacity, permuted, nullptr, (int64_t *)at(TERRACE_DP_PLACE),
+                                (uint8_t *)at(TERRACE_DP_KEPT), nullptr, (int64_t *)at(TERRACE_DP_TOKENS_PER_EXPERT),
+                                (int64_t *)at(TERRACE_DP_KEPT_PER_EXPERT), where ? pair_src : nullptr, where, n_tags,
+                                status_b, ws + g.ws_k2, g.ws_b, s);
+    int64_t *carried = where ? (int64_t *)(ws + g.ws_k2 + g.ws_a + g.ws_r) : nullptr;
+    rc = run_k1_arrival(payload, (const int64_t *)at(TERRACE_DP_MASK), at(TERRACE_DP_GATE_ROWS), g.S, row_bytes,
+                        gate_bytes, g.quota, g.epr, rpn, 0, send_buf, at(TERRACE_DP_GATE_PAIRS),
+                        (int64_t *)at(TERRACE_DP_R_IDX), (int64_t *)at(TERRACE_DP_SLOT_IDX),
+                        (int64_t *)at(TERRACE_DP_I_SEND), (int64_t *)at(TERRACE_DP_PAIR_POS),
+                        status_b, ws + g.ws_k2, g.ws_a, g.quota, g.quota, nullptr,
+                        where ? pair_src : nullptr, carried, s);
+    if (rc != TERRACE_OK) return rc;
+    return run_regroup(send_buf, (const int64_t *)at(TERRACE_DP_SLOT_IDX), nullptr, g.P, row_bytes, gate_bytes,
+                       g.slots, 0, capacity, permuted, nullptr, (int64_t *)at(TERRACE_DP_ORDER),
+                       (int64_t *)at(TERRACE_DP_PLACE), (uint8_t *)at(TERRACE_DP_KEPT),
+                       (int64_t *)at(TERRACE_DP_TOKENS_PER_EXPERT), (int64_t *)at(TERRACE_DP_KEPT_PER_EXPERT),
+                       status_r, ws + g.ws_k2 + g.ws_a, g.ws_r, 1, 1, carried, where, n_tags, s);
 }
 
 int terrace_hopa_send_splits(const int64_t *node_counts, int world, int rpn, int my_local, int64_t *send,

@@ -49,6 +49,89 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// stream probes: what this part sustains for the traffic mixes the row movers are made of, measured
+// with the movers' own launch shape (one-wave workgroups, one 16-byte vector per lane, streaming
+// loads and stores).  They carry no result anybody uses; the benchmark times them beside the movers.
+// ---------------------------------------------------------------------------------------------
+// read only: a wave reads eight kilobytes, one from each eighth of the source (one kilobyte per one-wave workgroup
+// would measure the rate workgroups can be launched at, not the memory); what is read decides a store that never
+// happens for the data the benchmark feeds (all-zero words), so the loads cannot be dropped
+__global__ __launch_bounds__(kWave) void probe_read_kernel(const u32x4 *__restrict__ x, u32x4 *__restrict__ y,
+                                                           int64_t eighth_vecs) {
+    const int64_t g = (int64_t)blockIdx.x * kWave + threadIdx.x;
+    u32x4 v = ld_stream(x + g);
+#pragma unroll
+    for (int j = 1; j < 8; ++j) v ^= ld_stream(x + j * eighth_vecs + g);
+    if (v[0] == 0x7E57AB1Eu && v[3] == 0x5EED5EEDu) st_stream(y + g, v);
+}
+
+// write only: one aligned 4 KB block per 256-lane workgroup (the fastest pure-write shape on this part)
+__global__ __launch_bounds__(kBlock) void probe_write_kernel(u32x4 *__restrict__ y) {
+    const int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    st_stream(y + g, u32x4{(uint32_t)g, 1u, 2u, 3u});
+}
+
+// eight contiguous streams of bf16 summed into one in fp32: the combine's 8:1 read:write mix and its
+// arithmetic with no row ids and no table
+__global__ __launch_bounds__(kWave) void probe_sum8_kernel(const u32x4 *__restrict__ x, u32x4 *__restrict__ y,
+                                                           int64_t n_vecs) {
+    const int64_t g = (int64_t)blockIdx.x * kWave + threadIdx.x;
+    u32x4 raw[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) raw[j] = ld_stream(x + j * n_vecs + g);
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i] = __fadd_rn(acc[2 * i], __fmul_rn(__uint_as_float(raw[j][i] << 16), 0.125f));
+            acc[2 * i + 1] = __fadd_rn(acc[2 * i + 1], __fmul_rn(__uint_as_float(raw[j][i] & 0xFFFF0000u), 0.125f));
+        }
+    }
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (f32_to_bf16_bits(acc[2 * i]) & 0xFFFFu) | (f32_to_bf16_bits(acc[2 * i + 1]) << 16);
+    st_stream(y + g, o);
+}
+
+// copy in the movers' shape: one wave per kilobyte
+__global__ __launch_bounds__(kWave) void probe_copy_kernel(const u32x4 *__restrict__ x, u32x4 *__restrict__ y) {
+    const int64_t g = (int64_t)blockIdx.x * kWave + threadIdx.x;
+    st_stream(y + g, ld_stream(x + g));
+}
+
+// `nbytes` is what the probe writes (reads, for the read-only one): a positive multiple of 8192, both
+// pointers 16-byte aligned; the 8:1 sum reads 8 * nbytes from `x`.
+int launch_stream_probe(int kind, const void *x, void *y, size_t nbytes, hipStream_t s) {
+    if (nbytes == 0) return TERRACE_OK;
+    if (nbytes % 8192 || (((uintptr_t)x | (uintptr_t)y) & 15) || !y) return TERRACE_EINVAL;
+    const int64_t vecs = (int64_t)(nbytes / 16);
+    if (vecs / kWave > ((int64_t)1 << 31) - 1) return TERRACE_EINVAL;
+    const unsigned waves = (unsigned)(vecs / kWave);
+    switch (kind) {
+        case TERRACE_PROBE_READ:
+            if (!x) return TERRACE_EINVAL;
+            probe_read_kernel<<<waves / 8, kWave, 0, s>>>((const u32x4 *)x, (u32x4 *)y, vecs / 8);
+            break;
+        case TERRACE_PROBE_WRITE:
+            probe_write_kernel<<<(unsigned)(vecs / kBlock), kBlock, 0, s>>>((u32x4 *)y);
+            break;
+        case TERRACE_PROBE_SUM8:
+            if (!x) return TERRACE_EINVAL;
+            probe_sum8_kernel<<<waves, kWave, 0, s>>>((const u32x4 *)x, (u32x4 *)y, vecs);
+            break;
+        case TERRACE_PROBE_COPY:
+            if (!x) return TERRACE_EINVAL;
+            probe_copy_kernel<<<waves, kWave, 0, s>>>((const u32x4 *)x, (u32x4 *)y);
+            break;
+        default: return TERRACE_EINVAL;
+    }
+    return check_launch();
+}
+
 // Row ids a caller hands in are never trusted with an address: an id is used only if it lies in [0, bound),
 // which one unsigned compare decides ((uint64_t)id < (uint64_t)bound is false for negative ids too).  An id
 // outside is a dead entry -- a zero row for a gather, no contribution for the combine, a copy not made for a

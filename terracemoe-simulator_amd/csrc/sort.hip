@@ -704,9 +704,9 @@ struct EmitHopB {            // arrival + expert-order regroup in one placement 
 };
 
 // The places of a capacity layout that hold no row: zero rows, zero gates, no pair.  blockIdx.x = x * chunks + c
-// looks after places [c * kPadRows, (c + 1) * kPadRows) of expert x and leaves at once when they are all in use;
+// looks after places [c * pad_rows, (c + 1) * pad_rows) of expert x and leaves at once when they are all in use;
 // the first workgroup of an expert also writes kept_per_expert.
-constexpr int kPadRows = 16;
+constexpr int kPadRows = 16;             // the most places one workgroup looks after (the launcher picks pad_rows)
 template <typename V>
 __global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restrict__ start, int epr, int64_t capacity,
                                                           int chunks, int pad_rows, V *__restrict__ rows, int64_t row_vecs,
@@ -1216,9 +1216,14 @@ static int launch_zero_pad(const int32_t *start, int epr, int64_t capacity, void
                            void *gate_plane, int gate_bytes, int64_t *pair_of_place, int64_t *kept_per_expert,
                            hipStream_t s) {
     if (epr <= 0) return TERRACE_OK;
-    // kPadRows places per workgroup; more where that many workgroups would pass what one launch can hold
-    // (blocks * kBlock has to stay below 2^32)
+    // places per workgroup: about 16 KB of rows (a shorter run of padding per workgroup measured faster -- the
+    // one-pass Hop B of the 4 KB-row capacity workload went 0.673 -> 0.658 ms from 16 places to 4 -- until the
+    // workgroups that find nothing to do, which still have to be launched, outweigh it), at most kPadRows; more
+    // where that many workgroups would pass what one launch can hold (blocks * kBlock has to stay below 2^32)
     int pad_rows = kPadRows;
+    if (rows && row_bytes > 0) {
+        while (pad_rows > 1 && (int64_t)pad_rows * row_bytes > 16384) pad_rows /= 2;
+    }
     while ((int64_t)epr * ((capacity + pad_rows - 1) / pad_rows) > (int64_t)1 << 22) pad_rows *= 2;
     const int chunks = capacity > 0 ? (int)((capacity + pad_rows - 1) / pad_rows) : 1;
     const int64_t blocks = (int64_t)epr * chunks;

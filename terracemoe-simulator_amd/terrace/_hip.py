@@ -22,7 +22,13 @@ F32, BF16, F16, FP8_B128 = 0, 1, 2, 3
 MODE_CODES = {"full": 0, "group_limited": 1, "quota_only": 2, "global_topk": 3}
 FORCE_GENERIC = 0x100
 GATES_FLAG = {torch.float32: 0, torch.bfloat16: 0x200, torch.float16: 0x400}
+PROBE_READ, PROBE_WRITE, PROBE_SUM8, PROBE_COPY = 0, 1, 2, 3
 FAULT_ID_RANGE, FAULT_QUOTA, FAULT_FANOUT = 1, 2, 4
+# enum terrace_dispatch_plane, in order
+DISPATCH_PLANES = ("mask", "gate_rows", "u_src", "node_counts", "u_node", "inverse", "node_offsets", "pair_table",
+                   "sort_order", "token_rows", "gate_sorted", "pair_src", "where", "status", "gate_pairs", "r_idx",
+                   "slot_idx", "i_send", "pair_pos", "status_hopb", "order", "place", "kept", "tokens_per_expert",
+                   "kept_per_expert", "status_regroup")
 STATUS_WORDS = 4
 
 _P, _I, _L, _Z = c_void_p, c_int, c_int64, c_size_t
@@ -32,6 +38,7 @@ SIGNATURES = {
     "terrace_version": (c_char_p, []),
     "terrace_strerror": (c_char_p, [_I]),
     "terrace_passthrough": (_I, [_P, _P, _Z, _P]),
+    "terrace_stream_probe": (_I, [_I, _P, _P, _Z, _P]),
     "terrace_t_route": (_I, [_P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P]),
     "terrace_hist_workspace": (_Z, [_L, _I]),
     "terrace_hist": (_I, [_P, _L, _I, _P, _I, _P, _P, _Z, _P]),
@@ -83,6 +90,8 @@ SIGNATURES = {
     "terrace_routing_map_count": (_I, [_P, _L, _I, _P, _P]),
     "terrace_routing_map_topk": (_I, [_P, _P, _I, _L, _I, _I, _P, _P, _P]),
     "terrace_hopa_send_splits": (_I, [_P, _I, _I, _I, _P, _P]),
+    "terrace_dispatch_workspace": (_Z, [_L, _I, _I, _I, _I, _I, _L, _I]),
+    "terrace_dispatch": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I, _L, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "terrace_static_scratch_bytes": (_Z, []),
     "terrace_static_init": (_I, []),
     "terrace_k1_arrival_static": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I,

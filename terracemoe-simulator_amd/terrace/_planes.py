@@ -22,11 +22,11 @@ _LAZY = object()          # placeholder of a plane nobody has read yet
 
 class Layout:
     """Where each named plane sits in the slab: name -> (offset, shape, dtype, nbytes)."""
-    __slots__ = ("at", "total")
+    __slots__ = ("at", "total", "offsets")
 
     def __init__(self, planes):
         """planes: iterable of (name, shape, dtype); a None shape leaves the name out."""
-        self.at, self.total = {}, 0
+        self.at, self.total, self.offsets = {}, 0, None
         for name, shape, dtype in planes:
             if shape is None:
                 continue

@@ -1038,6 +1038,22 @@ def passthrough(x: torch.Tensor) -> torch.Tensor:
     return TerracePassthroughFn.apply(x)
 
 
+def stream_probe(kind: str, x, y):
+    """One launch of a stream probe (``read`` | ``write`` | ``sum8`` | ``copy``): ``y``'s byte size is what the
+    probe writes (reads, for ``read``); ``sum8`` reads eight times that from ``x``.  Returns ``y``."""
+    _require()
+    _hip.need_device(x, y)
+    code = {"read": _hip.PROBE_READ, "write": _hip.PROBE_WRITE, "sum8": _hip.PROBE_SUM8, "copy": _hip.PROBE_COPY}[kind]
+    nbytes = y.numel() * y.element_size()
+    need = {"read": nbytes, "write": 0, "sum8": 8 * nbytes, "copy": nbytes}[kind]
+    if not y.is_contiguous() or (x is not None and (not x.is_contiguous() or x.numel() * x.element_size() < need)):
+        raise RuntimeError("stream_probe: contiguous tensors, and a source at least as large as the probe reads")
+    if x is None and need:
+        raise RuntimeError(f"stream_probe: {kind} needs a source")
+    _hip.call("terrace_stream_probe", code, _hip.ptr(x), _hip.ptr(y), nbytes, _hip.stream(y.device))
+    return y
+
+
 def _k1_grad_rx(g_send, pair_pos, rx_shape, quota):
     """Adjoint of ``send_buf = rx[r_idx]``: row r sums its quota pairs, in pair order."""
     return combine(g_send, pair_pos.view(rx_shape[0], quota), None, out_dtype=g_send.dtype)

@@ -11,6 +11,7 @@ the balanced size) and every expert slot of the node treated as local.
 from __future__ import annotations
 
 import os
+from ctypes import c_int64, c_void_p
 
 import torch
 
@@ -208,14 +209,27 @@ def loopback_dispatch_onepass(x, expert_idx, gates, world: int, n_experts: int, 
 
 _DISPATCH_LAYOUTS: dict = {}
 
+# slab names of the planes terrace_dispatch addresses, in the order of enum terrace_dispatch_plane
+_SLAB_NAME = {"u_node": "x.u_node", "inverse": "x.inverse", "node_offsets": "x.node_offsets",
+              "pair_table": "x.pair_table", "sort_order": "x.sort_order", "token_rows": "x.token_rows",
+              "gate_sorted": "x.gate_sorted", "pair_src": "x.pair_src", "where": "x.where", "status": "x.status",
+              "status_hopb": "_status_b", "status_regroup": "_status_r", "order": "_order",
+              "kept_per_expert": "x.kept_per_expert"}
 
-def _dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass):
-    """The slab arrangement of a dispatch's small planes (cached per geometry).  Names: state fields as they are,
-    ``x.<key>`` the entries of ``extras``, ``_<name>`` scratch nobody reads."""
-    key = (T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass)
+
+def _align256(n):
+    return (int(n) + 255) // 256 * 256
+
+
+def _dispatch_layout(T, k, world, n_experts, rpn, groups_m, capacity, gdt, onepass):
+    """The slab arrangement of a dispatch's small planes (cached per geometry) and, as ``lay.offsets``, the table
+    of plane offsets ``terrace_dispatch`` takes.  Names: state fields as they are, ``x.<key>`` the entries of
+    ``extras``, ``_<name>`` scratch nobody reads."""
+    key = (T, k, world, n_experts, rpn, groups_m, capacity, gdt, onepass)
     lay = _DISPATCH_LAYOUTS.get(key)
     if lay is not None:
         return lay
+    n_nodes, slots = world // rpn, (n_experts // world) * rpn
     S, P, quota = T * groups_m, T * k, k // groups_m
     cap = -1 if capacity is None else int(capacity)
     i64, i32, u8 = torch.int64, torch.int32, torch.uint8
@@ -225,27 +239,26 @@ def _dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gdt, onepass
               ("x.u_node", (S,), i64), ("x.inverse", (P,), i64), ("x.node_offsets", (n_nodes,), i64),
               ("x.pair_table", (T, k), i64), ("x.sort_order", (T, k), i64), ("x.token_rows", (T, groups_m), i64),
               ("x.gate_sorted", (T, k), gdt), ("x.pair_src", (P,), i64), ("x.where", (T, k), i64),
-              ("x.status", (4,), i32), ("x.kept_per_expert", (slots,), i64),
-              ("_ws_k2", (_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m),), u8)]
-    if onepass:
-        planes += [("_status_b", (4,), i32),
-                   ("_ws_b", (_hip.query("terrace_hopb_scatter_workspace", S, quota, slots),), u8)]
-    else:
+              ("x.status", (4,), i32), ("x.kept_per_expert", (slots,), i64), ("_status_b", (4,), i32),
+              ("_ws", (_hip.query("terrace_dispatch_workspace", T, k, world, n_experts, rpn, groups_m, cap,
+                                  1 if onepass else 0),), u8)]
+    if not onepass:
         planes += [("gate_pairs", (P,), gdt), ("r_idx", (P,), i64), ("slot_idx", (P,), i64), ("i_send", (rpn,), i64),
-                   ("pair_pos", (P,), i64), ("_carried", (P,), i64), ("_status_a", (4,), i32), ("_status_r", (4,), i32),
-                   ("_order", (P,) if capacity is None else None, i64),
-                   ("_ws_a", (_hip.query("terrace_k1_arrival_workspace", S, quota, rpn),), u8),
-                   ("_ws_r", (_hip.query("terrace_regroup_workspace", P, slots, cap),), u8)]
+                   ("pair_pos", (P,), i64), ("_status_r", (4,), i32), ("_order", (P,) if capacity is None else None, i64)]
     if len(_DISPATCH_LAYOUTS) > 64:
         _DISPATCH_LAYOUTS.clear()
     lay = _DISPATCH_LAYOUTS[key] = _planes.Layout(planes)
+    lay.offsets = (c_int64 * len(_hip.DISPATCH_PLANES))(
+        *[lay.at[n][0] if n in lay.at else -1 for n in (_SLAB_NAME.get(p, p) for p in _hip.DISPATCH_PLANES)])
     return lay
 
 
-def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity, onepass):
-    """Stages 2-4 through the C ABI with every small plane in one allocation (three library calls, or two with
-    Hop B as one pass).  The combine's [T, k] place table is filled on the way: every Hop-A pair carries the entry
-    it answers (pair_src) through the sorts, and the last one writes the pair's place there."""
+def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, capacity, onepass, stagewise=False):
+    """Stages 2-4 through the C ABI with every small plane in one allocation: one library call
+    (``terrace_dispatch``), or -- ``stagewise`` -- the three stage entry points one after the other (two with Hop B
+    as one pass), which launch the same kernels on the same planes.  The combine's [T, k] place table is filled on
+    the way: every Hop-A pair carries the entry it answers (pair_src) through the sorts, and the last one writes
+    the pair's place there."""
     _ops._require()
     _hip.need_device(x, expert_idx, gates)
     _ops._check_k2(x, expert_idx, gates, world, n_experts, rpn, groups_m)
@@ -259,39 +272,50 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
     cap = -1 if capacity is None else int(capacity)
     places = P if capacity is None else slots * cap
     row_bytes, gb = H * x.element_size(), gates.element_size()
-    slab = _planes.Slab(_dispatch_layout(T, k, groups_m, n_nodes, rpn, slots, capacity, gates.dtype, onepass), dev)
+    lay = _dispatch_layout(T, k, world, n_experts, rpn, groups_m, capacity, gates.dtype, onepass)
+    slab = _planes.Slab(lay, dev)
     payload = torch.empty((S, H), dtype=x.dtype, device=dev)
     permuted = torch.empty((places, H), dtype=x.dtype, device=dev)
+    send_buf = None if onepass else torch.empty((P, H), dtype=x.dtype, device=dev)
     ptr, at, stream = _hip.ptr, slab.ptr, _hip.stream(dev)
-    _hip.call("terrace_k2_pack", ptr(x), ptr(expert_idx), ptr(gates), T, row_bytes, gb, k, world, n_experts, rpn,
-              groups_m, ptr(payload), at("mask"), at("gate_rows"), at("u_src"), at("node_counts"), at("x.u_node"),
-              at("x.inverse"), at("x.node_offsets"), at("x.pair_table"), at("x.sort_order"), at("x.token_rows"),
-              at("x.gate_sorted"), at("x.pair_src"), at("x.where"), at("x.status"), at("_ws_k2"), slab.nbytes("_ws_k2"),
-              stream)
-    extras = _planes.LazyDict(slab, "x.")
     # the plan's guard (terrace/ta2a.py:161-204 of the reference): the status words are read back on the first
-    # dispatch of a shape and on every 256th, after the last launch below so the read-back waits for nothing extra
+    # dispatch of a shape and on every 256th, after the last launch so the read-back waits for nothing extra
     from . import ta2a as _plan
     guard_key = (T, k, n_nodes, groups_m)
     guard = _plan._guard_due(guard_key)
-    if onepass:
-        _hip.call("terrace_hopb_scatter", ptr(payload), at("mask"), None, S, row_bytes, gb, quota, 0, slots, cap,
-                  ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"), at("x.kept_per_expert"),
-                  at("x.pair_src"), at("x.where"), P, at("_status_b"), at("_ws_b"), slab.nbytes("_ws_b"), stream)
-        if guard:
-            _plan._raise_from_status(extras["status"], T, k, groups_m)
-            _plan._VERIFIED.add(guard_key)
-        return OnePassState(slab, ("kept",), payload=payload, permuted=permuted, extras=extras, capacity=capacity)
-    send_buf = torch.empty((P, H), dtype=x.dtype, device=dev)
-    _hip.call("terrace_k1_arrival", ptr(payload), at("mask"), at("gate_rows"), S, row_bytes, gb, quota, epr, rpn, 0,
-              ptr(send_buf), at("gate_pairs"), at("r_idx"), at("slot_idx"), at("i_send"), at("pair_pos"),
-              at("x.pair_src"), at("_carried"), at("_status_a"), at("_ws_a"), slab.nbytes("_ws_a"), stream)
-    _hip.call("terrace_regroup", ptr(send_buf), at("slot_idx"), None, P, row_bytes, gb, slots, 0, cap, ptr(permuted),
-              None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"), at("x.kept_per_expert"),
-              at("_carried"), at("x.where"), P, at("_status_r"), at("_ws_r"), slab.nbytes("_ws_r"), stream)
+    if not stagewise:
+        _hip.call("terrace_dispatch", ptr(x), ptr(expert_idx), ptr(gates), T, row_bytes, gb, k, world, n_experts, rpn,
+                  groups_m, cap, 1 if onepass else 0, ptr(payload), ptr(send_buf), ptr(permuted), c_void_p(slab.base),
+                  lay.offsets, at("_ws"), slab.nbytes("_ws"), stream)
+    else:
+        ws = slab.base + lay.at["_ws"][0]
+        n_k2 = _align256(_hip.query("terrace_k2_pack_workspace", T, k, n_nodes, groups_m))
+        _hip.call("terrace_k2_pack", ptr(x), ptr(expert_idx), ptr(gates), T, row_bytes, gb, k, world, n_experts, rpn,
+                  groups_m, ptr(payload), at("mask"), at("gate_rows"), at("u_src"), at("node_counts"), at("x.u_node"),
+                  at("x.inverse"), at("x.node_offsets"), at("x.pair_table"), at("x.sort_order"), at("x.token_rows"),
+                  at("x.gate_sorted"), at("x.pair_src"), at("x.where"), at("x.status"), c_void_p(ws), n_k2, stream)
+        if onepass:
+            _hip.call("terrace_hopb_scatter", ptr(payload), at("mask"), None, S, row_bytes, gb, quota, 0, slots, cap,
+                      ptr(permuted), None, at("place"), at("kept"), None, at("tokens_per_expert"),
+                      at("x.kept_per_expert"), at("x.pair_src"), at("x.where"), P, at("_status_b"), c_void_p(ws + n_k2),
+                      slab.nbytes("_ws") - n_k2, stream)
+        else:
+            n_a = _align256(_hip.query("terrace_k1_arrival_workspace", S, quota, rpn))
+            n_r = _align256(_hip.query("terrace_regroup_workspace", P, slots, cap))
+            carried = c_void_p(ws + n_k2 + n_a + n_r)
+            _hip.call("terrace_k1_arrival", ptr(payload), at("mask"), at("gate_rows"), S, row_bytes, gb, quota, epr,
+                      rpn, 0, ptr(send_buf), at("gate_pairs"), at("r_idx"), at("slot_idx"), at("i_send"),
+                      at("pair_pos"), at("x.pair_src"), carried, at("_status_b"), c_void_p(ws + n_k2), n_a, stream)
+            _hip.call("terrace_regroup", ptr(send_buf), at("slot_idx"), None, P, row_bytes, gb, slots, 0, cap,
+                      ptr(permuted), None, at("_order"), at("place"), at("kept"), at("tokens_per_expert"),
+                      at("x.kept_per_expert"), carried, at("x.where"), P, at("_status_r"), c_void_p(ws + n_k2 + n_a),
+                      n_r, stream)
+    extras = _planes.LazyDict(slab, "x.")
     if guard:
         _plan._raise_from_status(extras["status"], T, k, groups_m)
         _plan._VERIFIED.add(guard_key)
+    if onepass:
+        return OnePassState(slab, ("kept",), payload=payload, permuted=permuted, extras=extras, capacity=capacity)
     return LoopbackState(slab, ("kept",), payload=payload, send_buf=send_buf, permuted=permuted, extras=extras,
                          capacity=capacity)
 

@@ -69,6 +69,34 @@ def test_passthrough_is_a_bitwise_copy(shape, dtype):
     assert torch.equal(torch.ops.terrace.passthrough(xd).cpu(), x)
 
 
+def test_stream_probes_do_what_they_are_priced_for():
+    """The benchmark prices the probes by the bytes they are said to move: the copy must copy, the 8:1 sum must be
+    the fp32 sum of eight bf16 streams scaled by 1/8 and rounded once, the write probe must write every vector and
+    the read probe must leave its destination alone."""
+    import terrace.ops as tops
+    announce("stream probes")
+    n = 1 << 20                                            # bytes written
+    g = torch.Generator().manual_seed(3)
+    src = torch.randn(8 * n // 2, generator=g).to(torch.bfloat16).to(DEV)
+    out = torch.full((n // 2,), 7.0, dtype=torch.bfloat16, device=DEV)
+    tops.stream_probe("copy", src, out)
+    assert torch.equal(out.view(torch.int16), src[: n // 2].view(torch.int16))
+    tops.stream_probe("sum8", src, out)
+    parts = src.view(8, n // 2).float()
+    acc = torch.zeros(n // 2, device=DEV)
+    for j in range(8):
+        acc = acc + parts[j] * 0.125
+    assert torch.equal(out.view(torch.int16), acc.to(torch.bfloat16).view(torch.int16))
+    out.fill_(7.0)
+    tops.stream_probe("read", torch.zeros(n, dtype=torch.uint8, device=DEV), out.view(torch.uint8))
+    assert bool((out == 7.0).all())
+    tops.stream_probe("write", None, out)
+    words = out.view(torch.int32).view(-1, 4).cpu()
+    assert torch.equal(words[:, 0], torch.arange(n // 16, dtype=torch.int32)) and bool((words[:, 1:] == torch.tensor([1, 2, 3])).all())
+    with pytest.raises(RuntimeError):
+        tops.stream_probe("copy", src, out[:1000])          # not a multiple of 8192 bytes
+
+
 # ------------------------------------------------------------------------------- routing
 
 ROUTE_GEOMS = [  # (T, E, N_g, k, M)
@@ -458,6 +486,38 @@ def test_malformed_routing_is_contained_and_counted():
         assert torch.equal(payload.cpu()[rows_of_clean.reshape(-1)], x.cpu()[clean].repeat_interleave(M, 0))
 
 
+@pytest.mark.parametrize("onepass", [False, True])
+def test_one_call_dispatch_equals_the_stage_calls(onepass):
+    """terrace_dispatch against terrace_k2_pack + terrace_k1_arrival + terrace_regroup (or terrace_hopb_scatter) called
+    one after the other: every plane and every row buffer bit for bit, with and without a capacity, on the
+    lane-per-token send side and on the item kernels, and on an empty batch."""
+    from terrace import ta2a_fwd
+    announce("dispatch one call", onepass)
+    cases = [(64, 8, 256, 1000, 8, 4, 48, torch.bfloat16, None), (64, 8, 256, 1000, 8, 4, 48, torch.bfloat16, 30),
+             (64, 8, 64, 777, 4, 2, 33, torch.float32, None), (8, 2, 64, 90, 24, 4, 16, torch.float16, 20),
+             (160, 2, 160, 50, 4, 2, 8, torch.float32, None), (64, 8, 256, 0, 8, 4, 48, torch.bfloat16, None)]
+    for world, rpn, E, T, k, M, H, dtype, cap in cases:
+        n_nodes = world // rpn
+        g = torch.Generator().manual_seed(T + k)
+        e = torch.from_numpy(equal_quota_routing(T, k, E, n_nodes, M, 3, False)).reshape(T, k).to(DEV)
+        x = torch.randn(T, H, generator=g).to(dtype).to(DEV)
+        gts = torch.rand(T, k, generator=g).to(dtype).to(DEV)
+        a = ta2a_fwd._dispatch_one_slab(x, e, gts, world, E, rpn, M, cap, onepass)
+        b = ta2a_fwd._dispatch_one_slab(x, e, gts, world, E, rpn, M, cap, onepass, stagewise=True)
+        torch.cuda.synchronize()
+        names = [n for n in a._slab.layout.at if not n.startswith("_")]
+        assert names and set(names) == {n for n in b._slab.layout.at if not n.startswith("_")}
+        for n in names:
+            ta, tb = a._slab.tensor(n), b._slab.tensor(n)
+            if n in ("x.status",):
+                assert ta.tolist()[:3] == tb.tolist()[:3], n
+                continue
+            assert torch.equal(ta.view(torch.uint8) if ta.is_floating_point() else ta,
+                               tb.view(torch.uint8) if tb.is_floating_point() else tb), (n, T, k, cap)
+        for n in ("payload", "permuted") + (() if onepass else ("send_buf",)):
+            assert torch.equal(getattr(a, n).view(torch.uint8), getattr(b, n).view(torch.uint8)), n
+
+
 def _poison_next_allocation(nbytes):
     """Leaves a freed block of ``nbytes`` full of 0x5A bytes at the head of torch's cache, so that the next
     allocation of that size starts from garbage that reads as huge positive ids."""
@@ -486,7 +546,7 @@ def test_malformed_routing_through_the_whole_dispatch(onepass):
         e[7, :q + 1] = e[7, 0] // slots * slots + torch.arange(q + 1) % slots   # q + 1 experts on one node
         x = torch.randn(T, 32, generator=g).to(DEV)
         gts = torch.rand(T, k, generator=g).to(DEV)
-        lay = ta2a_fwd._dispatch_layout(T, k, M, n_nodes, rpn, slots, None, gts.dtype, onepass)
+        lay = ta2a_fwd._dispatch_layout(T, k, world, E, rpn, M, None, gts.dtype, onepass)
         dispatch = ta2a_fwd.loopback_dispatch_onepass if onepass else ta2a_fwd.loopback_dispatch
         # the first dispatch of a shape reads the guard's census back and raises on such a routing; later ones
         # (up to the 256th) run unchecked, which is the case that has to be contained
