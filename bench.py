@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--no-seam", action="store_true", help="skip the ta2a_permute / ta2a_unpermute timings")
+    ap.add_argument("--row-pitch", type=int, default=None,
+                    help="bytes between payload rows in every row buffer of --config (0: rows back to back; default: "
+                         "what the workload names)")
     ap.add_argument("--graph", action="store_true",
                     help="also capture the step into a HIP graph and time its replays (reported beside the eager "
                          "figure, which stays `value`)")
@@ -162,7 +165,7 @@ def torch_chain_baseline(cfg, sample_tokens, threads):
     from terrace import configs
     small = cfg.scaled(min(sample_tokens, cfg.T))
     inp = configs.make_inputs(small)
-    x = inp["x"]
+    x = inp["x"].contiguous()           # the CPU chain moves packed rows
     if small.fmt == "fp8":          # the rows travel as bytes; the expert output is dequantised where the combine reads it
         h = small.hidden
 
@@ -209,7 +212,7 @@ def openmp_port_baseline(cfg):
     elif cfg.fmt == "bf16":
         x, gcast, fmt = inp["x"].view(torch.int16).numpy().view(np.uint16), orc.f32_to_bf16, "bf16"
     else:
-        x, gcast, fmt = inp["x"].numpy(), orc.f32_to_bf16, "fp8"
+        x, gcast, fmt = inp["x"].contiguous().numpy(), orc.f32_to_bf16, "fp8"
     passes, began = [], time.perf_counter()
     while len(passes) < 3 or (len(passes) < 12 and time.perf_counter() - began < 6.0):
         passes.append(_openmp_pass(corc, np, cfg, logits, bias, ga, x, gcast, fmt))
@@ -412,7 +415,7 @@ def run_workload(cfg, args, torch, detail):
 
     dev = torch.device("cuda:0")
     inp = configs.make_inputs(cfg)
-    logits, bias, x = inp["logits"].to(dev), inp["bias"].to(dev), inp["x"].to(dev)
+    logits, bias, x = inp["logits"].to(dev), inp["bias"].to(dev), configs.rows_to(inp["x"], dev)
     gate_aff = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(dev)
     rcfg = terrace.TRouteConfig(cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups)
     cap = cfg.capacity(cfg.slots)
@@ -427,7 +430,8 @@ def run_workload(cfg, args, torch, detail):
     # fixed synthetic expert output, one row per place of the expert-order buffer
     if cfg.fmt == "fp8":
         g = torch.Generator(device=dev).manual_seed(cfg.seed)
-        ye = configs.quantise_fp8_rows(torch.randn(state.permuted.shape[0], cfg.hidden, generator=g, device=dev))
+        ye = configs.quantise_fp8_rows(torch.randn(state.permuted.shape[0], cfg.hidden, generator=g, device=dev),
+                                       cfg.row_pitch)
     else:
         ye = state.permuted.clone()
     torch.cuda.synchronize()
@@ -539,6 +543,7 @@ def run_workload(cfg, args, torch, detail):
     kb_rows = row % 1024 == 0
     k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
     k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
+    flat = torch.empty(cfg.pairs * row, dtype=torch.uint8, device=dev)      # as many bytes as the arrival buffer holds
     kernels = {     # name: (launch, bytes that must cross HBM per launch)
         f"{k_scatter}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), (cfg.T + cfg.send_rows) * row),
         f"{k_scatter}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
@@ -548,8 +553,7 @@ def run_workload(cfg, args, torch, detail):
         f"{k_gather}(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx), (kept + n_places) * row),
         "combine_kernel": (lambda: tops.combine(ye, where, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
                            kept * row + cfg.pairs * 12 + cfg.T * out_row),
-        "copy_kernel(passthrough)": (lambda: tops.passthrough(state.send_buf), 2 * state.send_buf.numel()
-                                     * state.send_buf.element_size()),
+        "copy_kernel(passthrough)": (lambda: tops.passthrough(flat), 2 * flat.numel()),
     }
     kern = {}
     for name, (fn, nb) in kernels.items():
@@ -614,6 +618,9 @@ def main():
         sys.exit(3)
     digest = _hip.load().terrace_version().decode().rsplit("src:", 1)[-1]
     cfg = configs.CONFIGS[args.config]
+    if args.row_pitch is not None:
+        import dataclasses
+        cfg = dataclasses.replace(cfg, row_pitch=args.row_pitch or None)
     torch.cuda.set_device(0)
 
     r = run_workload(cfg, args, torch, detail=True)
@@ -656,7 +663,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": cfg.name, "T": cfg.T, "E": cfg.n_experts, "n_groups": cfg.n_groups, "k": cfg.top_k,
                    "M": cfg.top_groups, "cards_per_group": cfg.rpn, "hidden": cfg.hidden, "row_bytes": cfg.row_bytes,
-                   "send_rows": cfg.send_rows, "pairs": cfg.pairs, "capacity": cap,
+                   "row_pitch": cfg.row_pitch, "send_rows": cfg.send_rows, "pairs": cfg.pairs, "capacity": cap,
                    "exchange": "loop-back (no all-to-all on one GPU)",
                    "expert_outputs": "fixed synthetic tensor prepared before the timed region"},
         "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),

@@ -78,6 +78,18 @@ enum terrace_fault {
 
 #define TERRACE_STATUS_WORDS 4
 
+/* Rows on a pitch.  Wherever an entry point takes `row_bytes` for the payload rows it moves, the rows may sit
+ * `pitch` bytes apart instead of back to back: pass TERRACE_ROW_PITCHED(width, pitch).  Every row buffer of that
+ * call (source and destination alike) is then [n_rows, pitch] bytes with `width` bytes of data at the start of
+ * each row; the bytes between width and pitch are never read and never written.  Requirements: width a multiple
+ * of 16, pitch a multiple of 1024 and >= width, every row buffer aligned to 16 bytes (to 1024 for full speed), width
+ * and pitch below 2^31; anything else is TERRACE_EINVAL.  A plain width (no pitch) means rows back to back, as in the reference.
+ * Why it exists: a wave of the row movers copies one aligned kilobyte of both buffers.  Rows that are not whole
+ * kilobytes (the 7392-byte fp8 row with its block scales) otherwise start at ever-shifting offsets inside a
+ * kilobyte, and every copy needs a re-loaded, shifted window; on an 8192-byte pitch the same rows move like
+ * kilobyte rows, at the cost of address space, not of traffic.  No counterpart in the reference. */
+#define TERRACE_ROW_PITCHED(width, pitch) ((int64_t)(width) | ((int64_t)(pitch) << 32))
+
 TERRACE_API const char *terrace_version(void);
 TERRACE_API const char *terrace_strerror(int status);
 
@@ -260,6 +272,10 @@ TERRACE_API int terrace_index_chain2(const int64_t *outer, int64_t n_outer, cons
  * out is [n_out,hidden] of out_dtype (F32, BF16 or F16).  The weights plane must be 4-byte aligned; a 16-bit
  * weight is read as the aligned 32-bit word that holds it, so when n_out*fan is odd the last read covers the two
  * bytes after the plane (the same aligned word: never another page, never used). */
+/* terrace_combine with the source rows `src_row_pitch` bytes apart (0: back to back, which is terrace_combine). */
+TERRACE_API int terrace_combine_pitched(const void *src, int64_t n_src, int src_dtype, int64_t src_row_pitch,
+                                        const int64_t *idx, const void *weights, int w_dtype, int64_t n_out, int fan,
+                                        int64_t hidden, void *out, int out_dtype, terrace_stream_t stream);
 TERRACE_API int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
                     int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
                     terrace_stream_t stream);

@@ -5,7 +5,8 @@ namespace terrace {
 int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
 int launch_stream_probe(int kind, const void *x, void *y, size_t nbytes, hipStream_t s);
 int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
-                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s);
+                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, int64_t src_pitch,
+                   hipStream_t s);
 int launch_index_chain(const int64_t *table, int64_t n_table, const int64_t *idx, int64_t n, int64_t *out,
                        hipStream_t s);
 int launch_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *inner, int64_t n_inner,
@@ -314,16 +315,23 @@ int terrace_index_chain2(const int64_t *outer, int64_t n_outer, const int64_t *i
     return launch_index_chain2(outer, n_outer, inner, n_inner, idx, n, out, (hipStream_t)stream);
 }
 
-int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
-                    int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
-                    terrace_stream_t stream) {
-    if (n_out < 0 || fan <= 0 || hidden < 0 || n_src < 0) return TERRACE_EINVAL;
+int terrace_combine_pitched(const void *src, int64_t n_src, int src_dtype, int64_t src_row_pitch, const int64_t *idx,
+                            const void *weights, int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out,
+                            int out_dtype, terrace_stream_t stream) {
+    if (n_out < 0 || fan <= 0 || hidden < 0 || n_src < 0 || src_row_pitch < 0) return TERRACE_EINVAL;
     if (src_dtype < TERRACE_F32 || src_dtype > TERRACE_FP8_E4M3_B128 || !float_dtype(out_dtype)) return TERRACE_EINVAL;
     if (weights && !float_dtype(w_dtype)) return TERRACE_EINVAL;
     if (src_dtype == TERRACE_FP8_E4M3_B128 && hidden % 128) return TERRACE_EINVAL;
     if (n_out && hidden && ((!src && n_src) || !idx || !out)) return TERRACE_EINVAL;
     return launch_combine(src, n_src, src_dtype, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
-                          (hipStream_t)stream);
+                          src_row_pitch, (hipStream_t)stream);
+}
+
+int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *weights,
+                    int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
+                    terrace_stream_t stream) {
+    return terrace_combine_pitched(src, n_src, src_dtype, 0, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
+                                   stream);
 }
 
 int terrace_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,

@@ -80,6 +80,24 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t c) {
     return __uint_as_float(__float_as_uint(mag) | sign);
 }
 
+// A row-width argument of the C ABI may carry a pitch (TERRACE_ROW_PITCHED): `width` bytes of data every `pitch`
+// bytes.  Packed rows have pitch == width.
+struct RowGeom {
+    int64_t width, pitch;
+    bool pitched() const { return pitch != width; }
+};
+inline RowGeom row_geom(int64_t row_bytes) {
+    RowGeom g{row_bytes & 0xFFFFFFFFll, row_bytes >> 32};
+    if (g.pitch == 0) g.pitch = g.width;
+    return g;
+}
+// Pitched rows move through the kilobyte-sliced kernels only: 16-byte-multiple widths on a whole number of
+// kilobytes.  (The buffers must also be 16-byte aligned; the launchers check that.)
+inline bool row_geom_ok(const RowGeom &g) {
+    if (g.width < 0 || g.pitch < g.width) return false;
+    return !g.pitched() || (g.width % 16 == 0 && g.pitch % 1024 == 0);
+}
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? TERRACE_OK : TERRACE_ELAUNCH; }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }

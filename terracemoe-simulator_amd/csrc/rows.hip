@@ -261,13 +261,17 @@ __global__ __launch_bounds__(kWave) void gather_rows_flat_kernel(const u32x4 *__
 }
 
 // Gather, rows that are whole kilobytes on a kilobyte-aligned destination: blockIdx.x = row * slices + slice.
+// `row_vecs` is the distance between rows (the pitch), `live_vecs` <= row_vecs what a row holds; the last slice of
+// a row whose width is not a whole number of kilobytes has idle lanes and touches nothing beyond the width.
 template <typename I>
 __global__ __launch_bounds__(kWave) void gather_rows_sliced_kernel(const u32x4 *__restrict__ src,
                                                                    u32x4 *__restrict__ out, const I *__restrict__ idx,
-                                                                   int64_t row_vecs, uint32_t slices, int64_t n_src) {
+                                                                   int64_t row_vecs, int64_t live_vecs, uint32_t slices,
+                                                                   int64_t n_src) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
     const int64_t i = (int64_t)slice * kWave + threadIdx.x;
+    if (i >= live_vecs) return;
     const int64_t from = (int64_t)idx[row];
     u32x4 v = zero_of<u32x4>();
     if (row_in(from, n_src)) v = ld_stream(src + from * row_vecs + i);
@@ -278,11 +282,12 @@ __global__ __launch_bounds__(kWave) void gather_rows_sliced_kernel(const u32x4 *
 template <typename I>
 __global__ __launch_bounds__(kWave) void scatter_rows_sliced_kernel(const u32x4 *__restrict__ src,
                                                                     u32x4 *__restrict__ dst, const I *__restrict__ pos,
-                                                                    int fan, int64_t row_vecs, uint32_t slices,
-                                                                    int64_t n_dst) {
+                                                                    int fan, int64_t row_vecs, int64_t live_vecs,
+                                                                    uint32_t slices, int64_t n_dst) {
     const uint32_t row = blockIdx.x / slices;
     const uint32_t slice = blockIdx.x - row * slices;
     const int64_t i = (int64_t)slice * kWave + threadIdx.x;
+    if (i >= live_vecs) return;
     const u32x4 v = ld_stream(src + (int64_t)row * row_vecs + i);
     const I *p = pos + (int64_t)row * fan;
     for (int f = 0; f < fan; ++f) {
@@ -692,15 +697,24 @@ static void launch_scatter_t(const void *src, void *dst, const I *pos, int64_t n
 template <typename I>
 int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src, int fan, int64_t row_bytes,
                         int64_t n_dst, hipStream_t s) {
-    if (n_src <= 0 || row_bytes <= 0 || fan <= 0) return TERRACE_OK;
+    const RowGeom geom = row_geom(row_bytes);
+    if (!row_geom_ok(geom)) return TERRACE_EINVAL;
+    if (n_src <= 0 || geom.width <= 0 || fan <= 0) return TERRACE_OK;
     if (n_src > kMaxGridRows) return TERRACE_EINVAL;
+    if (geom.pitched()) {        // rows on a kilobyte pitch: the sliced kernel, idle lanes past the width
+        const int64_t slices = (geom.width / 16 + kWave - 1) / kWave;
+        if ((((uintptr_t)src | (uintptr_t)dst) & 15) || n_src * slices > kMaxBlocks) return TERRACE_EINVAL;
+        scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * slices), kWave, 0, s>>>(
+            (const u32x4 *)src, (u32x4 *)dst, pos, fan, geom.pitch / 16, geom.width / 16, (uint32_t)slices, n_dst);
+        return check_launch();
+    }
     switch (vec_bytes_for(row_bytes, src, dst)) {
         case 16: {
             const int64_t rv = row_bytes / 16;
             const int head = (int)(((uintptr_t)dst >> 4) & (kWave - 1));
             if (rv % kWave == 0 && head == 0 && n_src * (rv / kWave) <= kMaxBlocks) {
                 scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, 0, s>>>(
-                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, (uint32_t)(rv / kWave), n_dst);
+                    (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, rv, (uint32_t)(rv / kWave), n_dst);
             } else {
                 const int64_t chunks = (rv + 2 * kWave - 2) / kWave;      // most kilobytes one copy can touch
                 if (n_src * chunks <= kMaxBlocks)
@@ -746,7 +760,7 @@ static bool launch_gather_sliced(const void *src, void *out, const I *idx, int64
     if (blocks > kMaxBlocks) return false;
     if (row_vecs % kWave == 0 && head == 0) {
         gather_rows_sliced_kernel<I><<<(unsigned)blocks, kWave, 0, s>>>((const u32x4 *)src, (u32x4 *)out, idx, row_vecs,
-                                                                       (uint32_t)(row_vecs / kWave), n_src);
+                                                                       row_vecs, (uint32_t)(row_vecs / kWave), n_src);
         return true;
     }
     // rows that are not whole lines: a row's chunks share lines on the source side
@@ -759,8 +773,17 @@ static bool launch_gather_sliced(const void *src, void *out, const I *idx, int64
 template <typename I>
 int launch_gather_rows(const void *src, void *out, const I *idx, int64_t n_out, int64_t row_bytes, int64_t n_src,
                        hipStream_t s) {
-    if (n_out <= 0 || row_bytes <= 0) return TERRACE_OK;
+    const RowGeom geom = row_geom(row_bytes);
+    if (!row_geom_ok(geom)) return TERRACE_EINVAL;
+    if (n_out <= 0 || geom.width <= 0) return TERRACE_OK;
     if (n_out > kMaxGridRows) return TERRACE_EINVAL;
+    if (geom.pitched()) {
+        const int64_t slices = (geom.width / 16 + kWave - 1) / kWave;
+        if ((((uintptr_t)src | (uintptr_t)out) & 15) || n_out * slices > kMaxBlocks) return TERRACE_EINVAL;
+        gather_rows_sliced_kernel<I><<<(unsigned)(n_out * slices), kWave, 0, s>>>(
+            (const u32x4 *)src, (u32x4 *)out, idx, geom.pitch / 16, geom.width / 16, (uint32_t)slices, n_src);
+        return check_launch();
+    }
     switch (vec_bytes_for(row_bytes, src, out)) {
         case 16:
             if (!launch_gather_sliced<I>(src, out, idx, n_out, row_bytes / 16, n_src, s))
@@ -792,9 +815,9 @@ static int64_t dtype_row_bytes(int dtype, int64_t hidden) {
 
 template <int SRC, int OUT>
 static void launch_combine_so(const void *src, int64_t n_src, const int64_t *idx, const void *w, int w_dtype,
-                              int64_t n_out, int fan, int64_t hidden, void *out, hipStream_t s) {
+                              int64_t n_out, int fan, int64_t hidden, void *out, int64_t src_pitch, hipStream_t s) {
     const int64_t chunks = hidden / Chunk<SRC>::N;
-    const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
+    const int64_t srb = src_pitch, orb = dtype_row_bytes(OUT, hidden);
     // one wave per workgroup when a row is a whole number of waves' worth of chunks (a workgroup
     // spanning a whole misaligned row, which would keep split cache lines inside one L2, measured
     // slower than this at the fp8 row shape)
@@ -810,17 +833,23 @@ static void launch_combine_so(const void *src, int64_t n_src, const int64_t *idx
 
 template <int SRC>
 static void launch_combine_s(const void *src, int64_t n_src, const int64_t *idx, const void *w, int w_dtype,
-                             int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
-    if (out_dtype == TERRACE_F32) launch_combine_so<SRC, TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
-    else if (out_dtype == TERRACE_BF16) launch_combine_so<SRC, TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
-    else launch_combine_so<SRC, TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, s);
+                             int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, int64_t src_pitch,
+                             hipStream_t s) {
+    if (out_dtype == TERRACE_F32) launch_combine_so<SRC, TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, src_pitch, s);
+    else if (out_dtype == TERRACE_BF16) launch_combine_so<SRC, TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, src_pitch, s);
+    else launch_combine_so<SRC, TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, src_pitch, s);
 }
 
+// `src_pitch`: bytes between source rows, 0 for rows back to back.
 int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
-                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, hipStream_t s) {
+                   int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, int64_t src_pitch,
+                   hipStream_t s) {
     if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
     if (n_out * ((hidden + 1023) / 1024 + 1) > kMaxGridRows) return TERRACE_EINVAL;
-    const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
+    const int64_t width = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
+    if (src_pitch == 0) src_pitch = width;
+    if (src_pitch < width) return TERRACE_EINVAL;
+    const int64_t srb = src_pitch;
     if (n_src <= 0) {           // no source rows: every entry is dead and every sum empty; no kernel needs to look
         zero_bytes_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)out, n_out * orb);
         return check_launch();
@@ -835,10 +864,10 @@ int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t 
         return check_launch();
     }
     switch (src_dtype) {
-        case TERRACE_F32: launch_combine_s<TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        case TERRACE_BF16: launch_combine_s<TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        case TERRACE_F16: launch_combine_s<TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
-        default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, s); break;
+        case TERRACE_F32: launch_combine_s<TERRACE_F32>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, srb, s); break;
+        case TERRACE_BF16: launch_combine_s<TERRACE_BF16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, srb, s); break;
+        case TERRACE_F16: launch_combine_s<TERRACE_F16>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, srb, s); break;
+        default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, srb, s); break;
     }
     return check_launch();
 }

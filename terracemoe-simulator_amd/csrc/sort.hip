@@ -710,6 +710,7 @@ constexpr int kPadRows = 16;             // the most places one workgroup looks 
 template <typename V>
 __global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restrict__ start, int epr, int64_t capacity,
                                                           int chunks, int pad_rows, V *__restrict__ rows, int64_t row_vecs,
+                                                          int64_t live_vecs,
                                                           void *__restrict__ gate_plane, int gate_bytes,
                                                           int64_t *__restrict__ pair_of_place,
                                                           int64_t *__restrict__ kept_per_expert) {
@@ -733,7 +734,14 @@ __global__ __launch_bounds__(kBlock) void zero_pad_kernel(const int32_t *__restr
     V *o = rows + first * row_vecs;
     V z;
     __builtin_memset(&z, 0, sizeof(V));
-    for (int64_t i = threadIdx.x; i < n * row_vecs; i += kBlock) __builtin_nontemporal_store(z, o + i);
+    if (live_vecs == row_vecs) {
+        for (int64_t i = threadIdx.x; i < n * row_vecs; i += kBlock) __builtin_nontemporal_store(z, o + i);
+    } else {                     // rows on a pitch: only the width of each row is written
+        for (int64_t i = threadIdx.x; i < n * live_vecs; i += kBlock) {
+            const int64_t r = i / live_vecs;
+            __builtin_nontemporal_store(z, o + r * row_vecs + (i - r * live_vecs));
+        }
+    }
 }
 
 struct EmitPairs {           // terrace/ta2a_fwd.py:605-628, general branch: pairs come as (row, slot) lists
@@ -1221,24 +1229,27 @@ static int launch_zero_pad(const int32_t *start, int epr, int64_t capacity, void
     // workgroups that find nothing to do, which still have to be launched, outweigh it), at most kPadRows; more
     // where that many workgroups would pass what one launch can hold (blocks * kBlock has to stay below 2^32)
     int pad_rows = kPadRows;
-    if (rows && row_bytes > 0) {
-        while (pad_rows > 1 && (int64_t)pad_rows * row_bytes > 16384) pad_rows /= 2;
+    const RowGeom geom = row_geom(row_bytes);
+    if (!row_geom_ok(geom) || (geom.pitched() && ((uintptr_t)rows & 15))) return TERRACE_EINVAL;
+    if (rows && geom.width > 0) {
+        while (pad_rows > 1 && (int64_t)pad_rows * geom.width > 16384) pad_rows /= 2;
     }
     while ((int64_t)epr * ((capacity + pad_rows - 1) / pad_rows) > (int64_t)1 << 22) pad_rows *= 2;
     const int chunks = capacity > 0 ? (int)((capacity + pad_rows - 1) / pad_rows) : 1;
     const int64_t blocks = (int64_t)epr * chunks;
-    if (!rows || row_bytes == 0) {
-        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows, nullptr, 0,
+    if (!rows || geom.width == 0) {
+        zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows, nullptr, 0, 0,
                                                                     gate_plane, gate_bytes, pair_of_place,
                                                                     kept_per_expert);
-    } else if ((((uintptr_t)rows | (uintptr_t)row_bytes) & 15) == 0) {
+    } else if ((((uintptr_t)rows | (uintptr_t)geom.width | (uintptr_t)geom.pitch) & 15) == 0) {
         zero_pad_kernel<pad_u32x4><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows,
-                                                                      (pad_u32x4 *)rows, row_bytes / 16, gate_plane,
-                                                                      gate_bytes, pair_of_place, kept_per_expert);
+                                                                      (pad_u32x4 *)rows, geom.pitch / 16, geom.width / 16,
+                                                                      gate_plane, gate_bytes, pair_of_place,
+                                                                      kept_per_expert);
     } else {
         zero_pad_kernel<uint8_t><<<(unsigned)blocks, kBlock, 0, s>>>(start, epr, capacity, chunks, pad_rows,
-                                                                    (uint8_t *)rows, row_bytes, gate_plane, gate_bytes,
-                                                                    pair_of_place, kept_per_expert);
+                                                                    (uint8_t *)rows, geom.pitch, geom.width, gate_plane,
+                                                                    gate_bytes, pair_of_place, kept_per_expert);
     }
     return check_launch();
 }
@@ -1260,7 +1271,7 @@ int run_hopb_scatter(const void *rx, const int64_t *rslot, const void *rgate, in
     if (P == 0) {
         int rc = empty_outputs(tokens_per_expert, nullptr, kept_per_expert, n_local, status, s);
         if (rc != TERRACE_OK || places == 0) return rc;
-        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_geom(row_bytes).pitch);
         if (permuted_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
         if (pair_of_place) fill_minus_one_kernel<<<64, kBlock, 0, s>>>(pair_of_place, places);
         return check_launch();
@@ -1303,7 +1314,7 @@ int run_hopb_scatter_move(const void *rx, int64_t R, int64_t row_bytes, int quot
     if (places == 0 || row_bytes == 0) return TERRACE_OK;
     if (!permuted) return TERRACE_EINVAL;
     if (P == 0) {       // all padding
-        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_geom(row_bytes).pitch);
         return check_launch();
     }
     if (!rx || !ws) return TERRACE_EINVAL;
@@ -1342,7 +1353,7 @@ int run_regroup(const void *node_rx, const int64_t *my_slot, const void *my_gate
     if (P == 0) {
         int rc = empty_outputs(tokens_per_expert, nullptr, kept_per_expert, epr, status, s);
         if (rc != TERRACE_OK || places == 0) return rc;
-        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        if (permuted && row_bytes) fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_geom(row_bytes).pitch);
         if (permuted_gate) fill_zero_kernel<<<64, kBlock, 0, s>>>((uint8_t *)permuted_gate, places * gate_bytes);
         return check_launch();
     }
@@ -1507,7 +1518,7 @@ int run_regroup_move(const void *node_rx, int64_t P, int64_t row_bytes, int epr,
     if (places == 0 || row_bytes == 0) return TERRACE_OK;
     if (!permuted) return TERRACE_EINVAL;
     if (P == 0) {       // all padding
-        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_bytes);
+        fill_zero_kernel<<<1024, kBlock, 0, s>>>((uint8_t *)permuted, places * row_geom(row_bytes).pitch);
         return check_launch();
     }
     if (!node_rx || !ws) return TERRACE_EINVAL;

@@ -63,6 +63,7 @@ SIGNATURES = {
     "terrace_index_chain": (_I, [_P, _L, _P, _L, _P, _P]),
     "terrace_index_chain2": (_I, [_P, _L, _P, _L, _P, _L, _P, _P]),
     "terrace_combine": (_I, [_P, _L, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
+    "terrace_combine_pitched": (_I, [_P, _L, _I, _L, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
     "terrace_pack_planes": (_I, [_P, _L, _P, _L, _P, _L, _L, _L, _P, _P]),
     "terrace_unpack_planes": (_I, [_P, _L, _L, _P, _L, _P, _L, _P, _L, _P]),
     "terrace_k2_pack_wire": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I,
@@ -202,6 +203,33 @@ def stream(device) -> c_void_p:
             index = torch.cuda.current_device()
         return c_void_p(_RAW_STREAM(index))
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def row_arg(t) -> int:
+    """The ``row_bytes`` argument for a 2-D row tensor: its width in bytes, or -- for a row-pitched view (unit
+    stride inside a row, rows further apart than they are wide) -- TERRACE_ROW_PITCHED(width, pitch)."""
+    width = t.shape[1] * t.element_size()
+    if t.shape[0] <= 1 or t.stride(0) == t.shape[1]:
+        return width
+    return width | ((t.stride(0) * t.element_size()) << 32)
+
+
+def is_rows(t) -> bool:
+    """Whether ``t`` can go to the library as it is: 2-D, unit stride inside a row, rows not overlapping."""
+    return t.dim() == 2 and (t.shape[1] <= 1 or t.stride(1) == 1) and (t.shape[0] <= 1 or t.stride(0) >= t.shape[1])
+
+
+def as_rows(t):
+    """``t`` itself when it is packed or row-pitched, else a packed copy."""
+    return t if t.is_contiguous() or is_rows(t) else t.contiguous()
+
+
+def empty_rows(n: int, like):
+    """[n, width] rows of ``like``'s dtype on ``like``'s device, on the same pitch as ``like``."""
+    width = like.shape[1]
+    if like.shape[0] <= 1 or like.stride(0) == width or not is_rows(like):
+        return torch.empty((n, width), dtype=like.dtype, device=like.device)
+    return torch.empty((n, like.stride(0)), dtype=like.dtype, device=like.device)[:, :width]
 
 
 def float_code(dtype) -> int:

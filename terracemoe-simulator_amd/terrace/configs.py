@@ -29,6 +29,7 @@ class PathConfig:
     softmax_gates: bool = False     # gates = renormalised softmax over the selected experts
     capacity_factor: float | None = None
     seed: int = 1234
+    row_pitch: int | None = None    # bytes between payload rows in every row buffer (None: rows back to back)
 
     @property
     def world(self) -> int:
@@ -88,25 +89,51 @@ CONFIGS = {
     "c3": PathConfig("c3_high_dedup", 32768, 128, 16, 8, 2, 8, 4096, "bf16", seed=1237),
     "c4": PathConfig("c4_skewed_capacity", 65536, 256, 8, 8, 4, 8, 2048, "bf16", bias="zipf",
                      capacity_factor=1.25, seed=1238),
+    # the 7392-byte fp8 row (codes, then the block scales) sits on an 8 KB pitch in every row buffer, so that the row
+    # movers copy aligned kilobytes of it; the 800 bytes between one row's end and the next row are never touched
     "c5": PathConfig("c5_fp8_payload", 16384, 256, 8, 8, 4, 8, 7168, "fp8", bias="normal",
-                     softmax_gates=True, seed=1239),
+                     softmax_gates=True, seed=1239, row_pitch=8192),
 }
 
 
-def quantise_fp8_rows(x: torch.Tensor) -> torch.Tensor:
+def pitched_rows(rows: torch.Tensor, pitch_bytes: int | None) -> torch.Tensor:
+    """The same [n, width] rows as a view of an [n, pitch] buffer (bytes past the width zero); unchanged when
+    ``pitch_bytes`` is None."""
+    if pitch_bytes is None:
+        return rows
+    n, width = rows.shape
+    per = pitch_bytes // rows.element_size()
+    assert per * rows.element_size() == pitch_bytes and per >= width
+    base = torch.zeros((n, per), dtype=rows.dtype, device=rows.device)
+    base[:, :width] = rows
+    return base[:, :width]
+
+
+def rows_to(rows: torch.Tensor, device) -> torch.Tensor:
+    """``rows.to(device)`` that keeps a row pitch (a plain ``.to`` packs a view with gaps)."""
+    if rows.dim() != 2 or rows.is_contiguous() or rows.shape[0] <= 1:
+        return rows.to(device)
+    n, width = rows.shape
+    whole = rows.as_strided((n, rows.stride(0)), (rows.stride(0), 1))
+    return whole.to(device)[:, :width]
+
+
+def quantise_fp8_rows(x: torch.Tensor, pitch_bytes: int | None = None) -> torch.Tensor:
     """[n, H] float -> uint8 [n, H + H/32]: e4m3 codes then one fp32 scale per 128 elements
-    (scale = max|x| / 448, or 1 for an all-zero block)."""
+    (scale = max|x| / 448, or 1 for an all-zero block); on a row pitch when ``pitch_bytes`` is given."""
     n, hidden = x.shape
     xb = x.float().reshape(n, hidden // FP8_BLOCK, FP8_BLOCK)
     amax = xb.abs().amax(-1)
     scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
     codes = (xb / scale[..., None]).to(torch.float8_e4m3fn).view(torch.uint8).reshape(n, hidden)
-    return torch.cat([codes, scale.contiguous().view(torch.uint8).reshape(n, -1)], dim=1).contiguous()
+    return pitched_rows(torch.cat([codes, scale.contiguous().view(torch.uint8).reshape(n, -1)], dim=1).contiguous(),
+                        pitch_bytes)
 
 
 def make_inputs(cfg: PathConfig) -> dict:
     """CPU tensors: logits [T,E] f32, bias [E] f32, gate_affinity [T,E] f32 or None,
-    x (payload rows in storage form: f32 / bf16 [T,H] or uint8 [T,row_bytes]), x_f32 or None."""
+    x (payload rows in storage form: f32 / bf16 [T,H] or uint8 [T,row_bytes]; a view of a wider buffer when the
+    geometry names a row pitch -- move it with ``rows_to``)."""
     g = torch.Generator().manual_seed(cfg.seed)
     logits = torch.randn(cfg.T, cfg.n_experts, generator=g)
     if cfg.bias == "normal":
@@ -127,7 +154,7 @@ def make_inputs(cfg: PathConfig) -> dict:
         x = x32.to(torch.bfloat16)
     else:
         x = quantise_fp8_rows(x32)
-    return {"logits": logits, "bias": bias, "gate_affinity": gate_aff, "x": x}
+    return {"logits": logits, "bias": bias, "gate_affinity": gate_aff, "x": pitched_rows(x, cfg.row_pitch)}
 
 
 def algorithmic_bytes(cfg: PathConfig, out_row_bytes: int | None = None) -> dict:

@@ -139,9 +139,9 @@ def k1_arrival_raw(rx, rslot, rgate, quota, epr, rpn, my_local=0, want_pair_pos=
     P = R * quota
     send_buf, row_bytes = None, 0
     if rx is not None:
-        rx = rx.contiguous()
-        row_bytes = rx.shape[1] * rx.element_size()
-        send_buf = torch.empty((P, rx.shape[1]), dtype=rx.dtype, device=dev)
+        rx = _hip.as_rows(rx)
+        row_bytes = _hip.row_arg(rx)
+        send_buf = _hip.empty_rows(P, rx)
     gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
     r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
@@ -259,9 +259,9 @@ def k2_pack_raw(hidden, expert_idx, gates, world, n_experts, rpn, groups_m, extr
     S, q, n_nodes = T * groups_m, k // groups_m, world // rpn
     payload, row_bytes = None, 0
     if hidden is not None:
-        hidden = hidden.contiguous()
-        row_bytes = hidden.shape[1] * hidden.element_size()
-        payload = torch.empty((S, hidden.shape[1]), dtype=hidden.dtype, device=dev)
+        hidden = _hip.as_rows(hidden)
+        row_bytes = _hip.row_arg(hidden)
+        payload = _hip.empty_rows(S, hidden)
     mask = torch.empty((S, q), dtype=torch.int64, device=dev)
     gate_rows = torch.empty((S, q), dtype=gates.dtype, device=dev)
     u_src = torch.empty((S,), dtype=torch.int64, device=dev)
@@ -419,15 +419,15 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None, tags
     _hip.need_device(node_rx, my_slot, my_gate)
     if my_slot.dtype != torch.int64:
         raise RuntimeError("regroup: my_slot must be int64")
-    node_rx, my_slot = node_rx.contiguous(), my_slot.contiguous().reshape(-1)
+    my_slot = my_slot.contiguous().reshape(-1)
     dev = my_slot.device
     P = my_slot.numel()
     if node_rx.dim() != 2 or node_rx.shape[0] != P:
         raise RuntimeError(f"regroup: node_rx {tuple(node_rx.shape)} does not have one row per slot id ({P})")
-    H = node_rx.shape[1]
+    node_rx = _hip.as_rows(node_rx)
     cap = -1 if capacity is None else int(capacity)
     places = P if capacity is None else epr * cap
-    permuted = torch.empty((places, H), dtype=node_rx.dtype, device=dev)
+    permuted = _hip.empty_rows(places, node_rx)
     tpe = torch.empty((epr,), dtype=torch.int64, device=dev)
     kpe = torch.empty((epr,), dtype=torch.int64, device=dev)
     order = torch.empty((P,), dtype=torch.int64, device=dev) if capacity is None else None
@@ -446,7 +446,7 @@ def regroup(node_rx, my_slot, epr, my_local=0, capacity=None, my_gate=None, tags
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_regroup_workspace", P, epr, cap), dev)
     _hip.call("terrace_regroup", _hip.ptr(node_rx), _hip.ptr(my_slot), _hip.ptr(my_gate), P,
-              H * node_rx.element_size(), gate_bytes, epr, my_local, cap, _hip.ptr(permuted), _hip.ptr(pgate),
+              _hip.row_arg(node_rx), gate_bytes, epr, my_local, cap, _hip.ptr(permuted), _hip.ptr(pgate),
               _hip.ptr(order), _hip.ptr(dest), _hip.ptr(kept), _hip.ptr(tpe), _hip.ptr(kpe), _hip.ptr(tags),
               _hip.ptr(table), n_tags, _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
     if capacity is None:
@@ -487,9 +487,9 @@ def hopb_scatter(rx, rslot, rgate, quota, n_local, first_slot=0, capacity=None, 
     i64 = dict(dtype=torch.int64, device=dev)
     permuted, row_bytes = None, 0
     if rx is not None:
-        rx = rx.contiguous()
-        row_bytes = rx.shape[1] * rx.element_size()
-        permuted = torch.empty((places, rx.shape[1]), dtype=rx.dtype, device=dev)
+        rx = _hip.as_rows(rx)
+        row_bytes = _hip.row_arg(rx)
+        permuted = _hip.empty_rows(places, rx)
     pgate, gate_bytes = None, 4
     if rgate is not None:
         rgate = rgate.contiguous()
@@ -621,13 +621,17 @@ def gather_rows(src, idx):
     zero rows -- the kernel never forms an address from them."""
     _require()
     _hip.need_device(src, idx)
-    src, idx = src.contiguous(), idx.contiguous().reshape(-1)
+    src, idx = (_hip.as_rows(src) if src.dim() == 2 else src.contiguous()), idx.contiguous().reshape(-1)
     if idx.dtype != torch.int64:
         raise RuntimeError("gather_rows: idx must be int64")
-    out = torch.empty((idx.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
-    row_bytes = src.element_size()
-    for d in src.shape[1:]:
-        row_bytes *= int(d)
+    if src.dim() == 2 and not src.is_contiguous():          # rows on a pitch: the output takes the same pitch
+        out = _hip.empty_rows(idx.numel(), src)
+        row_bytes = _hip.row_arg(src)
+    else:
+        out = torch.empty((idx.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+        row_bytes = src.element_size()
+        for d in src.shape[1:]:
+            row_bytes *= int(d)
     _hip.call("terrace_gather_rows", _hip.ptr(src), src.shape[0], _hip.ptr(idx), idx.numel(), row_bytes,
               _hip.ptr(out), _hip.stream(src.device))
     return out
@@ -639,13 +643,17 @@ def scatter_rows(src, pos, n_dst):
     names are left uninitialised."""
     _require()
     _hip.need_device(src, pos)
-    src, pos = src.contiguous(), pos.contiguous()
+    src, pos = (_hip.as_rows(src) if src.dim() == 2 else src.contiguous()), pos.contiguous()
     if pos.dtype != torch.int64 or pos.dim() != 2 or pos.shape[0] != src.shape[0]:
         raise RuntimeError("scatter_rows: pos must be int64 [n_src, fan]")
-    dst = torch.empty((n_dst,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
-    row_bytes = src.element_size()
-    for d in src.shape[1:]:
-        row_bytes *= int(d)
+    if src.dim() == 2 and not src.is_contiguous():          # rows on a pitch: the output takes the same pitch
+        dst = _hip.empty_rows(int(n_dst), src)
+        row_bytes = _hip.row_arg(src)
+    else:
+        dst = torch.empty((n_dst,) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+        row_bytes = src.element_size()
+        for d in src.shape[1:]:
+            row_bytes *= int(d)
     _hip.call("terrace_scatter_rows", _hip.ptr(src), _hip.ptr(pos), src.shape[0], pos.shape[1], row_bytes,
               _hip.ptr(dst), int(n_dst), _hip.stream(src.device))
     return dst
@@ -683,7 +691,7 @@ def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
     """
     _require()
     _hip.need_device(src, idx, weights)
-    src, idx = src.contiguous(), idx.contiguous()
+    src, idx = _hip.as_rows(src), idx.contiguous()
     if idx.dim() != 2 or idx.dtype != torch.int64:
         raise RuntimeError("combine: idx must be a 2-D int64 table")
     n_out, fan = idx.shape
@@ -704,8 +712,9 @@ def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
             raise RuntimeError("combine: weights must match idx")
         w_code = _hip.float_code(weights.dtype)
     out = torch.empty((n_out, hidden), dtype=out_dtype, device=src.device)
-    _hip.call("terrace_combine", _hip.ptr(src), src.shape[0], src_code, _hip.ptr(idx), _hip.ptr(weights), w_code, n_out, fan,
-              hidden, _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
+    pitch = 0 if src.is_contiguous() else src.stride(0) * src.element_size()
+    _hip.call("terrace_combine_pitched", _hip.ptr(src), src.shape[0], src_code, pitch, _hip.ptr(idx), _hip.ptr(weights),
+              w_code, n_out, fan, hidden, _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
     return out
 
 

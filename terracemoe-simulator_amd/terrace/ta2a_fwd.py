@@ -262,21 +262,20 @@ def _dispatch_one_slab(x, expert_idx, gates, world, n_experts, rpn, groups_m, ca
     _ops._require()
     _hip.need_device(x, expert_idx, gates)
     _ops._check_k2(x, expert_idx, gates, world, n_experts, rpn, groups_m)
-    x, expert_idx, gates = x.contiguous(), expert_idx.contiguous(), gates.contiguous()
+    x, expert_idx, gates = _hip.as_rows(x), expert_idx.contiguous(), gates.contiguous()
     dev = x.device
     T, k = expert_idx.shape
-    H = x.shape[1]
     epr, n_nodes = n_experts // world, world // rpn
     slots, quota = epr * rpn, k // groups_m
     S, P = T * groups_m, T * k
     cap = -1 if capacity is None else int(capacity)
     places = P if capacity is None else slots * cap
-    row_bytes, gb = H * x.element_size(), gates.element_size()
+    row_bytes, gb = _hip.row_arg(x), gates.element_size()        # rows on a pitch keep it through every stage
     lay = _dispatch_layout(T, k, world, n_experts, rpn, groups_m, capacity, gates.dtype, onepass)
     slab = _planes.Slab(lay, dev)
-    payload = torch.empty((S, H), dtype=x.dtype, device=dev)
-    permuted = torch.empty((places, H), dtype=x.dtype, device=dev)
-    send_buf = None if onepass else torch.empty((P, H), dtype=x.dtype, device=dev)
+    payload = _hip.empty_rows(S, x)
+    permuted = _hip.empty_rows(places, x)
+    send_buf = None if onepass else _hip.empty_rows(P, x)
     ptr, at, stream = _hip.ptr, slab.ptr, _hip.stream(dev)
     # the plan's guard (terrace/ta2a.py:161-204 of the reference): the status words are read back on the first
     # dispatch of a shape and on every 256th, after the last launch so the read-back waits for nothing extra

@@ -130,7 +130,7 @@ def _check_every_plane(cfg):
     e, g32, oe, og = _route(cfg, inp)
     gates = g32.to(cfg.gate_dtype)
     ogates = to_np(gates)
-    x = inp["x"].to(DEV)
+    x = configs.rows_to(inp["x"], DEV)
     ox = _np_rows(inp["x"])
     cap = cfg.capacity(cfg.slots)
     st = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
@@ -262,7 +262,7 @@ def _full_size_check(cfg):
     inp = configs.make_inputs(cfg)
     e, g32, oe, og = _route(cfg, inp)
     gates = g32.to(cfg.gate_dtype)
-    x = inp["x"].to(DEV)
+    x = configs.rows_to(inp["x"], DEV)
     cap = cfg.capacity(cfg.slots)
     st = loopback_dispatch(x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
     u_src, u_node, counts, inverse = orc.plan_ta2a(oe, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups)
@@ -348,7 +348,7 @@ def test_two_phase_operators_and_overlapped_dispatch_equal_the_single_calls(name
     announce("two-phase", cfg.name, cfg.T)
     inp = configs.make_inputs(cfg)
     e, g, _, _ = _route(cfg, inp)
-    x = inp["x"].to(DEV)
+    x = configs.rows_to(inp["x"], DEV)
     gates = g.to(cfg.gate_dtype)
     cap = cfg.capacity(cfg.slots)
     args = (x, e, gates, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups, cap)
@@ -407,7 +407,7 @@ def test_two_host_threads_on_two_streams_do_not_disturb_each_other():
         cfg = configs.CONFIGS[name].scaled(T)
         inp = configs.make_inputs(cfg)
         e, g, _, _ = _route(cfg, inp)
-        jobs.append((cfg, inp["x"].to(DEV), e, g.to(cfg.gate_dtype)))
+        jobs.append((cfg, configs.rows_to(inp["x"], DEV), e, g.to(cfg.gate_dtype)))
 
     def run(job):
         cfg, x, e, gates = job
@@ -453,7 +453,7 @@ def test_the_whole_step_replays_as_one_hip_graph(name):
     cfg = configs.CONFIGS[name].scaled(2048)
     announce("graph replay", cfg.name)
     inp = configs.make_inputs(cfg)
-    logits, bias, x = inp["logits"].to(DEV), inp["bias"].to(DEV), inp["x"].to(DEV)
+    logits, bias, x = inp["logits"].to(DEV), inp["bias"].to(DEV), configs.rows_to(inp["x"], DEV)
     ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(DEV)
     rcfg = terrace.TRouteConfig(cfg.n_experts, cfg.n_groups, cfg.top_k, cfg.top_groups)
     cap = cfg.capacity(cfg.slots)
