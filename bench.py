@@ -486,6 +486,40 @@ def run_workload(cfg, args, torch, detail):
                             "(terrace_hopb_scatter) instead of arrival chain + regroup; priced on its own bytes"},
         "kept_pairs": kept_pairs, "places": places, "phys": phys, "conv": conv, "hopb_bytes": hopb_bytes,
     }
+    def measure_in_step():
+        # ---- each stage timed INSIDE the step: events between the stage calls of K whole steps, so that no stage sees
+        # inputs a previous launch of itself left in a cache (alone, back to back, the pack re-reads the same 235 MB)
+        names = ("route", "pack", "arrival", "regroup", "combine")
+        marks = []
+        for it in range(reps + 2):
+            ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+            ev[0].record()
+            e_, g_, _ = route()
+            ev[1].record()
+            (pl_, mk_, gr_, _us, _nc), ex_ = tops.k2_pack_raw(x, e_, g_, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups,
+                                                              extras=True, combine_table=True)
+            ev[2].record()
+            tg_ = []
+            sb_, _gp, _ri, si_, _is, _pp = tops.k1_arrival_raw(pl_, mk_, gr_, quota, cfg.epr, cfg.rpn, 0, want_pair_pos=True,
+                                                               tags=ex_["pair_src"], tags_out=tg_)
+            ev[3].record()
+            tops.regroup(sb_, si_, cfg.slots, 0, cap, tags=tg_[0], table=ex_["where"])
+            ev[4].record()
+            tops.combine(ye, ex_["where"], ex_["gate_sorted"], out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
+            ev[5].record()
+            if it >= 2:
+                marks.append(ev)
+        torch.cuda.synchronize()
+        in_step = {n: statistics.median(m[i].elapsed_time(m[i + 1]) for m in marks) for i, n in enumerate(names)}
+        pc_in = in_step["pack"] + in_step["combine"]
+        return {"stage_ms": {n: round(v, 4) for n, v in in_step.items()},
+                          "stage_frac_hbm_peak": {n: round(gbps(phys[n], v) / HBM_PEAK_GBPS, 4) for n, v in in_step.items()},
+                          "pack_plus_combine_ms": round(pc_in, 4),
+                          "pack_plus_combine_frac_hbm_peak": round(gbps(phys["pack"] + phys["combine"], pc_in) / HBM_PEAK_GBPS, 4),
+                          "note": "median over the timed steps of the time between HIP events recorded around each stage "
+                                  "call inside whole steps (stage operators called one by one, same kernels)"}
+
+    out["in_step"] = measure_in_step()
     if not detail:
         ms_arr, ms_pack, ms_comb = event_ms(arrival, reps, torch), event_ms(pack, reps, torch), event_ms(combine, reps, torch)
         out["arrival_us_per_row"] = ms_arr * 1e3 / cfg.pairs
@@ -540,7 +574,7 @@ def run_workload(cfg, args, torch, detail):
     kept = cfg.pairs if kept_pairs is None else kept_pairs
     out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
     # names of the kernels the library picks for this row width (whole kilobytes or not)
-    kb_rows = row % 1024 == 0
+    kb_rows = row % 1024 == 0 or cfg.row_pitch is not None
     k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
     k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
     flat = torch.empty(cfg.pairs * row, dtype=torch.uint8, device=dev)      # as many bytes as the arrival buffer holds
@@ -562,38 +596,7 @@ def run_workload(cfg, args, torch, detail):
                       "frac_hbm_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
     out["kernels"] = kern
     out["graph"] = graph_replay_ms(step, args, torch) if args.graph else None
-    # ---- each stage timed INSIDE the step: events between the stage calls of K whole steps, so that no stage sees
-    # inputs a previous launch of itself left in a cache (alone, back to back, the pack re-reads the same 235 MB)
-    names = ("route", "pack", "arrival", "regroup", "combine")
-    marks = []
-    for it in range(reps + 2):
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
-        ev[0].record()
-        e_, g_, _ = route()
-        ev[1].record()
-        (pl_, mk_, gr_, _us, _nc), ex_ = tops.k2_pack_raw(x, e_, g_, cfg.world, cfg.n_experts, cfg.rpn, cfg.top_groups,
-                                                          extras=True, combine_table=True)
-        ev[2].record()
-        tg_ = []
-        sb_, _gp, _ri, si_, _is, _pp = tops.k1_arrival_raw(pl_, mk_, gr_, quota, cfg.epr, cfg.rpn, 0, want_pair_pos=True,
-                                                           tags=ex_["pair_src"], tags_out=tg_)
-        ev[3].record()
-        tops.regroup(sb_, si_, cfg.slots, 0, cap, tags=tg_[0], table=ex_["where"])
-        ev[4].record()
-        tops.combine(ye, ex_["where"], ex_["gate_sorted"], out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden)
-        ev[5].record()
-        if it >= 2:
-            marks.append(ev)
-    torch.cuda.synchronize()
-    in_step = {n: statistics.median(m[i].elapsed_time(m[i + 1]) for m in marks) for i, n in enumerate(names)}
-    pc_in = in_step["pack"] + in_step["combine"]
-    out["in_step"] = {"stage_ms": {n: round(v, 4) for n, v in in_step.items()},
-                      "stage_frac_hbm_peak": {n: round(gbps(phys[n], v) / HBM_PEAK_GBPS, 4) for n, v in in_step.items()},
-                      "pack_plus_combine_ms": round(pc_in, 4),
-                      "pack_plus_combine_frac_hbm_peak": round(gbps(phys["pack"] + phys["combine"], pc_in) / HBM_PEAK_GBPS, 4),
-                      "note": "median over the timed steps of the time between HIP events recorded around each stage "
-                              "call inside whole steps (stage operators called one by one, same kernels)"}
-    out["raw_dispatch_plus_combine_ms"] = sum(v for n, v in in_step.items() if n != "route")
+    out["raw_dispatch_plus_combine_ms"] = sum(v for n, v in out["in_step"]["stage_ms"].items() if n != "route")
     out["tensors"] = (e, gates, x)
     return out
 
@@ -696,6 +699,7 @@ def main():
                             "frac_hbm_peak": round(o["GBps"] / HBM_PEAK_GBPS, 4),
                             "arrival_us_per_row": round(o["arrival_us_per_row"], 6),
                             "pack_plus_combine_frac_hbm_peak": round(o["pack_plus_combine_frac_hbm_peak"], 4),
+                            "pack_plus_combine_in_step_frac_hbm_peak": o["in_step"]["pack_plus_combine_frac_hbm_peak"],
                             "onepass_ms_per_step": o["onepass"]["ms_per_step"],
                             "onepass_frac_hbm_peak": o["onepass"]["frac_hbm_peak"],
                             "onepass_same_output": o["onepass"]["same_output_as_two_step"]}
