@@ -575,14 +575,16 @@ def run_workload(cfg, args, torch, detail):
     out_row = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
     # names of the kernels the library picks for this row width (whole kilobytes or not)
     kb_rows = row % 1024 == 0 or cfg.row_pitch is not None
-    k_scatter = "scatter_rows_sliced_kernel" if kb_rows else "scatter_rows_aligned_kernel"
+    def k_scatter(fan):     # two copies have a kernel of their own
+        return ("scatter_rows_sliced_fan2_kernel" if fan == 2 else "scatter_rows_sliced_kernel") if kb_rows \
+            else "scatter_rows_aligned_kernel"
     k_gather = "gather_rows_sliced_kernel" if kb_rows else "gather_rows_flat_kernel"
     flat = torch.empty(cfg.pairs * row, dtype=torch.uint8, device=dev)      # as many bytes as the arrival buffer holds
     kernels = {     # name: (launch, bytes that must cross HBM per launch)
-        f"{k_scatter}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), (cfg.T + cfg.send_rows) * row),
-        f"{k_scatter}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
+        f"{k_scatter(cfg.top_groups)}(pack)": (lambda: tops.scatter_rows(x, token_rows, cfg.send_rows), (cfg.T + cfg.send_rows) * row),
+        f"{k_scatter(quota)}(arrival)": (lambda: tops.scatter_rows(state.payload, pair_pos2, cfg.pairs),
                                   (cfg.send_rows + cfg.pairs) * row),
-        f"{k_scatter}(hopb_onepass)": (lambda: tops.scatter_rows(state.payload, place_of_pair, n_places),
+        f"{k_scatter(quota)}(hopb_onepass)": (lambda: tops.scatter_rows(state.payload, place_of_pair, n_places),
                                        (cfg.send_rows + kept) * row),
         f"{k_gather}(regroup)": (lambda: tops.gather_rows(state.send_buf, gather_idx), (kept + n_places) * row),
         "combine_kernel": (lambda: tops.combine(ye, where, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
