@@ -311,9 +311,9 @@ def predicted_floor_ms(ceil, read_bytes, written_bytes):
     return read_bytes / (ceil["read_only"]["GBps"] * 1e6) + written_bytes / (ceil["write_only"]["GBps"] * 1e6)
 
 
-def count_launches(fn, torch):
+def count_launches(fn, torch, names=None):
     """Kernel launches one call of fn() makes, from torch's profiler (None when it is unavailable, e.g. under
-    another profiler)."""
+    another profiler).  `names`, a dict, receives kernel name -> [launches, microseconds on the device]."""
     try:
         from torch.profiler import ProfilerActivity, profile
         fn()
@@ -326,6 +326,11 @@ def count_launches(fn, torch):
             if ev.device_type is not None and "cuda" in str(ev.device_type).lower() and "memcpy" not in ev.name.lower() \
                     and "memset" not in ev.name.lower():
                 n += 1
+                if names is not None:
+                    short = ev.name.split("(")[0].split("<")[0].split("::")[-1].strip() or ev.name[:40]
+                    rec = names.setdefault(short, [0, 0.0])
+                    rec[0] += 1
+                    rec[1] = round(rec[1] + float(getattr(ev, "device_time_total", 0.0) or 0.0), 1)
         return n or None
     except Exception:
         return None
@@ -369,8 +374,10 @@ def seam_block(cfg, args, torch, raw_step_ms, e, gates, x):
     with torch.no_grad():
         for name, (fn, syncs) in legs.items():
             ms = wall_ms(fn, max(args.steps // 2, 5), 2, torch)
+            names = {}
             out[name] = {"ms_per_call": round(ms, 4), "ratio_to_raw": round(ms / raw_step_ms, 3),
-                         "kernel_launches": count_launches(fn, torch), "host_syncs": syncs}
+                         "kernel_launches": count_launches(fn, torch, names), "host_syncs": syncs,
+                         "kernels_launches_us": names}
     return out
 
 

@@ -280,6 +280,19 @@ TERRACE_API int terrace_combine(const void *src, int64_t n_src, int src_dtype, c
                     int w_dtype, int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype,
                     terrace_stream_t stream);
 
+/* The reference's TWO combine levels in one pass (terrace/ta2a_dispatch.py:483-494: a send row sums the expert outputs
+ * of its pairs, a token sums its send rows, each level an fp32 index_add rounded once to the tensor dtype), for a
+ * caller whose two levels run on the same GPU with no exchange between them (loop-back):
+ *   out[t] = round_out( sum_m f32( round_src( sum_i f32(src[inner[outer[t, m], i]]) ) ) )
+ * inner [n_rows, fan_inner] i64 names source rows (fan_inner = 1, 2, 4 or 8), outer [n_out, fan_outer] i64 names rows
+ * of inner; entries outside their range are skipped.  Bit for bit terrace_combine(src, inner) into the source dtype
+ * followed by terrace_combine(that, outer), without the [n_rows, hidden] plane between them.  src f32 / bf16 / f16,
+ * rows 16-byte multiples on 16-byte-aligned buffers; anything else returns TERRACE_EINVAL (run the two levels). */
+TERRACE_API int terrace_combine_two_level(const void *src, int64_t n_src, int src_dtype, const int64_t *inner,
+                                          int64_t n_rows, int fan_inner, const int64_t *outer, int64_t n_out,
+                                          int fan_outer, int64_t hidden, void *out, int out_dtype,
+                                          terrace_stream_t stream);
+
 /* Wire containers (terrace/ta2a_pack.py:319-336 hopa_pack, :398-414 hopa_pack_small, :474-497
  * hopb_pack_meta): each out row of row_bytes is plane a's row, then b's, then c's, then zeros.
  * A NULL plane is absent (its width counts as 0).  Pure byte moves.

@@ -4,6 +4,9 @@
 namespace terrace {
 int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s);
 int launch_stream_probe(int kind, const void *x, void *y, size_t nbytes, hipStream_t s);
+int launch_combine2(const void *src, int64_t n_src, int src_dtype, const int64_t *inner, int64_t n_rows, int fan_inner,
+                    const int64_t *outer, int64_t n_out, int fan_outer, int64_t hidden, void *out, int out_dtype,
+                    hipStream_t s);
 int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t *idx, const void *w, int w_dtype,
                    int64_t n_out, int fan, int64_t hidden, void *out, int out_dtype, int64_t src_pitch,
                    hipStream_t s);
@@ -332,6 +335,13 @@ int terrace_combine(const void *src, int64_t n_src, int src_dtype, const int64_t
                     terrace_stream_t stream) {
     return terrace_combine_pitched(src, n_src, src_dtype, 0, idx, weights, w_dtype, n_out, fan, hidden, out, out_dtype,
                                    stream);
+}
+
+int terrace_combine_two_level(const void *src, int64_t n_src, int src_dtype, const int64_t *inner, int64_t n_rows,
+                              int fan_inner, const int64_t *outer, int64_t n_out, int fan_outer, int64_t hidden,
+                              void *out, int out_dtype, terrace_stream_t stream) {
+    return launch_combine2(src, n_src, src_dtype, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out,
+                           out_dtype, (hipStream_t)stream);
 }
 
 int terrace_pack_planes(const void *a, int64_t a_bytes, const void *b, int64_t b_bytes, const void *c, int64_t c_bytes,

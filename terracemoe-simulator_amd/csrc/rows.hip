@@ -542,6 +542,76 @@ __global__ __launch_bounds__(kBlock) void combine_kernel(const uint8_t *__restri
 #undef TERRACE_COMBINE_BODY
 }
 
+// Two levels in one pass: out[t] = round_OUT( sum_m f32( round_SRC( sum_i src[inner[outer[t, m], i]] ) ) ), both sums in
+// fp32 in table order, entries outside their range skipped.  This is, bit for bit, combine(src, inner) rounded to the
+// source dtype followed by combine(that, outer) -- the reference's two index_add levels
+// (terrace/ta2a_dispatch.py:483-494) -- without the [n_rows, H] plane between them ever reaching memory.  The inner
+// table is Q ids wide; a wave works on 8 / Q outer entries at a time, so about eight row loads are in flight.
+template <int SRC>
+__device__ __forceinline__ float round_to_src(float x) {
+    if constexpr (SRC == TERRACE_F32) return x;
+    else if constexpr (SRC == TERRACE_BF16) return __uint_as_float(f32_to_bf16_bits(x) << 16);
+    else return __half2float(__float2half_rn(x));
+}
+
+template <int SRC, int OUT, int Q>
+__global__ __launch_bounds__(kBlock) void combine2_kernel(const uint8_t *__restrict__ src, int64_t src_row_bytes,
+                                                          const int64_t *__restrict__ inner, int64_t n_rows,
+                                                          const int64_t *__restrict__ outer, int fan_outer,
+                                                          int64_t hidden, uint8_t *__restrict__ out,
+                                                          int64_t out_row_bytes, int slices, int64_t n_src) {
+    constexpr int N = Chunk<SRC>::N;
+    constexpr int MB = 8 / Q;
+    const int64_t t = blockIdx.x / slices;
+    const int64_t c = (int64_t)(blockIdx.x - t * slices) * blockDim.x + threadIdx.x;
+    if (c >= hidden / N) return;
+    float total[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) total[i] = 0.0f;
+    const int64_t *outer_row = outer + t * fan_outer;
+    for (int m0 = 0; m0 < fan_outer; m0 += MB) {
+        int64_t r[MB], from[MB][Q];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) r[b] = m0 + b < fan_outer ? outer_row[m0 + b] : -1;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+#pragma unroll
+            for (int i = 0; i < Q; ++i) from[b][i] = -1;
+            if (row_in(r[b], n_rows)) {
+#pragma unroll
+                for (int i = 0; i < Q; ++i) from[b][i] = inner[r[b] * Q + i];
+            }
+        }
+        u32x4 raw[MB][Q];
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+#pragma unroll
+            for (int i = 0; i < Q; ++i) {
+                raw[b][i] = zero_of<u32x4>();
+                if (row_in(from[b][i], n_src))               // wave-uniform: a dead entry touches no memory
+                    raw[b][i] = ld_stream((const u32x4 *)(src + from[b][i] * src_row_bytes) + c);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            if (!row_in(r[b], n_rows)) continue;             // wave-uniform
+            float acc[N];
+#pragma unroll
+            for (int i = 0; i < N; ++i) acc[i] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < Q; ++i) {
+                float f[N];
+                decode_chunk<SRC>(raw[b][i], f);             // a dead entry decodes to +0.0, which changes no sum
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[e] = __fadd_rn(acc[e], f[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < N; ++e) total[e] = __fadd_rn(total[e], round_to_src<SRC>(acc[e]));
+        }
+    }
+    store_chunk<OUT, N>(out + t * out_row_bytes, c * N, total);
+}
+
 // Element path: any hidden, any alignment.
 __device__ __forceinline__ float load_elem(const uint8_t *row, int src_dtype, int64_t e, int64_t hidden) {
     switch (src_dtype) {
@@ -900,6 +970,54 @@ int launch_combine(const void *src, int64_t n_src, int src_dtype, const int64_t 
         default: launch_combine_s<TERRACE_FP8_E4M3_B128>(src, n_src, idx, w, w_dtype, n_out, fan, hidden, out, out_dtype, srb, s); break;
     }
     return check_launch();
+}
+
+template <int SRC, int OUT>
+static int launch_combine2_so(const void *src, int64_t n_src, const int64_t *inner, int64_t n_rows, int fan_inner,
+                              const int64_t *outer, int64_t n_out, int fan_outer, int64_t hidden, void *out,
+                              hipStream_t s) {
+    const int64_t chunks = hidden / Chunk<SRC>::N;
+    const int64_t srb = dtype_row_bytes(SRC, hidden), orb = dtype_row_bytes(OUT, hidden);
+    const bool one_wave = chunks % kWave == 0 && n_out * (chunks / kWave) <= kMaxBlocks;
+    const int bt = one_wave ? kWave : kBlock;
+    const int slices = (int)((chunks + bt - 1) / bt);
+    const unsigned grid = (unsigned)(n_out * slices);
+#define TERRACE_C2(Q)                                                                                              \
+    combine2_kernel<SRC, OUT, Q><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, inner, n_rows, outer, fan_outer, hidden, \
+                                                     (uint8_t *)out, orb, slices, n_src)
+    switch (fan_inner) {
+        case 1: TERRACE_C2(1); break;
+        case 2: TERRACE_C2(2); break;
+        case 4: TERRACE_C2(4); break;
+        case 8: TERRACE_C2(8); break;
+        default: return TERRACE_EINVAL;
+    }
+#undef TERRACE_C2
+    return check_launch();
+}
+
+// Vector path only: float rows (f32 / bf16 / f16) that are 16-byte multiples on 16-byte-aligned buffers, inner
+// tables 1, 2, 4 or 8 ids wide.  Anything else returns TERRACE_EINVAL and the caller runs the two levels one by one.
+int launch_combine2(const void *src, int64_t n_src, int src_dtype, const int64_t *inner, int64_t n_rows, int fan_inner,
+                    const int64_t *outer, int64_t n_out, int fan_outer, int64_t hidden, void *out, int out_dtype,
+                    hipStream_t s) {
+    if (n_out <= 0 || hidden <= 0) return TERRACE_OK;
+    if (src_dtype != TERRACE_F32 && src_dtype != TERRACE_BF16 && src_dtype != TERRACE_F16) return TERRACE_EINVAL;
+    if (out_dtype != TERRACE_F32 && out_dtype != TERRACE_BF16 && out_dtype != TERRACE_F16) return TERRACE_EINVAL;
+    if (fan_outer <= 0 || n_rows < 0 || n_src < 0) return TERRACE_EINVAL;
+    if (n_out * ((hidden + 1023) / 1024 + 1) > kMaxGridRows) return TERRACE_EINVAL;
+    const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
+    const int n = src_dtype == TERRACE_F32 ? 4 : 8;
+    if (hidden % n || ((uintptr_t)src & 15) || ((uintptr_t)out & 15) || srb % 16 || orb % 16) return TERRACE_EINVAL;
+    if (!inner || !outer || !out || (!src && n_src > 0)) return TERRACE_EINVAL;
+#define TERRACE_C2O(S)                                                                                             \
+    (out_dtype == TERRACE_F32    ? launch_combine2_so<S, TERRACE_F32>(src, n_src, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out, s) \
+     : out_dtype == TERRACE_BF16 ? launch_combine2_so<S, TERRACE_BF16>(src, n_src, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out, s) \
+                                 : launch_combine2_so<S, TERRACE_F16>(src, n_src, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out, s))
+    if (src_dtype == TERRACE_F32) return TERRACE_C2O(TERRACE_F32);
+    if (src_dtype == TERRACE_BF16) return TERRACE_C2O(TERRACE_BF16);
+    return TERRACE_C2O(TERRACE_F16);
+#undef TERRACE_C2O
 }
 
 int launch_copy(const void *x, void *y, size_t nbytes, hipStream_t s) {

@@ -64,6 +64,7 @@ SIGNATURES = {
     "terrace_index_chain2": (_I, [_P, _L, _P, _L, _P, _L, _P, _P]),
     "terrace_combine": (_I, [_P, _L, _I, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
     "terrace_combine_pitched": (_I, [_P, _L, _I, _L, _P, _P, _I, _L, _I, _L, _P, _I, _P]),
+    "terrace_combine_two_level": (_I, [_P, _L, _I, _P, _L, _I, _P, _L, _I, _L, _P, _I, _P]),
     "terrace_pack_planes": (_I, [_P, _L, _P, _L, _P, _L, _L, _L, _P, _P]),
     "terrace_unpack_planes": (_I, [_P, _L, _L, _P, _L, _P, _L, _P, _L, _P]),
     "terrace_k2_pack_wire": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _I, _I, _I,

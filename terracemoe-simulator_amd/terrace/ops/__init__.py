@@ -324,10 +324,11 @@ def k2_pack_wire(hidden, expert_idx, gates, world, n_experts, rpn, groups_m):
     return (payload, mask, gate_rows, u_src, node_counts), ex
 
 
-def k1_arrival_wire(rx, rwire, gate_dtype, quota, epr, rpn, my_local=0):
+def k1_arrival_wire(rx, rwire, gate_dtype, quota, epr, rpn, my_local=0, want_slot_idx=False):
     """The arrival chain reading an arrived Hop-A small container and writing the Hop-B container:
     (send_buf, meta [P,2] int64, r_idx, i_send, pair_pos); ``meta[:, 0]`` is slot_idx and the first
-    element of word 1 (viewed in ``gate_dtype``) is gate_pairs."""
+    element of word 1 (viewed in ``gate_dtype``) is gate_pairs.  ``want_slot_idx`` appends slot_idx as a dense [P]
+    plane of its own (the same kernel writes it; a caller that needs it contiguous saves a strided copy)."""
     _require()
     _hip.need_device(rx, rwire)
     if rx.dim() != 2 or rwire.dim() != 2 or rwire.dtype != torch.int64 or rwire.shape[0] != rx.shape[0]:
@@ -347,11 +348,15 @@ def k1_arrival_wire(rx, rwire, gate_dtype, quota, epr, rpn, my_local=0):
     r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
     pair_pos = torch.empty((P,), dtype=torch.int64, device=dev)
+    slot_idx = torch.empty((P,), dtype=torch.int64, device=dev) if want_slot_idx else None
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_k1_arrival_workspace", R, quota, rpn), dev)
     _hip.call("terrace_k1_arrival_wire", _hip.ptr(rx), _hip.ptr(rwire), rwire.shape[1], R, H * rx.element_size(), gb,
-              quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(meta), _hip.ptr(r_idx), None, None,
+              quota, epr, rpn, my_local, _hip.ptr(send_buf), _hip.ptr(meta), _hip.ptr(r_idx),
+              _hip.ptr(slot_idx) if want_slot_idx else None, None,
               _hip.ptr(i_send), _hip.ptr(pair_pos), _hip.ptr(st), _hip.ptr(ws), ws.numel(), _hip.stream(dev))
+    if want_slot_idx:
+        return send_buf, meta, r_idx, i_send, pair_pos, slot_idx
     return send_buf, meta, r_idx, i_send, pair_pos
 
 
@@ -715,6 +720,32 @@ def combine(src, idx, weights=None, out_dtype=None, fp8_hidden=None):
     pitch = 0 if src.is_contiguous() else src.stride(0) * src.element_size()
     _hip.call("terrace_combine_pitched", _hip.ptr(src), src.shape[0], src_code, pitch, _hip.ptr(idx), _hip.ptr(weights),
               w_code, n_out, fan, hidden, _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
+    return out
+
+
+def combine_two_level(src, inner, outer, out_dtype=None):
+    """``combine(combine(src, inner, out_dtype=src.dtype), outer, out_dtype=out_dtype)`` -- the reference's two
+    ``index_add`` levels, each an fp32 sum rounded once -- bit for bit, in one pass when the shape allows it (the
+    ``[len(inner), H]`` plane between the levels is then never written): float rows that are 16-byte multiples and an
+    inner table 1, 2, 4 or 8 ids wide; any other shape runs the two levels one after the other."""
+    _require()
+    _hip.need_device(src, inner, outer)
+    if inner.dim() != 2 or outer.dim() != 2 or inner.dtype != torch.int64 or outer.dtype != torch.int64:
+        raise RuntimeError("combine_two_level: inner and outer must be 2-D int64 tables")
+    out_dtype = out_dtype or src.dtype
+    fused = (src.dim() == 2 and src.is_contiguous() and src.dtype in (torch.float32, torch.bfloat16, torch.float16)
+             and out_dtype in (torch.float32, torch.bfloat16, torch.float16)
+             and inner.shape[1] in (1, 2, 4, 8) and outer.shape[1] >= 1
+             and (src.shape[1] * src.element_size()) % 16 == 0
+             and (src.shape[1] * torch.empty((), dtype=out_dtype).element_size()) % 16 == 0
+             and src.data_ptr() % 16 == 0)
+    if not fused:
+        return combine(combine(src, inner, None, out_dtype=src.dtype), outer, None, out_dtype=out_dtype)
+    inner, outer = inner.contiguous(), outer.contiguous()
+    out = torch.empty((outer.shape[0], src.shape[1]), dtype=out_dtype, device=src.device)
+    _hip.call("terrace_combine_two_level", _hip.ptr(src), src.shape[0], _hip.float_code(src.dtype), _hip.ptr(inner),
+              inner.shape[0], inner.shape[1], _hip.ptr(outer), outer.shape[0], outer.shape[1], src.shape[1],
+              _hip.ptr(out), _hip.float_code(out_dtype), _hip.stream(src.device))
     return out
 
 

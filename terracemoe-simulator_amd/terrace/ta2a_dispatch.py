@@ -90,8 +90,7 @@ class _UnpermuteFn(torch.autograd.Function):
     def forward(ctx, expert_out, red_table, tok_table, where, out_dtype):
         ctx.save_for_backward(where)
         ctx.n_places, ctx.dtype = expert_out.shape[0], expert_out.dtype
-        red = _ops.combine(expert_out, red_table, None, out_dtype=expert_out.dtype)
-        return _ops.combine(red, tok_table, None, out_dtype=out_dtype)
+        return _ops.combine_two_level(expert_out, red_table, tok_table, out_dtype=out_dtype)
 
     @staticmethod
     def backward(ctx, gy):
@@ -159,9 +158,8 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
 
     if fused_wire:
         # Hop B (loop-back): the container the arrival kernel wrote is what the expert card reads
-        node_rx, my_meta, r_idx, _i_send, pair_pos = _ops.k1_arrival_wire(rx, rwire, gates.dtype, quota, epr, rpn,
-                                                                          my_local)
-        my_slot = my_meta[:, 0]
+        node_rx, my_meta, r_idx, _i_send, pair_pos, my_slot = _ops.k1_arrival_wire(
+            rx, rwire, gates.dtype, quota, epr, rpn, my_local, want_slot_idx=True)   # = my_meta[:, 0], dense
         permuted, order, tokens_per_expert, place, pprobs = _ops.regroup_wire(node_rx, my_meta, gates.dtype, slots, 0)
     else:
         if quota is not None:
@@ -211,8 +209,9 @@ def ta2a_unpermute(expert_out, st: TA2AState, out_like):
     _hip.need_device(expert_out)
     if torch.is_grad_enabled() and expert_out.requires_grad:
         return _UnpermuteFn.apply(expert_out, st.red_table, st.tok_table, st.where, out_like.dtype)
-    red = _ops.combine(expert_out, st.red_table, None, out_dtype=expert_out.dtype)
-    return _ops.combine(red, st.tok_table, None, out_dtype=out_like.dtype)
+    # loop-back: no exchange stands between the two levels, so one pass computes both (same bits, and the [R, H]
+    # plane of per-row sums never reaches memory)
+    return _ops.combine_two_level(expert_out, st.red_table, st.tok_table, out_dtype=out_like.dtype)
 
 
 # --------------------------------------------------------------------------------------

@@ -155,8 +155,12 @@ def test_routing_map_to_topk_and_refusals():
     from terrace.ta2a_dispatch import routing_map_to_topk
     announce("routing_map_to_topk")
     rng = np.random.default_rng(2)
+    # E = 24 and 300 take the byte-per-lane census, the others the 16-byte one at every lanes-per-token it has
+    # (E/16 = 1 .. 64), with token counts that leave the last wave ragged
     for T, E, k, dt in [(19, 24, 5, torch.float32), (1000, 256, 8, torch.bfloat16), (64, 64, 64, torch.float16),
-                        (3, 300, 2, torch.float32)]:
+                        (3, 300, 2, torch.float32), (130, 16, 3, torch.float32), (77, 32, 5, torch.bfloat16),
+                        (1031, 128, 8, torch.float32), (65, 512, 9, torch.float16), (33, 1024, 4, torch.float32),
+                        (4099, 64, 4, torch.float32)]:
         e = np.sort(np.stack([rng.permutation(E)[:k] for _ in range(T)]), 1)
         rm = np.zeros((T, E), dtype=bool)
         rm[np.arange(T)[:, None], e] = True
@@ -164,6 +168,15 @@ def test_routing_map_to_topk_and_refusals():
         ge, gg = routing_map_to_topk(torch.from_numpy(rm).to(DEV), probs.to(DEV))
         we, wg = orc.routing_map_to_topk(rm, to_np(probs))
         same(ge, we, "expert_idx"), same(gg, wg, "gates")
+        # a byte map: any non-zero byte means chosen (0x80 and 0xFF included)
+        rm8 = rm.astype(np.uint8) * rng.choice(np.array([1, 2, 0x7F, 0x80, 0xFF], dtype=np.uint8), size=rm.shape)
+        ge, gg = routing_map_to_topk(torch.from_numpy(rm8).to(DEV), probs.to(DEV))
+        same(ge, we, "expert_idx (byte map)"), same(gg, wg, "gates (byte map)")
+        if T > 1 and k > 1:          # one token short of an expert, somewhere in the middle
+            bad = rm.copy()
+            bad[T // 2, e[T // 2, 0]] = False
+            with pytest.raises(RuntimeError, match="exactly k experts"):
+                routing_map_to_topk(torch.from_numpy(bad).to(DEV), probs.to(DEV))
     bad = rm.copy()
     bad[1, e[1, 0]] = False
     with pytest.raises(RuntimeError, match="exactly k experts"):
@@ -485,3 +498,49 @@ def test_overlap_seam_switches(monkeypatch):
                             run_shared_experts=lambda: calls.append(len(save)))
     assert calls == [7]
     td.reset_shared_overlap()
+
+
+# ---------------------------------------------------------------------------------------------
+# the two combine levels in one pass (terrace_combine_two_level)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt,out_fmt", [("f32", "f32"), ("bf16", "bf16"), ("f16", "f16"), ("bf16", "f32"),
+                                         ("f32", "bf16")])
+@pytest.mark.parametrize("q,M,H", [(1, 3, 64), (2, 4, 512), (4, 2, 1024), (8, 1, 72), (2, 5, 8), (4, 9, 520)])
+def test_two_level_combine_in_one_pass(fmt, out_fmt, q, M, H):
+    """Against the oracle's two fp32 levels (round to the source format between them) and against the two launches,
+    bit for bit: tables with dead entries at both levels (negative and past-the-end ids), outer fans that do not fill
+    the last batch of rows, widths on the one-wave and the 256-lane shape."""
+    import terrace.ops as tops
+    announce("two-level combine", fmt, out_fmt, (q, M, H))
+    rng = np.random.default_rng(q * 100 + M)
+    n_src, R, T = 301, 97, 53
+    src = torch.from_numpy(rng.standard_normal((n_src, H)).astype(np.float32)).to(DT[fmt])
+    inner = rng.integers(0, n_src, size=(R, q)).astype(np.int64)
+    inner[rng.random((R, q)) < 0.15] = -1
+    inner[3, 0] = n_src + 5                     # past the end: dead
+    outer = rng.integers(0, R, size=(T, M)).astype(np.int64)
+    outer[rng.random((T, M)) < 0.2] = -1
+    outer[7, 0] = R                             # past the end: dead
+    outer[11, :] = -1                           # a token with no rows at all: a zero row
+    want_red = orc.combine(to_np(src), np.where((inner >= 0) & (inner < n_src), inner, -1), None, fmt, fmt)
+    want = orc.combine(want_red, np.where((outer >= 0) & (outer < R), outer, -1), None, fmt, out_fmt)
+    sd, ind, outd = src.to(DEV), torch.from_numpy(inner).to(DEV), torch.from_numpy(outer).to(DEV)
+    got = tops.combine_two_level(sd, ind, outd, out_dtype=DT[out_fmt])
+    same(got, want, "one pass vs the oracle's two levels")
+    two = tops.combine(tops.combine(sd, ind, None, out_dtype=sd.dtype), outd, None, out_dtype=DT[out_fmt])
+    assert torch.equal(got.view(torch.uint8), two.view(torch.uint8)), "one pass differs from the two launches"
+
+
+def test_two_level_combine_shapes_outside_the_one_pass_form():
+    """An inner table three ids wide, and rows that are not 16-byte multiples: the operator runs the two levels one
+    after the other and gives the same definition."""
+    import terrace.ops as tops
+    announce("two-level combine, fallback shapes")
+    rng = np.random.default_rng(5)
+    for q, H in [(3, 64), (2, 7)]:
+        src = torch.from_numpy(rng.standard_normal((40, H)).astype(np.float32))
+        inner = rng.integers(-1, 40, size=(19, q)).astype(np.int64)
+        outer = rng.integers(-1, 19, size=(11, 2)).astype(np.int64)
+        want = orc.combine(orc.combine(to_np(src), inner, None, "f32", "f32"), outer, None, "f32", "f32")
+        got = tops.combine_two_level(src.to(DEV), torch.from_numpy(inner).to(DEV), torch.from_numpy(outer).to(DEV))
+        same(got, want, f"fallback q={q} H={H}")
