@@ -137,8 +137,9 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         _plan._guard(ex["status"], T, k, n_nodes, groups_m)
         u_node = ex["u_node"]
     else:
+        token_rows = []
         payload, mask, gate_rows, u_src, node_counts, _inverse, u_node = general_hopa_planes(
-            hidden_states, expert_idx, gates, world, n_experts, rpn)
+            hidden_states, expert_idx, gates, world, n_experts, rpn, token_rows_out=token_rows)
 
     # Hop A (loop-back): what was packed for the wire is what arrives
     if fused_wire:
@@ -189,7 +190,7 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
     else:
         per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
         st.red_table = _ops.index_chain(place, per_row)
-        st.tok_table, _ = _ops.segment_table(u_src, T, min(k, n_nodes))
+        st.tok_table = token_rows[0]
     st.where, st.token_of_place = _ops.pair_places(order, r_idx, my_slot, u_src, u_node, expert_idx, slots)
     if torch.is_grad_enabled():
         if hidden_states.requires_grad:
@@ -393,9 +394,10 @@ def ta2a_permute_overlap(hidden_states, probs, routing_map, *, world, rank, rpn,
                 by_col = torch.empty_like(ex["pair_table"]).scatter_(1, ex["sort_order"], ex["pair_table"])
                 gate_rows = _SparseGateRowsEdge.apply(gates_p, by_col.reshape(-1), gate_rows)
         else:
+            token_rows = []
             payload, mask, gate_rows, u_src, node_counts, inverse, u_node = general_hopa_planes(
-                h.detach(), expert_idx, gates_p.detach(), world, n_experts, rpn)
-            tok_table, _ = _ops.segment_table(u_src, T, min(k, n_nodes))
+                h.detach(), expert_idx, gates_p.detach(), world, n_experts, rpn, token_rows_out=token_rows)
+            tok_table = token_rows[0]
             if gates_p.requires_grad:
                 cells = inverse.view(T, k) * slots + expert_idx % slots
                 gate_rows = _SparseGateRowsEdge.apply(gates_p, cells.reshape(-1), gate_rows)

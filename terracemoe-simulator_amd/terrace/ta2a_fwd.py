@@ -86,10 +86,15 @@ def build_expansion(expert_idx, inverse, n_rows: int, world: int, n_experts: int
     return mask
 
 
-def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8):
+def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: int = 8, token_rows_out=None):
     """Send side of the general (non-quota) branch: (payload, mask, gate_rows, u_src,
     node_counts, inverse, u_node) with ``mask`` the [n_rows] int64 bitmask plane and ``gate_rows``
-    the sparse [n_rows, slots] plane in the payload dtype."""
+    the sparse [n_rows, slots] plane in the payload dtype.
+
+    The payload ``x[u_src]`` is moved as a scatter over the token -> send rows table (each token's row is read once
+    and written to its rows) rather than as a gather that reads a token's row once per copy; a list passed as
+    ``token_rows_out`` receives that [T, min(k, n_nodes)] table (-1 padded), which is also the second level of the
+    combine."""
     from .ta2a import plan_ta2a
     slots = (n_experts // world) * rpn
     if gates.dtype != x.dtype:
@@ -97,7 +102,11 @@ def general_hopa_planes(x, expert_idx, gates, world: int, n_experts: int, rpn: i
                            f"for the destination and {gates.dtype} for the source.")
     u_src, u_node, node_counts, inverse = plan_ta2a(expert_idx, world, n_experts, rpn, groups_m=None)
     n_rows = u_src.numel()
-    payload = _ops.gather_rows(x, u_src)
+    T, k = expert_idx.shape
+    token_rows, _ = _ops.segment_table(u_src, T, min(k, world // rpn))
+    if token_rows_out is not None:
+        token_rows_out.append(token_rows)
+    payload = _ops.scatter_rows(x, token_rows, n_rows)
     mask = build_expansion(expert_idx, inverse, n_rows, world, n_experts, rpn)
     gate_rows = torch.zeros((n_rows, slots), dtype=x.dtype, device=x.device)
     _ops.scatter_elems(gates, inverse, expert_idx, gate_rows, col_mod=slots)
