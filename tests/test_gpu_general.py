@@ -107,7 +107,9 @@ def test_expand_arrival_both_forms(slots):
 
 
 @pytest.mark.parametrize("R,slots,epr,rpn,H,fmt", [(30, 12, 3, 4, 5, "f32"), (700, 32, 4, 8, 64, "bf16"),
-                                                    (1, 8, 1, 8, 16, "f16"), (4096, 16, 2, 8, 512, "bf16")])
+                                                    (1, 8, 1, 8, 16, "f16"), (4096, 16, 2, 8, 512, "bf16"),
+                                                    # whole-kilobyte rows of other widths
+                                                    (257, 8, 1, 8, 256, "f32"), (300, 32, 4, 8, 1536, "bf16")])
 def test_arrival_pairs_general(R, slots, epr, rpn, H, fmt):
     import terrace.ops as tops
     announce("arrival_pairs", R, slots, epr, rpn, H, fmt)
@@ -126,6 +128,31 @@ def test_arrival_pairs_general(R, slots, epr, rpn, H, fmt):
     z = torch.zeros(0, dtype=torch.int64, device=DEV)
     out = tops.arrival_pairs(rx.to(DEV), z, z, rgate.to(DEV), epr, rpn)
     assert out[0].shape == (0, H) and out[4].tolist() == [0] * rpn
+
+
+@pytest.mark.parametrize("H", [256, 24])
+def test_arrival_pairs_row_ids_out_of_range_give_zero_rows(H):
+    """A pair naming a row that did not arrive: its place holds a zero row, whichever gather kernel the row width
+    takes (whole kilobytes at H = 256 floats, 96-byte rows at H = 24)."""
+    import terrace.ops as tops
+    from terrace import _hip
+    announce("arrival_pairs bad rows", H)
+    R, epr, rpn = 50, 2, 4
+    rng = np.random.default_rng(H)
+    r = np.sort(rng.integers(0, R, size=180)).astype(np.int64)
+    c = rng.integers(0, epr * rpn, size=180).astype(np.int64)
+    bad = rng.random(180) < 0.1
+    r[bad] = np.where(rng.random(bad.sum()) < 0.5, -1, R + 7)
+    rx = torch.randn(R, H, generator=torch.Generator().manual_seed(1))
+    send, _gp, r_idx, slot_idx, i_send, ordo = tops.arrival_pairs(rx.to(DEV), torch.from_numpy(r).to(DEV),
+                                                                  torch.from_numpy(c).to(DEV), None, epr, rpn)
+    order = np.argsort(c // epr, kind="stable")
+    same(ordo, order.astype(np.int64), "ordo"), same(r_idx, r[order], "r_idx"), same(slot_idx, c[order], "slot_idx")
+    want = np.zeros((180, H), dtype=np.float32)
+    ok = (r[order] >= 0) & (r[order] < R)
+    want[ok] = rx.numpy()[r[order][ok]]
+    same(send, want, "send_buf")
+    assert int(i_send.sum()) == 180
 
 
 def test_segment_table_lists_items_in_ascending_order():
