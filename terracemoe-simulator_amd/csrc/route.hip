@@ -421,7 +421,9 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
                 float cv = kNegInf;
                 int ci = 0x7FFFFFFF;
                 for (int c = lane; c < M * g; c += kWave) {
-                    const float v = s[selg[c / g] * g + c % g];
+                    const int G = selg[c / g];
+                    if ((unsigned)G >= (unsigned)n_groups) continue;     // a rank no group took (NaN group scores)
+                    const float v = s[G * g + c % g];
                     if (after(v, c, pv, pi) && ahead(v, c, cv, ci)) {
                         cv = v;
                         ci = c;
@@ -430,7 +432,9 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
                 wave_best(cv, ci);
                 pv = cv;
                 pi = ci;
-                if (lane == 0) sel[j] = selg[ci / g] * g + ci % g;
+                // no candidate left (NaN scores are never ranked): an id no expert has, which the epilogue turns
+                // into expert 0 as in the other modes -- and no read of selg[] at a position that does not exist
+                if (lane == 0) sel[j] = ci == 0x7FFFFFFF ? 0x7FFFFFFF : selg[ci / g] * g + ci % g;
             }
             for (int m = lane; m < M; m += kWave) group_idx[t * n_group_out + m] = selg[m];
         } else {

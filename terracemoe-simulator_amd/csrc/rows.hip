@@ -1009,7 +1009,7 @@ int launch_combine2(const void *src, int64_t n_src, int src_dtype, const int64_t
     const int64_t srb = dtype_row_bytes(src_dtype, hidden), orb = dtype_row_bytes(out_dtype, hidden);
     const int n = src_dtype == TERRACE_F32 ? 4 : 8;
     if (hidden % n || ((uintptr_t)src & 15) || ((uintptr_t)out & 15) || srb % 16 || orb % 16) return TERRACE_EINVAL;
-    if (!inner || !outer || !out || (!src && n_src > 0)) return TERRACE_EINVAL;
+    if ((!inner && n_rows > 0) || !outer || !out || (!src && n_src > 0)) return TERRACE_EINVAL;
 #define TERRACE_C2O(S)                                                                                             \
     (out_dtype == TERRACE_F32    ? launch_combine2_so<S, TERRACE_F32>(src, n_src, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out, s) \
      : out_dtype == TERRACE_BF16 ? launch_combine2_so<S, TERRACE_BF16>(src, n_src, inner, n_rows, fan_inner, outer, n_out, fan_outer, hidden, out, s) \

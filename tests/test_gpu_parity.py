@@ -263,6 +263,34 @@ def test_route_contains_nan_scores(generic):
     assert np.array_equal(to_np(grp)[ok.numpy()], ogrp[ok.numpy()])
 
 
+@pytest.mark.parametrize("mode", ["full", "group_limited", "quota_only", "global_topk"])
+@pytest.mark.parametrize("E,Ng,k,M", [(8, 8, 8, 8), (64, 8, 8, 4), (48, 6, 6, 3)])
+def test_route_nan_rows_are_contained_and_repeatable_in_every_mode(mode, E, Ng, k, M):
+    """A token whose scores are all NaN ranks nothing: in every mode its ids must be valid experts, the same on every
+    run (what is written must not depend on what a workgroup's LDS held), and the tokens beside it untouched."""
+    import terrace
+    announce("route nan, every mode", mode, (E, Ng, k, M))
+    T = 300
+    g = torch.Generator().manual_seed(E + k)
+    logits = torch.randn(T, E, generator=g)
+    poisoned = logits.clone()
+    poisoned[3] = float("nan")
+    poisoned[77, ::2] = float("nan")
+    zero = torch.zeros(E)
+    cfg = terrace.TRouteConfig(E, Ng, k, M)
+    runs = [terrace.t_route(poisoned.to(DEV), zero.to(DEV), cfg, mode) for _ in range(3)]
+    torch.cuda.synchronize()
+    e, gt, grp = runs[0]
+    assert bool(((e >= 0) & (e < E)).all())
+    for e2, gt2, grp2 in runs[1:]:
+        assert torch.equal(e, e2) and torch.equal(grp, grp2)
+        assert torch.equal(gt.view(torch.int32), gt2.view(torch.int32))
+    oe, og, _ = orc.t_route(logits.numpy(), zero.numpy(), E, Ng, k, M, mode=mode)
+    ok = np.ones(T, dtype=bool)
+    ok[[3, 77]] = False
+    assert np.array_equal(to_np(e)[ok], oe[ok]) and np.array_equal(to_np(gt)[ok], og[ok])
+
+
 def test_expert_load_and_hist_and_argsort():
     import terrace
     from terrace.ta2a_fwd import _stable_argsort_small, fixed_hist
