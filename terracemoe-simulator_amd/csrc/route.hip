@@ -394,6 +394,10 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
         if (mode == TERRACE_ROUTE_FULL || mode == TERRACE_ROUTE_QUOTA_ONLY) {
             for (int m = 0; m < n_sel_groups; ++m) {
                 const int G = selg[m];
+                if ((unsigned)G >= (unsigned)n_groups) {      // a rank no group took (NaN group scores): no scores to
+                    for (int i = lane; i < per_group; i += kWave) sel[m * per_group + i] = 0x7FFFFFFF;   // read
+                    continue;
+                }
                 float pv = kPosInf;
                 int pi = -1;
                 for (int i = 0; i < per_group; ++i) {
@@ -409,7 +413,7 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
                     wave_best(cv, ci);
                     pv = cv;
                     pi = ci;
-                    if (lane == 0) sel[m * per_group + i] = G * g + ci;
+                    if (lane == 0) sel[m * per_group + i] = ci == 0x7FFFFFFF ? 0x7FFFFFFF : G * g + ci;
                 }
             }
             for (int m = lane; m < n_sel_groups; m += kWave) group_idx[t * n_group_out + m] = selg[m];
@@ -455,7 +459,7 @@ __global__ __launch_bounds__(kBlock) void route_generic_kernel(const float *__re
                 pi = ci;
                 if (lane == 0) {
                     sel[j] = ci;
-                    group_idx[t * n_group_out + j] = ci / g;
+                    group_idx[t * n_group_out + j] = ci == 0x7FFFFFFF ? 0x7FFFFFFF : ci / g;   // nothing ranked: no group
                 }
             }
         }

@@ -282,6 +282,7 @@ def test_route_nan_rows_are_contained_and_repeatable_in_every_mode(mode, E, Ng, 
     torch.cuda.synchronize()
     e, gt, grp = runs[0]
     assert bool(((e >= 0) & (e < E)).all())
+    assert bool(((grp >= 0) & (grp < Ng) | (grp == 0x7FFFFFFF)).all())      # a group, or the no-group sentinel
     for e2, gt2, grp2 in runs[1:]:
         assert torch.equal(e, e2) and torch.equal(grp, grp2)
         assert torch.equal(gt.view(torch.int32), gt2.view(torch.int32))
