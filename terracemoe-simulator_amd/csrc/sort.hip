@@ -36,11 +36,13 @@ Units make_units(int64_t n_items, int n_buckets) {
     u.n_buckets = n_buckets;
     // Unit size.  A chunk more per wave costs the count and rank passes about 1 us; more units cost the direct
     // path more workgroup totals to re-read and the scan path a larger table (16K entries 5.5 us, 64K entries
-    // 12 us).  One chunk per wave up to 2048 units, then four, then sixteen; when even that leaves a table
-    // the scan path must take, the scan path's own limits (16K / 64K entries) choose.
+    // 12 us).  One chunk per wave up to 4096 units, then four, then sixteen (at 262144 items one chunk per wave
+    // measured 8 us a step better than four, arrival and regroup together; at 524288 items one and four measured the
+    // same); when even that leaves a table the scan path must take, the scan path's own limits (16K / 64K entries)
+    // choose.
     u.chunks = 16;
     for (int c : {1, 4}) {
-        if ((n_items + 64 * c - 1) / (64 * c) <= 2048) {
+        if ((n_items + 64 * c - 1) / (64 * c) <= 4096) {
             u.chunks = c;
             break;
         }
