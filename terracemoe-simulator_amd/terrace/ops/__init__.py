@@ -865,10 +865,13 @@ def expand_mask(rmask, slots, quota=None):
     return r_idx, slot_idx
 
 
-def arrival_pairs(rx, r_in, slot_in, rgate, epr, rpn):
+def arrival_pairs(rx, r_in, slot_in, rgate, epr, rpn, move=True):
     """Arrival chain over an explicit pair list (the general branch):
     (send_buf, gate_pairs, r_idx, slot_idx, i_send, ordo) with pairs in stable owner-card order
-    and ``gate_pairs = rgate[r_idx, slot_idx]`` looked up in the sparse [R, width] plane."""
+    and ``gate_pairs = rgate[r_idx, slot_idx]`` looked up in the sparse [R, width] plane.
+
+    ``move=False``: the index planes only (``send_buf`` is None), for a caller that moves the rows itself -- a scatter
+    over the per-row table of ``r_idx`` reads each arrived row once, where this call's gather reads it once per pair."""
     _require()
     _hip.need_device(rx, r_in, slot_in, rgate)
     rx, r_in, slot_in = rx.contiguous(), r_in.contiguous().reshape(-1), slot_in.contiguous().reshape(-1)
@@ -886,14 +889,14 @@ def arrival_pairs(rx, r_in, slot_in, rgate, epr, rpn):
             raise RuntimeError("arrival_pairs: rgate must be a [R, width] plane of 2- or 4-byte elements")
         gate_bytes, width = rgate.element_size(), rgate.shape[1]
         gate_pairs = torch.empty((P,), dtype=rgate.dtype, device=dev)
-    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev)
+    send_buf = torch.empty((P, H), dtype=rx.dtype, device=dev) if move else None
     r_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     slot_idx = torch.empty((P,), dtype=torch.int64, device=dev)
     ordo = torch.empty((P,), dtype=torch.int64, device=dev)
     i_send = torch.empty((rpn,), dtype=torch.int64, device=dev)
     st = _hip.new_status(dev)
     ws = _hip.workspace(_hip.query("terrace_arrival_pairs_workspace", P, rpn), dev)
-    _hip.call("terrace_arrival_pairs", _hip.ptr(rx), _hip.ptr(r_in), _hip.ptr(slot_in), _hip.ptr(rgate), R, P,
+    _hip.call("terrace_arrival_pairs", _hip.ptr(rx) if move else None, _hip.ptr(r_in), _hip.ptr(slot_in), _hip.ptr(rgate), R, P,
               H * rx.element_size(), gate_bytes, width, epr, rpn, _hip.ptr(send_buf), _hip.ptr(gate_pairs),
               _hip.ptr(r_idx), _hip.ptr(slot_idx), _hip.ptr(i_send), _hip.ptr(ordo), _hip.ptr(st), _hip.ptr(ws),
               ws.numel(), _hip.stream(dev))

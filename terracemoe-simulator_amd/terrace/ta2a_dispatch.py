@@ -168,7 +168,12 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
                 rx, rmask, rgate, quota, epr, rpn, my_local, want_pair_pos=True)
         else:
             r_in, s_in = _expand_arrival(rmask, slots, None)
-            exp_rx, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx, r_in, s_in, rgate, epr, rpn)
+            # index planes first, then the rows as a scatter over the per-row table of arrival positions (which the
+            # combine's first level needs anyway): each arrived row is read once, not once per pair
+            _none, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx, r_in, s_in, rgate, epr, rpn,
+                                                                                   move=False)
+            per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
+            exp_rx = _ops.scatter_rows(rx, per_row, r_idx.numel())
         # Hop B (loop-back)
         node_rx = exp_rx
         if pack_mode != "off":
@@ -188,7 +193,6 @@ def ta2a_permute(hidden_states, probs, routing_map, *, world, rank, rpn, n_exper
         st.red_table = _ops.index_chain(place, pair_pos).view(R, quota)
         st.tok_table = ex["token_rows"]
     else:
-        per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
         st.red_table = _ops.index_chain(place, per_row)
         st.tok_table = token_rows[0]
     st.where, st.token_of_place = _ops.pair_places(order, r_idx, my_slot, u_src, u_node, expert_idx, slots)
@@ -436,8 +440,10 @@ def ta2a_permute_overlap(hidden_states, probs, routing_map, *, world, rank, rpn,
                     rx_d, rmask, rgate_d, quota, epr, rpn, my_local, want_pair_pos=True)
             else:
                 r_in, s_in = _expand_arrival(rmask, slots, None)
-                exp_rx, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx_d, r_in, s_in, rgate_d,
-                                                                                         epr, rpn)
+                _none, gate_pairs, r_idx, slot_idx, _i_send, _ordo = _ops.arrival_pairs(rx_d, r_in, s_in, rgate_d,
+                                                                                        epr, rpn, move=False)
+                per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
+                exp_rx = _ops.scatter_rows(rx_d, per_row, r_idx.numel())      # each arrived row read once
             if pack_mode != "off":
                 bbuf = _pk.hopb_pack_meta(slot_idx, gate_pairs)
                 my_slot, my_gate = _pk.hopb_unpack_meta(bbuf, gate_pairs.dtype)
@@ -448,7 +454,6 @@ def ta2a_permute_overlap(hidden_states, probs, routing_map, *, world, rank, rpn,
                 red_table = _ops.index_chain(place, pair_pos).view(R, quota)
                 cols = torch.arange(quota, device=h.device, dtype=torch.int64).unsqueeze(0).expand(R, quota).contiguous()
             else:
-                per_row, _ = _ops.segment_table(r_idx, R, min(k, slots))
                 red_table = _ops.index_chain(place, per_row)
                 cols = _ops.index_chain(slot_idx, per_row)
         permuted = _FanOutEdge.apply(rx_d, red_table, permuted)
