@@ -253,7 +253,7 @@ def _dispatch_layout(T, k, world, n_experts, rpn, groups_m, capacity, gdt, onepa
                                   1 if onepass else 0),), u8)]
     if not onepass:
         planes += [("gate_pairs", (P,), gdt), ("r_idx", (P,), i64), ("slot_idx", (P,), i64), ("i_send", (rpn,), i64),
-                   ("pair_pos", (P,), i64), ("_status_r", (4,), i32), ("_order", (P,) if capacity is None else None, i64)]
+                   ("pair_pos", (P,), i64), ("_status_r", (4,), i32)]     # `order` is optional and nobody reads it here
     if len(_DISPATCH_LAYOUTS) > 64:
         _DISPATCH_LAYOUTS.clear()
     lay = _DISPATCH_LAYOUTS[key] = _planes.Layout(planes)
