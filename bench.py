@@ -17,7 +17,11 @@ keeps) over the step time; no figure in the line named `frac_hbm_peak` uses any 
 The convention that counts a payload row once on the read and once on the write side of every stage
 is reported beside it as `rows_counted_twice_GBps` only.  Also in the line: per-stage ms / GB/s /
 fraction of the 8 TB/s HBM peak and the arrival chain's us/row (`stages`), the same step with Hop B
-as one pass (`onepass`), the other four workloads (`other_configs`), the roofline record of the
+as one pass (`onepass`), every stage timed between events inside whole steps (`in_step`), the row movers alone
+with their floor at the run's own stream rates (`kernels`), those stream rates -- read-only, write-only, 8:1 sum,
+copy -- from the library's probe kernels (`ceilings`), the seam halves ta2a_permute + ta2a_unpermute on the quota
+branch, the general branch and the overlap seam with their launches named (`seam`), the other four workloads
+(`other_configs`), the roofline record of the
 slowest row-moving kernel (timed alone with HIP events on the launch stream; `traffic` from
 profiles/traffic.json when that file was measured on the sources the loaded library was built
 from), and the CPU baseline: the fastest CPU implementation measured in the run (the OpenMP C restatement of
