@@ -303,17 +303,27 @@ __global__ __launch_bounds__(kBlock) void fill_i32_kernel(int32_t *__restrict__ 
     if (i < n) p[i] = v;
 }
 
+// cursors cleared and the status block zeroed in one launch
+__global__ __launch_bounds__(kBlock) void segment_init_kernel(int32_t *__restrict__ cursor, int64_t n_seg,
+                                                              int32_t *__restrict__ status) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n_seg) cursor[i] = 0;
+    if (status && blockIdx.x == 0 && threadIdx.x < TERRACE_STATUS_WORDS) status[threadIdx.x] = 0;
+}
+
 size_t segment_table_workspace(int64_t n_seg) { return align_up((size_t)(n_seg > 0 ? n_seg : 1) * sizeof(int32_t), 256); }
 
 int run_segment_table(const int64_t *seg, int64_t n, int64_t n_seg, int width, int64_t *table, int32_t *status,
                       void *ws, size_t ws_bytes, hipStream_t s) {
     if (n < 0 || n_seg < 0 || width <= 0 || width > 64) return TERRACE_EINVAL;
-    if (status) fill_i32_kernel<<<1, kBlock, 0, s>>>(status, TERRACE_STATUS_WORDS, 0);
-    if (n_seg == 0) return check_launch();
+    if (n_seg == 0) {
+        if (status) fill_i32_kernel<<<1, kBlock, 0, s>>>(status, TERRACE_STATUS_WORDS, 0);
+        return check_launch();
+    }
     if (!table || !ws || (n > 0 && !seg)) return TERRACE_EINVAL;
     if (ws_bytes < segment_table_workspace(n_seg)) return TERRACE_ENOSPC;
     int32_t *cursor = (int32_t *)ws;
-    fill_i32_kernel<<<(unsigned)((n_seg + kBlock - 1) / kBlock), kBlock, 0, s>>>(cursor, n_seg, 0);
+    segment_init_kernel<<<(unsigned)((n_seg + kBlock - 1) / kBlock), kBlock, 0, s>>>(cursor, n_seg, status);
     if (n > 0)
         segment_claim_kernel<<<(unsigned)((n + kBlock - 1) / kBlock), kBlock, 0, s>>>(seg, n, n_seg, width, cursor, table, status);
     segment_sort_kernel<<<(unsigned)((n_seg + kBlock - 1) / kBlock), kBlock, 0, s>>>(n_seg, width, cursor, table);
