@@ -50,6 +50,31 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V
 }
 
 // ---------------------------------------------------------------------------------------------
+// resident waves per CU
+// ---------------------------------------------------------------------------------------------
+// A one-wave mover uses no LDS and few registers, so a CU would hold 32 of its waves.  The scatters (one read,
+// several writes per wave) and the combine of eight rows per output row stream faster with fewer: the memory system
+// then sees fewer interleaved streams per CU.  A launch asks for that by reserving dynamic LDS that no kernel
+// touches: a CU has 160 KB, and a reservation of 160 KB / n per one-wave workgroup keeps at most n of them resident.
+// Launch time relative to no reservation, rows of 2-14 KB, 0.25-2 GB per launch:
+//   scatter  fan 1: 24 waves 0.99-1.00, 16 waves 1.04-1.13, 12 waves 1.4  -> no cap (the gathers, likewise one
+//            read and one write per wave, lose 19 % at 16 waves)
+//            fan 2: 20 waves 0.975 on the arrival's positions (0.99 on a random permutation, where 16 give 0.975)
+//            fan 4: 16 waves 0.95 on the pack's positions, 0.975 on a random permutation; fan 8: 0.91
+//   combine  8 rows per output row, bf16 / f16 / f32, launches that read 0.5 GB or more: 12 waves 0.95-0.98,
+//            16 waves 0.99; launches the 256 MB memory-side cache holds lose up to 40 % at 12 waves, and so do 2 or
+//            4 rows per output row at any size (fewer loads in flight per wave: 12 waves 1.06-1.4) and fp8 rows,
+//            whose scale loads want the waves (12 waves 1.05), and so does a table of mostly dead entries (the
+//            two-level combine on the general branch's table: 1.75) -> capped only where it gains
+constexpr size_t kLdsPerCu = 160 * 1024;
+constexpr size_t lds_for_waves(int waves) { return (kLdsPerCu / (size_t)waves) & ~(size_t)511; }
+constexpr size_t kLdsScatterFan2 = lds_for_waves(20);
+constexpr size_t kLdsScatterFanN = lds_for_waves(16);
+constexpr size_t kLdsCombine8 = lds_for_waves(12);
+constexpr int64_t kCombineCapFromBytes = (int64_t)512 << 20;
+static_assert(kLdsScatterFan2 == 8192 && kLdsScatterFanN == 10240 && kLdsCombine8 == 13312, "LDS reservations");
+
+// ---------------------------------------------------------------------------------------------
 // stream probes: what this part sustains for the traffic mixes the row movers are made of, measured
 // with the movers' own launch shape (one-wave workgroups, one 16-byte vector per lane, streaming
 // loads and stores).  They carry no result anybody uses; the benchmark times them beside the movers.
@@ -72,8 +97,8 @@ __global__ __launch_bounds__(kBlock) void probe_write_kernel(u32x4 *__restrict__
     st_stream(y + g, u32x4{(uint32_t)g, 1u, 2u, 3u});
 }
 
-// eight contiguous streams of bf16 summed into one in fp32: the combine's 8:1 read:write mix and its
-// arithmetic with no row ids and no table
+// eight contiguous streams of bf16 summed into one in fp32: the combine's 8:1 read:write mix, its arithmetic
+// and its cap on resident waves, with no row ids and no table
 __global__ __launch_bounds__(kWave) void probe_sum8_kernel(const u32x4 *__restrict__ x, u32x4 *__restrict__ y,
                                                            int64_t n_vecs) {
     const int64_t g = (int64_t)blockIdx.x * kWave + threadIdx.x;
@@ -121,7 +146,8 @@ int launch_stream_probe(int kind, const void *x, void *y, size_t nbytes, hipStre
             break;
         case TERRACE_PROBE_SUM8:
             if (!x) return TERRACE_EINVAL;
-            probe_sum8_kernel<<<waves, kWave, 0, s>>>((const u32x4 *)x, (u32x4 *)y, vecs);
+            probe_sum8_kernel<<<waves, kWave, nbytes * 8 >= (size_t)kCombineCapFromBytes ? kLdsCombine8 : 0, s>>>(
+                (const u32x4 *)x, (u32x4 *)y, vecs);
             break;
         case TERRACE_PROBE_COPY:
             if (!x) return TERRACE_EINVAL;
@@ -797,10 +823,10 @@ int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src,
         const int64_t slices = (geom.width / 16 + kWave - 1) / kWave;
         if ((((uintptr_t)src | (uintptr_t)dst) & 15) || n_src * slices > kMaxBlocks) return TERRACE_EINVAL;
         if (fan == 2)
-            scatter_rows_sliced_fan2_kernel<I><<<(unsigned)(n_src * slices), kWave, 0, s>>>(
+            scatter_rows_sliced_fan2_kernel<I><<<(unsigned)(n_src * slices), kWave, kLdsScatterFan2, s>>>(
                 (const u32x4 *)src, (u32x4 *)dst, pos, geom.pitch / 16, geom.width / 16, (uint32_t)slices, n_dst);
         else
-            scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * slices), kWave, 0, s>>>(
+            scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * slices), kWave, fan > 2 ? kLdsScatterFanN : 0, s>>>(
                 (const u32x4 *)src, (u32x4 *)dst, pos, fan, geom.pitch / 16, geom.width / 16, (uint32_t)slices, n_dst);
         return check_launch();
     }
@@ -810,10 +836,11 @@ int launch_scatter_rows(const void *src, void *dst, const I *pos, int64_t n_src,
             const int head = (int)(((uintptr_t)dst >> 4) & (kWave - 1));
             if (rv % kWave == 0 && head == 0 && n_src * (rv / kWave) <= kMaxBlocks) {
                 if (fan == 2)
-                    scatter_rows_sliced_fan2_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, 0, s>>>(
+                    scatter_rows_sliced_fan2_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, kLdsScatterFan2, s>>>(
                         (const u32x4 *)src, (u32x4 *)dst, pos, rv, rv, (uint32_t)(rv / kWave), n_dst);
                 else
-                    scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, 0, s>>>(
+                    scatter_rows_sliced_kernel<I><<<(unsigned)(n_src * (rv / kWave)), kWave, fan > 2 ? kLdsScatterFanN : 0,
+                                                 s>>>(
                         (const u32x4 *)src, (u32x4 *)dst, pos, fan, rv, rv, (uint32_t)(rv / kWave), n_dst);
             } else {
                 const int64_t chunks = (rv + 2 * kWave - 2) / kWave;      // most kilobytes one copy can touch
@@ -927,8 +954,12 @@ static void launch_combine_so(const void *src, int64_t n_src, const int64_t *idx
     const unsigned grid = (unsigned)(n_out * slices);
     // source rows that are not whole lines (and fp8 rows, whose scales share a line): one XCD per output row
     const uint32_t run = (srb % 128 || SRC == TERRACE_FP8_E4M3_B128) && slices > 1 ? (uint32_t)slices : 0u;
-    combine_kernel<SRC, OUT><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, idx, w, w_dtype, n_out, fan, hidden,
-                                                 (uint8_t *)out, orb, slices, run, n_src);
+    // (a table with fewer source rows than three quarters of its entries is taken to be mostly dead entries -- a
+    // source row of this path belongs to one entry -- and keeps all its waves)
+    const bool cap = one_wave && SRC != TERRACE_FP8_E4M3_B128 && fan >= 8 &&
+                     n_out * fan * srb >= kCombineCapFromBytes && n_src * 4 >= n_out * fan * 3;
+    combine_kernel<SRC, OUT><<<grid, bt, cap ? kLdsCombine8 : 0, s>>>(
+        (const uint8_t *)src, srb, idx, w, w_dtype, n_out, fan, hidden, (uint8_t *)out, orb, slices, run, n_src);
 }
 
 template <int SRC>
@@ -982,6 +1013,8 @@ static int launch_combine2_so(const void *src, int64_t n_src, const int64_t *inn
     const int bt = one_wave ? kWave : kBlock;
     const int slices = (int)((chunks + bt - 1) / bt);
     const unsigned grid = (unsigned)(n_out * slices);
+    // no cap on resident waves here: 12 waves per CU measured equal on the dense tables of the quota branch and
+    // 1.75x slower on the general branch's, whose entries are mostly dead (few loads in flight per wave)
 #define TERRACE_C2(Q)                                                                                              \
     combine2_kernel<SRC, OUT, Q><<<grid, bt, 0, s>>>((const uint8_t *)src, srb, inner, n_rows, outer, fan_outer, hidden, \
                                                      (uint8_t *)out, orb, slices, n_src)
