@@ -66,6 +66,8 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const V *__restrict__ x, V
 //            4 rows per output row at any size (fewer loads in flight per wave: 12 waves 1.06-1.4) and fp8 rows,
 //            whose scale loads want the waves (12 waves 1.05), and so does a table of mostly dead entries (the
 //            two-level combine on the general branch's table: 1.75) -> capped only where it gains
+// While such a launch runs, its waves hold most of a CU's LDS: a kernel that another stream runs beside it and that
+// needs LDS gets a CU's share only as mover waves retire (each lives a few microseconds).
 constexpr size_t kLdsPerCu = 160 * 1024;
 constexpr size_t lds_for_waves(int waves) { return (kLdsPerCu / (size_t)waves) & ~(size_t)511; }
 constexpr size_t kLdsScatterFan2 = lds_for_waves(20);
