@@ -1,7 +1,7 @@
 """Benchmark of one rank's dispatch/combine path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--no-other-configs]
-                    [--no-seam] [--graph]
+                    [--no-seam] [--no-in-order] [--graph]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM: T-Route -> dispatch index build + Hop-A deduplicated pack -> Hop-B arrival chain ->
@@ -18,7 +18,8 @@ The convention that counts a payload row once on the read and once on the write 
 is reported beside it as `rows_counted_twice_GBps` only.  Also in the line: per-stage ms / GB/s /
 fraction of the 8 TB/s HBM peak and the arrival chain's us/row (`stages`), the same step with Hop B
 as one pass (`onepass`), every stage timed between events inside whole steps (`in_step`), the row movers alone
-with their floor at the run's own stream rates (`kernels`), those stream rates -- read-only, write-only, 8:1 sum,
+with their floor at the run's own stream rates and their time over tables that list the rows in order (`kernels`:
+`ms_rows_in_order`), those stream rates -- read-only, write-only, 8:1 sum,
 copy -- from the library's probe kernels (`ceilings`), the seam halves ta2a_permute + ta2a_unpermute on the quota
 branch, the general branch and the overlap seam with their launches named (`seam`), the other four workloads
 (`other_configs`), the roofline record of the
@@ -56,6 +57,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
     ap.add_argument("--no-seam", action="store_true", help="skip the ta2a_permute / ta2a_unpermute timings")
+    ap.add_argument("--no-in-order", action="store_true",
+                    help="skip the movers' launches over renumbered tables (a kernel trace then holds only launches "
+                         "over the workload's own tables)")
     ap.add_argument("--row-pitch", type=int, default=None,
                     help="bytes between payload rows in every row buffer of --config (0: rows back to back; default: "
                          "what the workload names)")
@@ -607,6 +611,25 @@ def run_workload(cfg, args, torch, detail):
         ms = event_ms(fn, reps, torch)
         kern[name] = {"ms": round(ms, 4), "bytes_per_launch": nb, "GBps": round(nb / ms / 1e6, 1),
                       "frac_hbm_peak": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    if detail and not args.no_in_order:
+        # The same launches over the same tables with their live entries renumbered in order of appearance (entry i of
+        # the table names row i; dead entries stay where they are): every read and every write becomes one
+        # contiguous stream.  Same kernels, same bytes: what remains of a mover's distance to the stream rates here
+        # is the kernel's own, the rest is what the placement of the rows costs.
+        def in_order(t):
+            live = (t >= 0).reshape(-1)
+            r = torch.cumsum(live.to(torch.int64), 0) - 1
+            return torch.where(live, r, torch.full_like(r, -1)).view_as(t).contiguous()
+        ordered = {
+            f"{k_scatter(cfg.top_groups)}(pack)": lambda t=in_order(token_rows): tops.scatter_rows(x, t, cfg.send_rows),
+            f"{k_scatter(quota)}(arrival)": lambda t=in_order(pair_pos2): tops.scatter_rows(state.payload, t, cfg.pairs),
+            f"{k_scatter(quota)}(hopb_onepass)": lambda t=in_order(place_of_pair): tops.scatter_rows(state.payload, t, n_places),
+            f"{k_gather}(regroup)": lambda t=in_order(gather_idx): tops.gather_rows(state.send_buf, t),
+            "combine_kernel": lambda t=in_order(where): tops.combine(
+                ye, t, w_sorted, out_dtype=cfg.out_dtype, fp8_hidden=fp8_hidden),
+        }
+        for name, fn in ordered.items():
+            kern[name]["ms_rows_in_order"] = round(event_ms(fn, reps, torch), 4)
     out["kernels"] = kern
     out["graph"] = graph_replay_ms(step, args, torch) if args.graph else None
     out["raw_dispatch_plus_combine_ms"] = sum(v for n, v in out["in_step"]["stage_ms"].items() if n != "route")
@@ -661,6 +684,8 @@ def main():
                 floor = predicted_floor_ms(ceilings, rd, wr)
                 v["floor_ms_at_stream_rates"] = round(floor, 4)
                 v["ms_over_floor"] = round(v["ms"] / floor, 3)
+                if "ms_rows_in_order" in v:
+                    v["rows_in_order_over_floor"] = round(v["ms_rows_in_order"] / floor, 3)
     dominant = max((k for k in kern if not k.startswith("copy") and "onepass" not in k), key=lambda k: kern[k]["ms"])
     # algorithmic bytes of the dominant kernel per launch: every row it moves, read once and written once
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": kern[dominant]["GBps"], "peak": HBM_PEAK_GBPS,
