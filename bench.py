@@ -1,7 +1,7 @@
 """Benchmark of one rank's dispatch/combine path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--no-cpu-baseline] [--no-other-configs]
-                    [--no-seam] [--no-in-order] [--graph]
+                    [--no-seam] [--no-in-order] [--tokens N] [--graph]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM: T-Route -> dispatch index build + Hop-A deduplicated pack -> Hop-B arrival chain ->
@@ -63,6 +63,9 @@ def parse():
     ap.add_argument("--row-pitch", type=int, default=None,
                     help="bytes between payload rows in every row buffer of --config (0: rows back to back; default: "
                          "what the workload names)")
+    ap.add_argument("--tokens", type=int, default=None,
+                    help="run --config with this many tokens instead of its own (e.g. a decode-sized batch; the "
+                         "measured-traffic record of profiles/ then does not apply and `traffic` is null)")
     ap.add_argument("--graph", action="store_true",
                     help="also capture the step into a HIP graph and time its replays (reported beside the eager "
                          "figure, which stays `value`)")
@@ -660,6 +663,12 @@ def main():
     if args.row_pitch is not None:
         import dataclasses
         cfg = dataclasses.replace(cfg, row_pitch=args.row_pitch or None)
+    if args.tokens is not None:
+        import dataclasses
+        if args.tokens < 1:
+            print("bench.py: --tokens must be positive", file=sys.stderr)
+            sys.exit(2)
+        cfg = dataclasses.replace(cfg, T=args.tokens, name=f"{cfg.name}_T{args.tokens}")
     torch.cuda.set_device(0)
 
     r = run_workload(cfg, args, torch, detail=True)
@@ -690,7 +699,7 @@ def main():
     # algorithmic bytes of the dominant kernel per launch: every row it moves, read once and written once
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": kern[dominant]["GBps"], "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": kern[dominant]["frac_hbm_peak"],
-                "traffic": measured_traffic(args.config, dominant, digest),
+                "traffic": None if args.tokens is not None else measured_traffic(args.config, dominant, digest),
                 "traffic_source": "profiles/traffic.json (null when measured on other sources than the loaded library's)",
                 "avg_launch_ms": kern[dominant]["ms"], "algorithmic_bytes_per_launch": kern[dominant]["bytes_per_launch"]}
 
