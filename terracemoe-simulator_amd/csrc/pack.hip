@@ -1,6 +1,7 @@
 // Send side (dispatch index build + Hop-A wire planes) when a token's node set fits one 64-bit word.
 //
-// Applies when n_nodes <= 64 and k <= 16, which covers every benchmark geometry.  Two launches:
+// Applies when n_nodes <= 64 and k <= 16, which covers every benchmark geometry.  Two launches (one, the place
+// kernel counting for itself, when all tokens are one unit):
 //
 //   k2_count_kernel   one lane per token derives the set of nodes the token touches; a wave (64 tokens, one
 //                     "unit") counts its tokens per node with ballots, the workgroup leaves each unit's prefix
@@ -41,6 +42,9 @@ static Units token_units(int64_t T, int k, int n_nodes) {
     u.wpb = 16 / lanes_per_token(k);
     u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
     u.direct = n_nodes <= kDirectMaxBuckets && (int64_t)n_nodes * u.n_blocks <= kDirectMaxWords;
+    // up to 64 tokens are one place workgroup, which then counts for itself: no count launch (about 4.5 us of a
+    // decode-sized step)
+    u.solo = u.direct && u.n_units == 1 && n_nodes <= kWave;
     return u;
 }
 
@@ -173,6 +177,7 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     __shared__ int32_t s_tot[64], s_base[64], s_start[65], s_tab[64];
     __shared__ int32_t s_wcnt[kWaves][64];
     __shared__ int32_t s_dirty[kWaves];
+    __shared__ int32_t s_census[kWaves][3];          // solo: each wave's fault bits, occupied pairs, pairs off the quota
     const int lane = lane_id(), w = wave_in_block();
     const int unit = blockIdx.x;
     const int n_nodes = u.n_buckets;
@@ -189,13 +194,13 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     G gate = G(0);
     if (has_col && gates) gate = gates[t * k + col];
     int tab = 0;
-    if (threadIdx.x < n_nodes) tab = table[(int64_t)threadIdx.x * u.n_units + unit];
+    if (!u.solo && threadIdx.x < n_nodes) tab = table[(int64_t)threadIdx.x * u.n_units + unit];
     // ---- cursors of this unit: start[n] + earlier workgroups (+ s_tab: earlier units of the count workgroup) ----
     const int me = unit / u.wpb;
     TableOut out;
     out.hist_i64 = node_counts;
     out.offsets_i64 = node_offsets;
-    direct_block_base(u, table, me, unit == 0, (lds_i32 *)s_tot, (lds_i32 *)s_base, (lds_i32 *)s_start, out);
+    if (!u.solo) direct_block_base(u, table, me, unit == 0, (lds_i32 *)s_tot, (lds_i32 *)s_base, (lds_i32 *)s_start, out);
     // ---- the token's ids, shared inside the group; ranks by (id, column) ----
     TokenView<LPT> tv;
     tv.build(v, has_col, col, tok_lane, slots, n_experts, M, quota);
@@ -235,17 +240,59 @@ __global__ __launch_bounds__(kWave *LPT) void k2_place_kernel(
     // ---- does any token of the workgroup start from defaults?  (uniform across the workgroup after the barrier) ----
     const uint64_t any_dirty = __ballot(live && !clean);
     if (lane == 0) s_dirty[w] = any_dirty != 0;
+    if (u.solo) {           // the census the count kernel takes otherwise (same definitions), one entry per wave
+        int fault = (has_col && !ok) ? TERRACE_FAULT_ID_RANGE : 0;
+        if (live && col == 0 && __popcll(tv.all) != M) fault |= TERRACE_FAULT_FANOUT;
+        if (tv.bad_pair) fault |= TERRACE_FAULT_QUOTA;
+        const int occupied = __popcll(__ballot(tv.first_of_node)), off_quota = __popcll(__ballot(tv.bad_pair));
+#pragma unroll
+        for (int d = 1; d < kWave; d <<= 1) fault |= __shfl_xor(fault, d, kWave);
+        if (lane == 0) {
+            s_census[w][0] = fault;
+            s_census[w][1] = occupied;
+            s_census[w][2] = off_quota;
+        }
+    }
     __syncthreads();
+    if (u.solo) {
+        // this workgroup holds every token: the per-node totals are its waves' counts, the cursors start at the
+        // nodes' offsets, and wave 0 (lane n = node n) publishes what the count + base steps publish otherwise
+        if (w == 0) {
+            int tot = 0;
+            if (lane < n_nodes)
+                for (int x = 0; x < kWaves; ++x) tot += s_wcnt[x][lane];
+            const int incl = wave_inclusive_scan(tot);
+            if (lane < n_nodes) {
+                s_start[lane] = incl - tot;
+                s_base[lane] = incl - tot;
+                table[units_start_at(u) + lane] = incl - tot;
+                out.put(lane, tot, incl - tot);
+            }
+            if (lane == n_nodes - 1) {
+                s_start[n_nodes] = incl;
+                table[units_start_at(u) + n_nodes] = incl;
+            }
+        }
+        __syncthreads();
+    }
     bool dirty_block = false;
     for (int x = 0; x < kWaves; ++x) dirty_block = dirty_block || s_dirty[x];
     // ---- the status block: the count kernel's per-workgroup census, added up and stored by the first workgroup ----
     if (unit == 0 && w == 0 && status) {
         const int32_t *census = table + units_census_at(u);
         int f = 0, o = 0, q = 0;
-        for (int b = lane; b < u.n_blocks; b += kWave) {
-            f |= census[4 * b + 0];
-            o += census[4 * b + 1];
-            q += census[4 * b + 2];
+        if (u.solo) {
+            if (lane < kWaves) {
+                f = s_census[lane][0];
+                o = s_census[lane][1];
+                q = s_census[lane][2];
+            }
+        } else {
+            for (int b = lane; b < u.n_blocks; b += kWave) {
+                f |= census[4 * b + 0];
+                o += census[4 * b + 1];
+                q += census[4 * b + 2];
+            }
         }
 #pragma unroll
         for (int d = 1; d < kWave; d <<= 1) {
@@ -337,9 +384,11 @@ int run_k2_token(const void *hidden, const int64_t *expert_idx, const void *gate
 #define TERRACE_COUNT(L)                                                                                          \
     k2_count_kernel<L><<<u.n_blocks, kSortBlockMax, 0, s>>>(expert_idx, T, k, slots, n_experts, groups_m, k / groups_m, \
                                                            u, table)
-    if (k <= 4) TERRACE_COUNT(4);
-    else if (k <= 8) TERRACE_COUNT(8);
-    else TERRACE_COUNT(16);
+    if (!u.solo) {
+        if (k <= 4) TERRACE_COUNT(4);
+        else if (k <= 8) TERRACE_COUNT(8);
+        else TERRACE_COUNT(16);
+    }
 #undef TERRACE_COUNT
 #define TERRACE_PLACE(L, G)                                                                                        \
     launch_place<L, G>(expert_idx, gates, T, k, slots, n_experts, groups_m, u, table, mask, gate_rows, u_src, u_node, \

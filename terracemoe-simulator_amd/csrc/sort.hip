@@ -14,20 +14,25 @@
 //          items with wave ballots, and emits the outputs.
 //   (scan  tables too large for every rank workgroup to re-read: one workgroup turns the plain [unit][bucket]
 //          counts into exclusive cursors between the two.)
+// Up to 1024 items the rank launch is one workgroup that counts for itself, and no count launch runs.
 // The row payload itself is moved afterwards by the scatter/gather kernels of rows.hip.
 #include "sort.hpp"
 
 namespace terrace {
 
 void finish_units(Units &u) {
-    // direct: 16-wave workgroups keep the number of workgroup totals a rank workgroup re-reads small
-    u.wpb = u.n_units >= 64 ? 16 : 4;
+    // direct: 16-wave workgroups keep the number of workgroup totals a rank workgroup re-reads small; up to 16
+    // units are one such workgroup, which then needs no count launch (solo).  Per sort at 512 items: 5.6 us against
+    // 4.6 + 6.4 as count + rank; larger inputs in one workgroup (2048 items as four chunks per wave: 8.9 us
+    // against 4.0 + 6.4) gain too little to be worth one CU writing every output plane.
+    u.wpb = (u.n_units >= 64 || u.n_units <= 16) ? 16 : 4;
     u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
     u.direct = u.n_buckets <= kDirectMaxBuckets && (int64_t)u.n_buckets * u.n_blocks <= kDirectMaxWords;
     if (!u.direct) {
         u.wpb = 4;
         u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
     }
+    u.solo = u.direct && u.n_blocks == 1 && u.n_items <= kSoloMaxItems;
 }
 
 Units make_units(int64_t n_items, int n_buckets) {
@@ -516,7 +521,69 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
         pre[c] = emit.fetch(safe);
     }
     const int32_t *start = table + units_start_at(u);
-    if (u.direct) {
+    int keys[CH];
+    if (u.solo) {
+        // The whole input is this one workgroup's, and no count launch ran: each wave counts its own unit into its
+        // row of LDS, the rows become prefixes over the waves, the totals are scanned, and the status block -- which
+        // the count launch clears otherwise -- is cleared here, fenced, ahead of the barriers every later atomic
+        // sits behind.
+        lds_i32 *rows = (lds_i32 *)lds;
+        lds_i32 *tot = rows + u.wpb * u.n_buckets, *lstart = tot + 2 * u.n_buckets;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int64_t item = first + (int64_t)c * kWave + lane;
+            bool bad = false;
+            const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
+            keys[c] = item < u.n_items ? key : -1;
+            if (bad && item < u.n_items) fault |= TERRACE_FAULT_ID_RANGE;
+        }
+        for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = 0;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int key = keys[c];
+            const bool valid = key >= 0;
+            const uint64_t peers = same_key_lanes(key, valid, key_bits);
+            if (valid && lane == __builtin_ctzll(peers)) cursor[key] = cursor[key] + __popcll(peers);
+            __builtin_amdgcn_wave_barrier();
+        }
+        if (status && threadIdx.x < TERRACE_STATUS_WORDS) {
+            status[threadIdx.x] = 0;
+            __threadfence();
+        }
+        __syncthreads();
+        for (int b = threadIdx.x; b < u.n_buckets; b += blockDim.x) {
+            int run = 0;
+            for (int x = 0; x < u.wpb; ++x) {
+                const int v = rows[x * u.n_buckets + b];
+                rows[x * u.n_buckets + b] = run;
+                run += v;
+            }
+            tot[b] = run;
+        }
+        __syncthreads();
+        if (w == 0) {
+            int carry = 0;
+            for (int b0 = 0; b0 < u.n_buckets; b0 += kWave) {
+                const int b = b0 + lane;
+                const int v = b < u.n_buckets ? tot[b] : 0;
+                const int incl = wave_inclusive_scan(v);
+                if (b < u.n_buckets) lstart[b] = carry + incl - v;
+                carry += __shfl(incl, kWave - 1, kWave);
+            }
+            if (lane == 0) lstart[u.n_buckets] = carry;
+        }
+        __syncthreads();
+        int32_t *start_out = table + units_start_at(u);
+        for (int b = threadIdx.x; b <= u.n_buckets; b += blockDim.x) {
+            const int32_t s0 = lstart[b];
+            start_out[b] = s0;
+            if (b < u.n_buckets) out.put(b, tot[b], s0);
+        }
+        if (!active) return;
+        for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = cursor[b] + lstart[b];
+        start = (const int32_t *)lstart;
+    } else if (u.direct) {
         // this unit's prefixes inside its workgroup: loaded now, with the keys, so that the only memory round trip
         // of the kernel is the one the workgroup totals below share with them
         constexpr int kTabRegs = kDirectMaxBuckets / kWave;
@@ -539,14 +606,15 @@ __global__ __launch_bounds__(kSortBlockMax) void rank_kernel(KeyFn key_of, EmitF
     } else {
         for (int b = lane; b < u.n_buckets; b += kWave) cursor[b] = table[(int64_t)b * u.n_units + unit];
     }
-    int keys[CH];
+    if (!u.solo) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int64_t item = first + (int64_t)c * kWave + lane;
-        bool bad = false;
-        const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
-        keys[c] = item < u.n_items ? key : -1;
-        if (bad && item < u.n_items) fault |= TERRACE_FAULT_ID_RANGE;
+        for (int c = 0; c < CH; ++c) {
+            const int64_t item = first + (int64_t)c * kWave + lane;
+            bool bad = false;
+            const int key = key_of.bucket(item < u.n_items ? item : u.n_items - 1, fetched[c], &bad);
+            keys[c] = item < u.n_items ? key : -1;
+            if (bad && item < u.n_items) fault |= TERRACE_FAULT_ID_RANGE;
+        }
     }
     __builtin_amdgcn_wave_barrier();
     int tally[2] = {0, 0};
@@ -1065,14 +1133,17 @@ static int run_sort(const KeyFn &key, const EmitFn &emit, Units u, int32_t *tabl
                     int32_t *status, bool do_rank, hipStream_t s) {
     if (!do_rank && u.direct) {          // the histogram alone: the scan launch writes it, so take that path
         u.direct = 0;                    // (the table region of a direct layout is large enough for it)
+        u.solo = 0;
         u.wpb = 4;
         u.n_blocks = (u.n_units + u.wpb - 1) / u.wpb;
     }
     const int blocks = u.n_blocks, threads = u.wpb * kWave;
     const size_t lc = lds_count(u), lr = lds_rank(u);
-    if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, threads, lc, s>>>(key, u, table, status);
-    else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, threads, lc, s>>>(key, u, table, status);
-    else count_kernel<KeyFn, 16><<<blocks, threads, lc, s>>>(key, u, table, status);
+    if (!u.solo) {
+        if (u.chunks == 1) count_kernel<KeyFn, 1><<<blocks, threads, lc, s>>>(key, u, table, status);
+        else if (u.chunks == 4) count_kernel<KeyFn, 4><<<blocks, threads, lc, s>>>(key, u, table, status);
+        else count_kernel<KeyFn, 16><<<blocks, threads, lc, s>>>(key, u, table, status);
+    }
     if (!u.direct) launch_scan(u, table, out, status, s);
     if (do_rank) {
         if (u.chunks == 1) rank_kernel<KeyFn, EmitFn, 1><<<blocks, threads, lr, s>>>(key, emit, u, table, out, status);

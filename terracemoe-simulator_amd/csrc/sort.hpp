@@ -18,6 +18,8 @@ constexpr int kScanThreads = 1024;
 //           words from L2 -- and no launch stands between count and rank;
 //   scan    the count kernel leaves plain per-unit counts and a one-workgroup scan launch turns the whole table
 //           into cursors (tables too large for every workgroup to re-read).
+// And for inputs one workgroup can hold (kSoloMaxItems): no count launch at all -- the rank workgroup counts its
+// waves' units in LDS first (`solo`).
 struct Units {
     int64_t n_items;
     int chunks;       // 64-item chunks per unit: 1, 4 or 16, growing with the item count
@@ -26,9 +28,11 @@ struct Units {
     int wpb;          // waves per workgroup of the count / rank kernels (4 or 16)
     int n_blocks;     // their grid
     int direct;       // 1: no scan launch (see above)
+    int solo = 0;     // 1: one workgroup holds every item and the rank launch counts for itself (no count launch)
 };
 
 constexpr int kDirectMaxBuckets = 256;
+constexpr int64_t kSoloMaxItems = 1024;  // 16 waves x 64 items
 constexpr int kDirectMaxWords = 16384;   // n_buckets * n_blocks a rank workgroup may re-read
 
 Units make_units(int64_t n_items, int n_buckets);

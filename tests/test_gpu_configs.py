@@ -123,6 +123,21 @@ def test_large_random_geometries_every_plane_matches_oracle(index):
     _check_every_plane(cfg)
 
 
+# Up to 64 tokens the send side is one place workgroup that counts for itself, and up to 1024 items a sort is one
+# rank workgroup that does; one more token or item and the count launch is back.  Token counts on both sides of each
+# limit, at k = 8 (pairs = 8 T: 1024 at T = 128) and at k = 2, M = 1 (pairs = 2 T: 1024 at T = 512), with and
+# without a capacity.
+@pytest.mark.parametrize("capacity_factor", [None, 0.5])
+@pytest.mark.parametrize("T,k,M", [(63, 8, 4), (64, 8, 4), (65, 8, 4), (127, 8, 4), (128, 8, 4), (129, 8, 4),
+                                   (511, 2, 1), (512, 2, 1), (513, 2, 1), (1, 8, 4)])
+def test_one_workgroup_limits_every_plane_matches_oracle(T, k, M, capacity_factor):
+    from terrace import configs
+    cfg = configs.PathConfig(f"limits_T{T}_k{k}", T, 64, 8, k, M, 4, 64, "bf16", bias="normal", softmax_gates=True,
+                             capacity_factor=capacity_factor, seed=4000 + T)
+    announce("one-workgroup limits", cfg)
+    _check_every_plane(cfg)
+
+
 def _check_every_plane(cfg):
     from terrace.ta2a_fwd import loopback_combine, loopback_dispatch, twolevel_combine
     from terrace import configs

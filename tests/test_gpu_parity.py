@@ -463,28 +463,30 @@ def test_malformed_routing_is_contained_and_counted():
     import terrace.ops as tops
     from terrace import _hip
     announce("k2 malformed")
-    cases = {
-        "three_one": ([[0, 2, 3, 5]] * 6, 12, 12),          # 2 nodes each, both off the 2/2 quota
-        "fanout_one": ([[0, 1, 2, 3]] * 6, 6, 6),           # one node holding 4
-        "id_range": ([[0, 2, 4, 99]] * 6, 12, 6),           # one id outside [0, 8)
-    }
-    for name, (rows, occupied, off_quota) in cases.items():
-        e = torch.tensor(rows, device=DEV)
-        x = torch.randn(6, 16, device=DEV)
-        gts = torch.rand(6, 4, device=DEV)
-        (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e, gts, 4, 8, 2, 2, extras=True,
-                                                                         combine_table=True)
-        assert ((ex["pair_src"] >= -1) & (ex["pair_src"] < 24)).all()
-        assert (ex["where"] == -1).all(), "the pre-set combine table of a malformed token must read -1"
-        fault, occ, offq, _ = ex["status"].tolist()
-        assert fault != 0 and occ == occupied and offq == off_quota, (name, fault, occ, offq)
-        assert int(counts.sum()) <= 12 and (counts >= 0).all()
-        assert ((u_src >= 0) & (u_src < 6)).all() and ((mask >= 0) & (mask < 4)).all()
-        assert ((ex["pair_table"] >= -1) & (ex["pair_table"] < 24)).all()
-        assert ((ex["token_rows"] >= -1) & (ex["token_rows"] < 12)).all()
-        assert torch.isfinite(gate_rows).all()
-        if name == "id_range":
-            assert fault & _hip.FAULT_ID_RANGE
+    # 6 tokens are one place workgroup that takes the census itself; 70 go through the count launch
+    for n in (6, 70):
+        cases = {
+            "three_one": ([[0, 2, 3, 5]] * n, 2 * n, 2 * n),        # 2 nodes each, both off the 2/2 quota
+            "fanout_one": ([[0, 1, 2, 3]] * n, n, n),               # one node holding 4
+            "id_range": ([[0, 2, 4, 99]] * n, 2 * n, n),            # one id outside [0, 8)
+        }
+        for name, (rows, occupied, off_quota) in cases.items():
+            e = torch.tensor(rows, device=DEV)
+            x = torch.randn(n, 16, device=DEV)
+            gts = torch.rand(n, 4, device=DEV)
+            (payload, mask, gate_rows, u_src, counts), ex = tops.k2_pack_raw(x, e, gts, 4, 8, 2, 2, extras=True,
+                                                                             combine_table=True)
+            assert ((ex["pair_src"] >= -1) & (ex["pair_src"] < 4 * n)).all()
+            assert (ex["where"] == -1).all(), "the pre-set combine table of a malformed token must read -1"
+            fault, occ, offq, _ = ex["status"].tolist()
+            assert fault != 0 and occ == occupied and offq == off_quota, (name, n, fault, occ, offq)
+            assert int(counts.sum()) <= 2 * n and (counts >= 0).all()
+            assert ((u_src >= 0) & (u_src < n)).all() and ((mask >= 0) & (mask < 4)).all()
+            assert ((ex["pair_table"] >= -1) & (ex["pair_table"] < 4 * n)).all()
+            assert ((ex["token_rows"] >= -1) & (ex["token_rows"] < 2 * n)).all()
+            assert torch.isfinite(gate_rows).all()
+            if name == "id_range":
+                assert fault & _hip.FAULT_ID_RANGE
     # the (token, run)-item kernels (k > 16, or more than 64 nodes) contain the same breakage: every address they
     # form comes from an item's sorted position or from a rank below k, never from an id
     g = torch.Generator().manual_seed(9)
