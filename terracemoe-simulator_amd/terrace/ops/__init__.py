@@ -792,16 +792,18 @@ def plan_general(expert_idx, world, n_experts, rpn):
     u_src = torch.empty((cap,), dtype=torch.int64, device=dev)
     u_node = torch.empty((cap,), dtype=torch.int64, device=dev)
     inverse = torch.empty((T * k,), dtype=torch.int64, device=dev)
-    counts = torch.empty((n_nodes,), dtype=torch.int64, device=dev)
-    st = _hip.new_status(dev)
+    # the counts and the status block share one allocation, so that one copy to the host brings both
+    words = _hip.STATUS_WORDS // 2
+    both = torch.empty((n_nodes + words,), dtype=torch.int64, device=dev)
+    counts, st = both[:n_nodes], both[n_nodes:].view(torch.int32)
     ws = _hip.workspace(_hip.query("terrace_plan_general_workspace", T, k, n_nodes), dev)
     _hip.call("terrace_plan_general", _hip.ptr(expert_idx), T, k, world, n_experts, rpn, _hip.ptr(u_src),
               _hip.ptr(u_node), _hip.ptr(counts), _hip.ptr(inverse), _hip.ptr(st), _hip.ptr(ws), ws.numel(),
               _hip.stream(dev))
-    both = torch.cat([counts.sum().reshape(1), st[:1].to(torch.int64)]).tolist()
-    if both[1] & _hip.FAULT_ID_RANGE:
+    host = both.tolist()
+    if (host[n_nodes] & 0xFFFFFFFF) & _hip.FAULT_ID_RANGE:           # status word 0: the low half of the first word
         raise ValueError("plan_ta2a: expert id out of range")
-    n_rows = int(both[0])
+    n_rows = sum(host[:n_nodes])
     return u_src[:n_rows], u_node[:n_rows], counts, inverse
 
 
