@@ -457,16 +457,20 @@ def test_two_host_threads_on_two_streams_do_not_disturb_each_other():
             assert torch.equal(w, g_)
 
 
-@pytest.mark.parametrize("name", ["c2", "c4", "c5"])
-def test_the_whole_step_replays_as_one_hip_graph(name):
+@pytest.mark.parametrize("name,tokens,onepass", [("c2", 2048, False), ("c4", 2048, False), ("c5", 2048, False),
+                                                 ("c2", 48, False), ("c2", 48, True), ("c4", 100, True)])
+def test_the_whole_step_replays_as_one_hip_graph(name, tokens, onepass):
     """Route, dispatch and combine launch kernels only (no allocation of their own, no memset, no host
     synchronisation), so a step records into a HIP graph; every replay, with eager work and synchronisations
-    in between, must reproduce the eager result bit for bit."""
+    in between, must reproduce the eager result bit for bit.  The decode-sized cases run the index kernels that
+    count for themselves (one workgroup, no count launch, the status block cleared inside the kernel)."""
     import terrace
     from terrace import configs
-    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch
-    cfg = configs.CONFIGS[name].scaled(2048)
-    announce("graph replay", cfg.name)
+    from terrace.ta2a_fwd import loopback_combine, loopback_dispatch_onepass
+    from terrace.ta2a_fwd import loopback_dispatch as two_step
+    loopback_dispatch = loopback_dispatch_onepass if onepass else two_step
+    cfg = configs.CONFIGS[name].scaled(tokens)
+    announce("graph replay", cfg.name, tokens, onepass)
     inp = configs.make_inputs(cfg)
     logits, bias, x = inp["logits"].to(DEV), inp["bias"].to(DEV), configs.rows_to(inp["x"], DEV)
     ga = None if inp["gate_affinity"] is None else inp["gate_affinity"].to(DEV)
