@@ -180,12 +180,10 @@ def minimum_traffic_bytes(cfg: PathConfig, kept_pairs: int | None = None, places
     written once (a scatter reads a source row once however many copies it writes), plus the same
     index and gate planes as ``algorithmic_bytes``.  ``kept_pairs`` / ``places`` describe a capacity
     layout (rows that survive the cut, rows of the padded buffer); default: drop-less."""
-    T, k, q = cfg.T, cfg.top_k, cfg.quota
-    S, P, row = cfg.send_rows, cfg.pairs, cfg.row_bytes
+    T, S, P, row = cfg.T, cfg.send_rows, cfg.pairs, cfg.row_bytes
     kept = P if kept_pairs is None else kept_pairs
     places = P if places is None else places
     alg = algorithmic_bytes(cfg)
-    orow = cfg.hidden * (4 if cfg.fmt == "f32" else 2)
     return {
         "route": alg["route"],
         "pack": alg["pack"] - 2 * S * row + (T + S) * row,
